@@ -1,0 +1,224 @@
+/* rocshmem_mi355x.h -- C ABI of librocshmem_mi355x.so.
+ *
+ * The reference (ROCm/ROC_SHMEM) exposes a C++ host/device interface that is
+ * linked into the user's kernels; it has no foreign-function boundary of its
+ * own.  This header is that boundary for the MI355X-native data path: plain C
+ * entry points that (a) mirror the reference's host lifecycle calls and
+ * (b) launch, for every PE of the job at once, a grid of workgroups in which
+ * each workgroup issues the named roc_shmem_* device call on its share of the
+ * data -- the role the reference's functional test kernels play
+ * (clients/functional_tests/ in the reference).  All PEs live in one process
+ * and one GPU; a symmetric address passed in is the address in PE 0's slice
+ * unless stated otherwise.
+ *
+ * Return value: 0 on success, negative on error (rsm_last_error() has the
+ * message).  No entry point takes or returns C++ or torch types.
+ */
+#ifndef ROCSHMEM_MI355X_C_ABI_H
+#define ROCSHMEM_MI355X_C_ABI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- codes -------------------------------------------------------------- */
+
+/* Element types of the reductions (reference: library/include/roc_shmem.hpp:1190-1198;
+ * RSM_BF16 is an extension). */
+enum rsm_dtype {
+  RSM_SHORT = 0,
+  RSM_INT = 1,
+  RSM_LONG = 2,
+  RSM_LONGLONG = 3,
+  RSM_FLOAT = 4,
+  RSM_DOUBLE = 5,
+  RSM_BF16 = 6
+};
+
+/* Reduction operators, numerically equal to ROC_SHMEM_OP (roc_shmem.hpp:52-61). */
+enum rsm_op {
+  RSM_SUM = 0,
+  RSM_MAX = 1,
+  RSM_MIN = 2,
+  RSM_PROD = 3,
+  RSM_AND = 4,
+  RSM_OR = 5,
+  RSM_XOR = 6
+};
+
+enum rsm_rma_kind { RSM_PUT = 0, RSM_GET = 1, RSM_PUT_NBI = 2, RSM_GET_NBI = 3 };
+enum rsm_granularity { RSM_THREAD = 0, RSM_WAVE = 1, RSM_WG = 2 };
+
+/* Kinds of the small-operation stream executed by rsm_small_ops(). */
+enum rsm_small_kind {
+  RSM_OP_P64 = 0,        /* roc_shmem_ctx_long_p            (8-byte inline put)        */
+  RSM_OP_FADD64 = 1,     /* roc_shmem_ctx_int64_atomic_fetch_add                       */
+  RSM_OP_ADD64 = 2,      /* roc_shmem_ctx_int64_atomic_add                             */
+  RSM_OP_FINC64 = 3,     /* roc_shmem_ctx_int64_atomic_fetch_inc                       */
+  RSM_OP_INC64 = 4,      /* roc_shmem_ctx_int64_atomic_inc                             */
+  RSM_OP_CSWAP64 = 5,    /* roc_shmem_ctx_int64_atomic_compare_swap (cond in `aux`)    */
+  RSM_OP_FETCH64 = 6,    /* roc_shmem_ctx_int64_atomic_fetch                           */
+  RSM_OP_SET64 = 7,      /* roc_shmem_ctx_int64_atomic_set                             */
+  RSM_OP_SWAP64 = 8,     /* roc_shmem_ctx_int64_atomic_swap                            */
+  RSM_OP_P32 = 9,        /* roc_shmem_ctx_int_p             (4-byte inline put)        */
+  RSM_OP_FADD32 = 10,    /* roc_shmem_ctx_int_atomic_fetch_add                         */
+  RSM_OP_PUTMEM = 11,    /* roc_shmem_ctx_putmem_nbi of `aux` bytes from `value` (a symmetric offset) */
+  RSM_OP_GETMEM = 12,    /* roc_shmem_ctx_getmem_nbi of `aux` bytes into `value` (a symmetric offset) */
+  RSM_OP_FAND64 = 13,    /* roc_shmem_ctx_uint64_atomic_fetch_and                      */
+  RSM_OP_FOR64 = 14,     /* roc_shmem_ctx_uint64_atomic_fetch_or                       */
+  RSM_OP_FXOR64 = 15,    /* roc_shmem_ctx_uint64_atomic_fetch_xor                      */
+  RSM_OP_NONE = 255      /* lane sits this round out (stays inactive)                  */
+};
+
+/* One small operation: issued by the thread that owns it, towards PE `pe`,
+ * on the symmetric object at byte offset `offset` of the heap. */
+typedef struct rsm_small_op {
+  uint32_t kind;
+  uint32_t pe;
+  uint64_t offset;
+  int64_t value;
+  int64_t aux;
+} rsm_small_op_t;
+
+/* Launch shape shared by the data-path entry points. */
+typedef struct rsm_launch {
+  int wgs_per_pe;   /* workgroups acting for each PE (>= 1)                        */
+  int wg_size;      /* threads per workgroup, multiple of 64, <= 1024              */
+  size_t tile;      /* elements (or bytes) per device call; 0 = split evenly       */
+  void *stream;     /* hipStream_t, NULL = the default stream                      */
+} rsm_launch_t;
+
+/* ---- lifecycle (reference: roc_shmem_init/finalize/malloc/free/n_pes,
+ *      library/src/roc_shmem.cpp:71-135) ------------------------------------- */
+
+/* Arguments equal to 0 fall back to ROC_SHMEM_NUM_PES / ROC_SHMEM_HEAP_SIZE /
+ * ROC_SHMEM_NUM_BLOCKS / ROC_SHMEM_SQ_SIZE and then to the defaults
+ * (8 PEs, 1 GiB per PE, 64 contexts per PE, 1024-entry send queues). */
+int rsm_init(int num_pes, size_t heap_bytes_per_pe, int num_blocks, unsigned sq_size);
+int rsm_finalize(void);
+int rsm_is_initialized(void);
+const char *rsm_last_error(void);
+int rsm_n_pes(void);
+int rsm_num_blocks(void);
+size_t rsm_heap_size(void);
+size_t rsm_slice_stride(void);
+void *rsm_malloc(size_t bytes);                 /* NULL on failure or bytes == 0 */
+int rsm_free(void *ptr);
+size_t rsm_heap_bytes_in_use(void);
+void *rsm_ptr(const void *sym, int pe);         /* roc_shmem_ptr: address of `sym` in PE `pe`'s slice */
+void *rsm_heap_base(int pe);                    /* first byte of PE `pe`'s slice (reference: base_heap[pe]) */
+int rsm_take_status(void);                      /* sticky device status word, cleared by the call */
+
+/* ---- teams (reference: roc_shmem.cpp:188-313, team.cpp:47-107) ------------ */
+
+uint64_t rsm_team_world(void);
+int rsm_team_split_strided(uint64_t parent, int start, int stride, int size, uint64_t *new_team);
+int rsm_team_destroy(uint64_t team);
+int rsm_team_n_pes(uint64_t team);
+int rsm_team_translate_pe(uint64_t src_team, int src_pe, uint64_t dst_team);
+
+/* ---- plumbing: host<->device copies, streams, events ---------------------- */
+
+int rsm_copy_to_device(void *dst, const void *host_src, size_t bytes);
+int rsm_copy_to_host(void *host_dst, const void *src, size_t bytes);
+int rsm_fill(void *dst, int byte_value, size_t bytes);
+int rsm_synchronize(void);
+void *rsm_device_alloc(size_t bytes);           /* ordinary (non-symmetric) device memory */
+int rsm_device_free(void *ptr);
+void *rsm_stream_create(void);
+int rsm_stream_destroy(void *stream);
+void *rsm_event_create(void);
+int rsm_event_destroy(void *event);
+int rsm_event_record(void *event, void *stream);
+int rsm_event_elapsed_ms(void *start, void *stop, float *ms);   /* synchronises on `stop` */
+
+/* ---- reductions ------------------------------------------------------------
+ * roc_shmem_ctx_<T>_<op>_wg_to_all, active-set form (roc_shmem.hpp:837-851;
+ * GPUIBContext::to_all, gpu_ib/context_ib_tmpl_device.hpp:262-307).  Workgroup w
+ * of every member PE reduces tiles w, w+wgs_per_pe, ... of `launch->tile`
+ * elements with its own pSync slice pSync + w*256.  `pSync` therefore holds
+ * wgs_per_pe*256 longs, all ROC_SHMEM_SYNC_VALUE on entry and on return;
+ * `pWrk` may be NULL (it is not used). */
+int rsm_to_all(int dtype, int op, void *dest, const void *source, size_t nreduce, int pe_start,
+               int log_pe_stride, int pe_size, void *pWrk, long *pSync,
+               const rsm_launch_t *launch);
+/* Team form (roc_shmem.hpp:848-851; context_ib_tmpl_device.hpp:238-260). */
+int rsm_to_all_team(int dtype, int op, uint64_t team, void *dest, const void *source,
+                    size_t nreduce, const rsm_launch_t *launch);
+
+/* ---- workgroup / wavefront / thread RMA -------------------------------------
+ * roc_shmemx_ctx_{put,get}mem[_nbi]_{wg,wave} and roc_shmem_ctx_{put,get}mem[_nbi]
+ * (roc_shmem.hpp:907-977,2029-2566; context_ib_device.cpp:84-321).  PE p
+ * moves messages m = 0..n_msgs-1 of `msg_bytes` each between its own
+ * `source + m*src_stride` / `dest + m*dst_stride` and PE (p+pe_shift)%n_pes,
+ * the messages being dealt round-robin to its workgroups, waves or threads
+ * according to `granularity`. */
+int rsm_rma(int kind, int granularity, void *dest, const void *source, size_t msg_bytes,
+            size_t n_msgs, size_t dst_stride, size_t src_stride, int pe_shift,
+            const rsm_launch_t *launch);
+
+/* ---- broadcast / alltoall / fcollect / barrier -------------------------------
+ * roc_shmem_ctx_<T>_wg_broadcast (roc_shmem.hpp:873-887; context_ib_tmpl_device.hpp:
+ * 455-519): `pe_root` is the root's ordinal in the active set; the root's
+ * dest is not written.  Tiled like rsm_to_all (pSync: wgs_per_pe*256 longs). */
+int rsm_broadcast(size_t elem_size, void *dest, const void *source, size_t nelem, int pe_root,
+                  int pe_start, int log_pe_stride, int pe_size, long *pSync,
+                  const rsm_launch_t *launch);
+int rsm_broadcast_team(size_t elem_size, uint64_t team, void *dest, const void *source,
+                       size_t nelem, int pe_root, const rsm_launch_t *launch);
+/* roc_shmem_ctx_<T>_wg_alltoall (roc_shmem.hpp:892-895; context_ib_tmpl_device.hpp:
+ * 521-558) and _wg_fcollect (:899-902; :845-876).  With wgs_per_pe > 1 the
+ * workgroups of a PE call the sharded extension, one shard each. */
+int rsm_alltoall(size_t elem_size, uint64_t team, void *dest, const void *source, size_t nelem,
+                 const rsm_launch_t *launch);
+int rsm_fcollect(size_t elem_size, uint64_t team, void *dest, const void *source, size_t nelem,
+                 const rsm_launch_t *launch);
+/* roc_shmem_ctx_wg_barrier_all repeated `iterations` times by every workgroup
+ * (context_ib_device_coll.cpp:105-120). */
+int rsm_barrier_all(int iterations, const rsm_launch_t *launch);
+
+/* ---- small puts and AMOs ------------------------------------------------------
+ * Thread t of the grid issues ops[t], ops[t+T], ... (T = total threads) through
+ * the thread-level API (roc_shmem.hpp:907-1147; context_ib_device.cpp:84-184,
+ * context_ib_tmpl_device.hpp:365-453), every op also leaving its 64-byte WQE
+ * in the issuing workgroup's send queue (queue_pair.cpp:205-273).  `ops` is
+ * device memory.  `fetched` (device, n_ops int64, may be NULL) receives the
+ * value returned by fetching operations. */
+int rsm_small_ops(const rsm_small_op_t *ops, size_t n_ops, int64_t *fetched,
+                  const rsm_launch_t *launch);
+
+/* ---- send-queue inspection (reference: debug_print_sq, include/debug.hpp,
+ *      gpu_ib/qe_dumper.cpp:51-76) ---------------------------------------------- */
+
+int rsm_sq_reset(void);                                        /* zero all rings and indices */
+int rsm_sq_read(int pe, int block, unsigned index, uint64_t out_words[8]);
+int rsm_sq_image(int pe, int block, void *host_out, size_t bytes);
+int rsm_sq_state(int pe, int block, uint32_t *sq_counter, uint32_t *published,
+                 uint32_t *atomic_counter, uint64_t mailbox[2]);
+/* Per-queue constants a CPU WQE builder needs. */
+int rsm_sq_constants(int pe, int block, uint32_t *ctrl_qp_sq, uint64_t *ctrl_sig, uint32_t *lkey,
+                     uint32_t *atomic_lkey, uint64_t *atomic_ret_base, uint32_t *max_nwqe);
+int rsm_sq_rkey(int dest_pe, uint32_t *rkey);
+
+/* ---- wave-level known-answer drivers ----------------------------------------------
+ * Block::fetch_incr contract (containers/share_strategy.hpp:70-83): lanes named
+ * by `lane_mask` of every wave of an n_wgs x wg_size grid call the
+ * wave-aggregated fetch-and-add on one zeroed counter.  `per_thread` (host,
+ * n_wgs*wg_size uint64, ~0 for inactive lanes) gets each lane's value,
+ * `*counter_out` the final counter. */
+int rsm_kat_fetch_incr(uint64_t lane_mask, int n_wgs, int wg_size, uint64_t *per_thread,
+                       uint64_t *counter_out);
+/* WfCoalOn::coalesce contract (wf_coal_policy.cpp:57-172) for one wave: inputs
+ * are 64-entry host arrays; outputs must_send[64] (0/1) and out_size[64]. */
+int rsm_kat_coalesce(uint64_t lane_mask, const int32_t *pe, const uint64_t *src,
+                     const uint64_t *dst, const uint64_t *size, uint8_t *must_send,
+                     uint64_t *out_size);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif

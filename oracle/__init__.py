@@ -1,0 +1,284 @@
+"""ctypes front end of the CPU oracle (``oracle/*.c``).
+
+Test infrastructure: only the tests, the smoke run and the benchmark's
+CPU-baseline leg import this package.  The GPU library never does.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+
+SHORT, INT, LONG, LONGLONG, FLOAT, DOUBLE, BF16 = range(7)
+SUM, MAX, MIN, PROD, AND, OR, XOR = range(7)
+
+
+def build():
+    """Compile liboracle.so with gcc (seconds)."""
+    subprocess.run(["make", "-s", "-C", _HERE], check=True)
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        build()
+    lib = C.CDLL(_LIB_PATH)
+    vp, sz, i32, u64, u32 = C.c_void_p, C.c_size_t, C.c_int, C.c_uint64, C.c_uint32
+    lib.orc_dtype_size.restype = sz
+    lib.orc_dtype_size.argtypes = [i32]
+    lib.orc_to_all.argtypes = [i32, i32, vp, sz, sz, sz, sz, i32, i32, i32]
+    lib.orc_to_all_mt.argtypes = [i32, i32, vp, sz, sz, sz, sz, i32, i32, i32, i32]
+    lib.orc_to_all_f64.argtypes = [i32, i32, vp, sz, sz, sz, i32, i32, i32, vp]
+    lib.orc_abs_sum_f64.argtypes = [i32, vp, sz, sz, sz, i32, i32, i32, vp]
+    lib.orc_float_to_bf16.restype = C.c_uint16
+    lib.orc_float_to_bf16.argtypes = [C.c_float]
+    lib.orc_bf16_to_float.restype = C.c_float
+    lib.orc_bf16_to_float.argtypes = [C.c_uint16]
+    for name in ("orc_put", "orc_get"):
+        getattr(lib, name).restype = None
+        getattr(lib, name).argtypes = [vp, sz, sz, sz, sz, i32, i32]
+    lib.orc_broadcast.restype = None
+    lib.orc_broadcast.argtypes = [vp, sz, sz, sz, sz, i32, i32, i32, i32]
+    for name in ("orc_alltoall", "orc_fcollect"):
+        getattr(lib, name).restype = None
+        getattr(lib, name).argtypes = [vp, sz, sz, sz, sz, i32, i32, i32]
+    lib.orc_copy_mt.restype = None
+    lib.orc_copy_mt.argtypes = [vp, vp, sz, i32]
+    lib.orc_small_ops.argtypes = [vp, sz, vp, vp, sz, vp]
+    lib.orc_wqe_build.restype = None
+    lib.orc_wqe_build.argtypes = [vp, vp, u32, vp]
+    lib.orc_doorbell.restype = None
+    lib.orc_doorbell.argtypes = [vp, u32, vp]
+    lib.orc_bswap16.restype = C.c_uint16
+    lib.orc_bswap16.argtypes = [C.c_uint16]
+    lib.orc_bswap32.restype = u32
+    lib.orc_bswap32.argtypes = [u32]
+    lib.orc_bswap64.restype = u64
+    lib.orc_bswap64.argtypes = [u64]
+    lib.orc_coalesce.restype = None
+    lib.orc_coalesce.argtypes = [u64, vp, vp, vp, vp, vp, vp]
+    lib.orc_fetch_incr.restype = None
+    lib.orc_fetch_incr.argtypes = [u64, vp, vp]
+    lib.orc_alloc_create.restype = vp
+    lib.orc_alloc_create.argtypes = [sz]
+    lib.orc_alloc_destroy.restype = None
+    lib.orc_alloc_destroy.argtypes = [vp]
+    lib.orc_alloc_alloc.restype = sz
+    lib.orc_alloc_alloc.argtypes = [vp, sz]
+    lib.orc_alloc_free.argtypes = [vp, sz]
+    lib.orc_alloc_in_use.restype = sz
+    lib.orc_alloc_in_use.argtypes = [vp]
+    return lib
+
+
+_lib = _load()
+
+NP_DTYPE = {SHORT: np.int16, INT: np.int32, LONG: np.int64, LONGLONG: np.int64,
+            FLOAT: np.float32, DOUBLE: np.float64, BF16: np.uint16}
+
+SMALL_OP_DTYPE = np.dtype([("kind", "<u4"), ("pe", "<u4"), ("offset", "<u8"),
+                           ("value", "<i8"), ("aux", "<i8")])
+
+
+def dtype_size(dtype):
+    return int(_lib.orc_dtype_size(dtype))
+
+
+class Heap:
+    """All PE slices in one host buffer: slice p is ``buf[p*stride:(p+1)*stride]``."""
+
+    def __init__(self, n_pes, stride, fill=0):
+        self.n_pes = n_pes
+        self.stride = stride
+        self.buf = np.full(n_pes * stride, fill, dtype=np.uint8)
+
+    @property
+    def ptr(self):
+        return self.buf.ctypes.data
+
+    def view(self, pe, offset, count, np_dtype):
+        start = pe * self.stride + offset
+        nbytes = count * np.dtype(np_dtype).itemsize
+        return self.buf[start:start + nbytes].view(np_dtype)
+
+
+def to_all(heap, dtype, op, dest_off, src_off, n, pe_start=0, log_stride=0, pe_size=None,
+           threads=1):
+    pe_size = heap.n_pes if pe_size is None else pe_size
+    if threads > 1:
+        rc = _lib.orc_to_all_mt(dtype, op, heap.ptr, heap.stride, dest_off, src_off, n, pe_start,
+                                log_stride, pe_size, threads)
+    else:
+        rc = _lib.orc_to_all(dtype, op, heap.ptr, heap.stride, dest_off, src_off, n, pe_start,
+                             log_stride, pe_size)
+    if rc != 0:
+        raise ValueError("reduction not defined for this (dtype, op)")
+
+
+def to_all_f64(heap, dtype, op, src_off, n, pe_start=0, log_stride=0, pe_size=None):
+    pe_size = heap.n_pes if pe_size is None else pe_size
+    out = np.empty(n, dtype=np.float64)
+    rc = _lib.orc_to_all_f64(dtype, op, heap.ptr, heap.stride, src_off, n, pe_start, log_stride,
+                             pe_size, out.ctypes.data)
+    if rc != 0:
+        raise ValueError("ground truth not defined for this (dtype, op)")
+    return out
+
+
+def abs_sum_f64(heap, dtype, src_off, n, pe_start=0, log_stride=0, pe_size=None):
+    pe_size = heap.n_pes if pe_size is None else pe_size
+    out = np.empty(n, dtype=np.float64)
+    _lib.orc_abs_sum_f64(dtype, heap.ptr, heap.stride, src_off, n, pe_start, log_stride, pe_size,
+                         out.ctypes.data)
+    return out
+
+
+def float_to_bf16(x):
+    """Round float32 array to bfloat16 bit patterns (nearest even)."""
+    u = np.asarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    r = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
+    r = np.where(nan, (u >> 16) | 0x40, r)
+    return r.astype(np.uint16)
+
+
+def bf16_to_float(b):
+    return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def put(heap, dest_off, src_off, nbytes, src_pe, dest_pe):
+    _lib.orc_put(heap.ptr, heap.stride, dest_off, src_off, nbytes, src_pe, dest_pe)
+
+
+def get(heap, dest_off, src_off, nbytes, my_pe, from_pe):
+    _lib.orc_get(heap.ptr, heap.stride, dest_off, src_off, nbytes, my_pe, from_pe)
+
+
+def broadcast(heap, dest_off, src_off, nbytes, root_idx, pe_start=0, log_stride=0, pe_size=None):
+    pe_size = heap.n_pes if pe_size is None else pe_size
+    _lib.orc_broadcast(heap.ptr, heap.stride, dest_off, src_off, nbytes, root_idx, pe_start,
+                       log_stride, pe_size)
+
+
+def alltoall(heap, dest_off, src_off, block_bytes, pe_start=0, log_stride=0, pe_size=None):
+    pe_size = heap.n_pes if pe_size is None else pe_size
+    _lib.orc_alltoall(heap.ptr, heap.stride, dest_off, src_off, block_bytes, pe_start, log_stride,
+                      pe_size)
+
+
+def fcollect(heap, dest_off, src_off, block_bytes, pe_start=0, log_stride=0, pe_size=None):
+    pe_size = heap.n_pes if pe_size is None else pe_size
+    _lib.orc_fcollect(heap.ptr, heap.stride, dest_off, src_off, block_bytes, pe_start, log_stride,
+                      pe_size)
+
+
+def copy_mt(dst, src, threads):
+    assert dst.nbytes == src.nbytes
+    _lib.orc_copy_mt(dst.ctypes.data, src.ctypes.data, src.nbytes, threads)
+
+
+def small_ops(heap, ops, issuer_pe):
+    ops = np.ascontiguousarray(ops, dtype=SMALL_OP_DTYPE)
+    issuer = np.ascontiguousarray(issuer_pe, dtype=np.uint32)
+    fetched = np.zeros(len(ops), dtype=np.int64)
+    rc = _lib.orc_small_ops(heap.ptr, heap.stride, ops.ctypes.data, issuer.ctypes.data, len(ops),
+                            fetched.ctypes.data)
+    if rc != 0:
+        raise ValueError("unknown small-op kind")
+    return fetched
+
+
+class Qp(C.Structure):
+    _fields_ = [("ctrl_qp_sq", C.c_uint32), ("ctrl_sig", C.c_uint64), ("lkey", C.c_uint32),
+                ("atomic_lkey", C.c_uint32), ("atomic_ret_base", C.c_uint64),
+                ("max_nwqe", C.c_uint32)]
+
+
+class WqeReq(C.Structure):
+    _fields_ = [("opcode", C.c_uint8), ("size", C.c_uint32), ("raddr", C.c_uint64),
+                ("rkey", C.c_uint32), ("laddr", C.c_uint64), ("atomic_data", C.c_uint64),
+                ("atomic_cmp", C.c_uint64), ("inline_bytes", C.c_uint8 * 8),
+                ("atomic_pos", C.c_uint32), ("request_cqe", C.c_int)]
+
+
+OP_WRITE, OP_READ, OP_ATOMIC_CS, OP_ATOMIC_FA = 0x08, 0x10, 0x11, 0x12
+
+
+def wqe_build(slot, qp, sq_counter, opcode, size=0, raddr=0, rkey=0, laddr=0, atomic_data=0,
+              atomic_cmp=0, inline=b"", atomic_pos=0, request_cqe=False):
+    """Write one entry into ``slot`` (a 64-byte uint8 array view), in place."""
+    assert slot.dtype == np.uint8 and slot.size == 64 and slot.flags["C_CONTIGUOUS"]
+    rq = WqeReq()
+    rq.opcode = opcode
+    rq.size = size
+    rq.raddr = raddr & 0xFFFFFFFFFFFFFFFF
+    rq.rkey = rkey
+    rq.laddr = laddr & 0xFFFFFFFFFFFFFFFF
+    rq.atomic_data = atomic_data & 0xFFFFFFFFFFFFFFFF
+    rq.atomic_cmp = atomic_cmp & 0xFFFFFFFFFFFFFFFF
+    for i, b in enumerate(bytes(inline)[:8]):
+        rq.inline_bytes[i] = b
+    rq.atomic_pos = atomic_pos
+    rq.request_cqe = 1 if request_cqe else 0
+    _lib.orc_wqe_build(slot.ctypes.data, C.byref(qp), sq_counter & 0xFFFFFFFF, C.byref(rq))
+    return slot
+
+
+def doorbell(last_slot, sq_counter_after):
+    out = np.zeros(2, dtype=np.uint64)
+    _lib.orc_doorbell(last_slot.ctypes.data, sq_counter_after & 0xFFFFFFFF, out.ctypes.data)
+    return out
+
+
+def bswap16(v):
+    return int(_lib.orc_bswap16(v))
+
+
+def bswap32(v):
+    return int(_lib.orc_bswap32(v))
+
+
+def bswap64(v):
+    return int(_lib.orc_bswap64(v))
+
+
+def coalesce(lane_mask, pe, src, dst, size):
+    pe = np.ascontiguousarray(pe, dtype=np.int32)
+    src = np.ascontiguousarray(src, dtype=np.uint64)
+    dst = np.ascontiguousarray(dst, dtype=np.uint64)
+    size = np.ascontiguousarray(size, dtype=np.uint64)
+    must = np.zeros(64, dtype=np.uint8)
+    out = np.zeros(64, dtype=np.uint64)
+    _lib.orc_coalesce(lane_mask, pe.ctypes.data, src.ctypes.data, dst.ctypes.data,
+                      size.ctypes.data, must.ctypes.data, out.ctypes.data)
+    return must, out
+
+
+def fetch_incr(lane_mask, counter):
+    ctr = C.c_uint64(counter)
+    out = np.zeros(64, dtype=np.uint64)
+    _lib.orc_fetch_incr(lane_mask, C.byref(ctr), out.ctypes.data)
+    return out, ctr.value
+
+
+class Allocator:
+    NONE = C.c_size_t(-1).value
+
+    def __init__(self, heap_bytes):
+        self._a = _lib.orc_alloc_create(heap_bytes)
+
+    def alloc(self, n):
+        return int(_lib.orc_alloc_alloc(self._a, n))
+
+    def free(self, off):
+        return int(_lib.orc_alloc_free(self._a, off))
+
+    def in_use(self):
+        return int(_lib.orc_alloc_in_use(self._a))
+
+    def __del__(self):
+        if getattr(self, "_a", None):
+            _lib.orc_alloc_destroy(self._a)
+            self._a = None

@@ -1,0 +1,136 @@
+/* oracle.h -- CPU restatement of the reference's algorithms for the device
+ * data path.  TEST INFRASTRUCTURE ONLY: it is the checker that tests, the
+ * smoke run and the benchmark's CPU-baseline leg compare the GPU library
+ * against; the library itself never calls it.
+ *
+ * All PEs are modelled in one address space: PE p's symmetric-heap slice is
+ * `heap + p*stride`.  Symmetric objects are named by their byte offset in the
+ * slice.  Each function cites the reference code it restates.
+ *
+ * Pinning status of each function (what independent evidence fixes it) is
+ * listed next to its definition.
+ */
+#ifndef ROCSHMEM_ORACLE_H
+#define ROCSHMEM_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum orc_dtype { ORC_SHORT = 0, ORC_INT, ORC_LONG, ORC_LONGLONG, ORC_FLOAT, ORC_DOUBLE, ORC_BF16 };
+enum orc_op { ORC_SUM = 0, ORC_MAX, ORC_MIN, ORC_PROD, ORC_AND, ORC_OR, ORC_XOR };
+
+size_t orc_dtype_size(int dtype);
+
+/* ---- reductions (reduce.c) ------------------------------------------------ */
+
+/* In-type fold in ascending member order, result to every member's dest.
+ * Returns 0, or -1 for an undefined (dtype, op) pair. */
+int orc_to_all(int dtype, int op, char *heap, size_t stride, size_t dest_off, size_t src_off,
+               size_t n, int pe_start, int log_stride, int pe_size);
+/* Ground truth: the same reduction evaluated in long double on the exact
+ * values of the inputs, returned as double.  out[n]. */
+int orc_to_all_f64(int dtype, int op, const char *heap, size_t stride, size_t src_off, size_t n,
+                   int pe_start, int log_stride, int pe_size, double *out);
+/* Sum over members of |x| per element (the scale of the tolerance test). */
+int orc_abs_sum_f64(int dtype, const char *heap, size_t stride, size_t src_off, size_t n,
+                    int pe_start, int log_stride, int pe_size, double *out);
+/* Multi-threaded orc_to_all over `threads` host threads (CPU baseline). */
+int orc_to_all_mt(int dtype, int op, char *heap, size_t stride, size_t dest_off, size_t src_off,
+                  size_t n, int pe_start, int log_stride, int pe_size, int threads);
+uint16_t orc_float_to_bf16(float f);
+float orc_bf16_to_float(uint16_t b);
+
+/* ---- put / get / broadcast / alltoall / fcollect (rma.c) ------------------- */
+
+void orc_put(char *heap, size_t stride, size_t dest_off, size_t src_off, size_t nbytes,
+             int src_pe, int dest_pe);
+void orc_get(char *heap, size_t stride, size_t dest_off, size_t src_off, size_t nbytes,
+             int my_pe, int from_pe);
+void orc_broadcast(char *heap, size_t stride, size_t dest_off, size_t src_off, size_t nbytes,
+                   int root_idx, int pe_start, int log_stride, int pe_size);
+void orc_alltoall(char *heap, size_t stride, size_t dest_off, size_t src_off, size_t block_bytes,
+                  int pe_start, int log_stride, int pe_size);
+void orc_fcollect(char *heap, size_t stride, size_t dest_off, size_t src_off, size_t block_bytes,
+                  int pe_start, int log_stride, int pe_size);
+/* memcpy spread over `threads` host threads (CPU baseline for put/get). */
+void orc_copy_mt(char *dst, const char *src, size_t nbytes, int threads);
+
+/* ---- small operations (amo.c) ----------------------------------------------- */
+
+typedef struct orc_small_op {
+  uint32_t kind;   /* same codes as rsm_small_kind */
+  uint32_t pe;
+  uint64_t offset;
+  int64_t value;
+  int64_t aux;
+} orc_small_op_t;
+
+/* Applies ops[0..n) one after the other (a legal serialisation) with op i
+ * issued by PE issuer_pe[i]; fetched[i] gets what a fetching op returns. */
+int orc_small_ops(char *heap, size_t stride, const orc_small_op_t *ops, const uint32_t *issuer_pe,
+                  size_t n, int64_t *fetched);
+
+/* ---- 64-byte WQE builder (wqe.c) ---------------------------------------------- */
+
+typedef struct orc_qp {
+  uint32_t ctrl_qp_sq;
+  uint64_t ctrl_sig;
+  uint32_t lkey;
+  uint32_t atomic_lkey;
+  uint64_t atomic_ret_base;
+  uint32_t max_nwqe;
+} orc_qp_t;
+
+typedef struct orc_wqe_req {
+  uint8_t opcode;        /* 0x08 write, 0x10 read, 0x11 compare-swap, 0x12 fetch-add */
+  uint32_t size;
+  uint64_t raddr;
+  uint32_t rkey;
+  uint64_t laddr;
+  uint64_t atomic_data;
+  uint64_t atomic_cmp;
+  uint8_t inline_bytes[8];
+  uint32_t atomic_pos;   /* return-slot index, already reduced modulo 4096 */
+  int request_cqe;       /* completion flag byte <- 8 */
+} orc_wqe_req_t;
+
+/* Overwrites, inside the 64-byte slot, exactly the bytes the reference writes. */
+void orc_wqe_build(uint8_t slot[64], const orc_qp_t *qp, uint32_t sq_counter,
+                   const orc_wqe_req_t *rq);
+/* Parse helpers used by the ring checker. */
+uint16_t orc_wqe_index(const uint8_t slot[64]);
+uint8_t orc_wqe_opcode(const uint8_t slot[64]);
+uint64_t orc_wqe_raddr(const uint8_t slot[64]);
+/* Doorbell record / doorbell value after the entry with counter `last_counter`
+ * closed a post that advanced the queue to `sq_counter_after`. */
+void orc_doorbell(const uint8_t last_slot[64], uint32_t sq_counter_after, uint64_t mailbox[2]);
+uint16_t orc_bswap16(uint16_t v);
+uint32_t orc_bswap32(uint32_t v);
+uint64_t orc_bswap64(uint64_t v);
+
+/* ---- wave-level models (wave.c) -------------------------------------------------- */
+
+/* WfCoalOn::coalesce for one 64-lane wave. */
+void orc_coalesce(uint64_t lane_mask, const int32_t *pe, const uint64_t *src, const uint64_t *dst,
+                  const uint64_t *size, uint8_t *must_send, uint64_t *out_size);
+/* Block::fetch_incr for one wave: returns the values the active lanes get,
+ * ~0 for inactive lanes; *counter advances by the number of active lanes. */
+void orc_fetch_incr(uint64_t lane_mask, uint64_t *counter, uint64_t out[64]);
+
+/* ---- symmetric allocator model (alloc.c) ------------------------------------------- */
+
+typedef struct orc_alloc orc_alloc_t;
+orc_alloc_t *orc_alloc_create(size_t heap_bytes);
+void orc_alloc_destroy(orc_alloc_t *a);
+size_t orc_alloc_alloc(orc_alloc_t *a, size_t request);   /* (size_t)-1 when nothing fits */
+int orc_alloc_free(orc_alloc_t *a, size_t offset);
+size_t orc_alloc_in_use(const orc_alloc_t *a);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,328 @@
+// C ABI: lifecycle, teams, plumbing and send-queue inspection.
+#include <cstring>
+#include <mutex>
+
+#include "cabi_common.hpp"
+#include "roc_shmem.hpp"
+
+namespace rsm {
+
+static std::string g_error;
+static std::mutex g_error_mu;
+
+int fail(const std::string &msg) {
+  std::lock_guard<std::mutex> lk(g_error_mu);
+  g_error = msg;
+  return -1;
+}
+void clear_error() {
+  std::lock_guard<std::mutex> lk(g_error_mu);
+  g_error.clear();
+}
+
+bool resolve_launch(const rsm_launch_t *in, Launch *out) {
+  using rocshmem::host::Runtime;
+  Runtime *rt = Runtime::get();
+  if (!rt) {
+    fail("rsm_init has not been called");
+    return false;
+  }
+  if (!in) {
+    fail("launch description is NULL");
+    return false;
+  }
+  if (in->wgs_per_pe < 1 || in->wg_size < 64 || in->wg_size > 1024 || (in->wg_size % 64)) {
+    fail("launch: wgs_per_pe must be >= 1 and wg_size a multiple of 64 in [64, 1024]");
+    return false;
+  }
+  unsigned long long grid = 1ull * in->wgs_per_pe * rt->num_pes();
+  if (grid > 0x7fffffffull) {
+    fail("launch: grid too large");
+    return false;
+  }
+  out->wgs_per_pe = in->wgs_per_pe;
+  out->wg_size = in->wg_size;
+  out->tile = in->tile;
+  out->stream = static_cast<hipStream_t>(in->stream);
+  out->grid = static_cast<unsigned>(grid);
+  return true;
+}
+
+bool check_symmetric(const void *p, const char *what, bool allow_null) {
+  using rocshmem::host::Runtime;
+  Runtime *rt = Runtime::get();
+  if (!p) {
+    if (allow_null) return true;
+    fail(std::string(what) + " is NULL");
+    return false;
+  }
+  if (!rt || rt->pe_of(p) != 0) {
+    fail(std::string(what) + " is not a symmetric address of PE 0");
+    return false;
+  }
+  return true;
+}
+
+int after_launch(const char *what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(std::string(what) + ": " + hipGetErrorString(e));
+  return 0;
+}
+
+}  // namespace rsm
+
+using rocshmem::host::Options;
+using rocshmem::host::Runtime;
+namespace detail = rocshmem::detail;
+
+#define RSM_NEED_RT(rt)                                       \
+  Runtime *rt = Runtime::get();                               \
+  if (!rt) return rsm::fail("rsm_init has not been called")
+
+#define RSM_HIP(expr)                                                              \
+  do {                                                                             \
+    hipError_t e_ = (expr);                                                        \
+    if (e_ != hipSuccess)                                                          \
+      return rsm::fail(std::string(#expr " failed: ") + hipGetErrorString(e_));    \
+  } while (0)
+
+extern "C" {
+
+int rsm_init(int num_pes, size_t heap_bytes_per_pe, int num_blocks, unsigned sq_size) {
+  rsm::clear_error();
+  Options o = Options::from_env();
+  if (num_pes) o.num_pes = num_pes;
+  if (heap_bytes_per_pe) o.heap_size = heap_bytes_per_pe;
+  if (num_blocks) o.num_blocks = num_blocks;
+  if (sq_size) o.sq_size = sq_size;
+  std::string err = Runtime::create(o);
+  if (!err.empty()) return rsm::fail(err);
+  rocshmem::ROC_SHMEM_TEAM_WORLD =
+      reinterpret_cast<rocshmem::roc_shmem_team_t>(Runtime::get()->team_world());
+  return 0;
+}
+
+int rsm_finalize(void) {
+  Runtime::destroy();
+  rocshmem::ROC_SHMEM_TEAM_WORLD = nullptr;
+  return 0;
+}
+
+int rsm_is_initialized(void) { return Runtime::get() ? 1 : 0; }
+
+const char *rsm_last_error(void) {
+  static thread_local std::string copy;
+  std::lock_guard<std::mutex> lk(rsm::g_error_mu);
+  copy = rsm::g_error;
+  return copy.c_str();
+}
+
+int rsm_n_pes(void) { return Runtime::get() ? Runtime::get()->num_pes() : -1; }
+int rsm_num_blocks(void) { return Runtime::get() ? Runtime::get()->options().num_blocks : -1; }
+size_t rsm_heap_size(void) { return Runtime::get() ? Runtime::get()->options().heap_size : 0; }
+size_t rsm_slice_stride(void) { return Runtime::get() ? Runtime::get()->slice_stride() : 0; }
+
+void *rsm_malloc(size_t bytes) {
+  Runtime *rt = Runtime::get();
+  if (!rt) {
+    rsm::fail("rsm_init has not been called");
+    return nullptr;
+  }
+  int keep = rt->current_pe();
+  rt->set_current_pe(0);
+  void *p = rt->sym_malloc(bytes);
+  rt->set_current_pe(keep);
+  if (!p && bytes) rsm::fail("symmetric heap exhausted");
+  return p;
+}
+
+int rsm_free(void *ptr) {
+  RSM_NEED_RT(rt);
+  (void)hipDeviceSynchronize();
+  return rt->sym_free(ptr) ? 0 : rsm::fail("rsm_free: not an outstanding symmetric allocation");
+}
+
+size_t rsm_heap_bytes_in_use(void) { return Runtime::get() ? Runtime::get()->bytes_in_use() : 0; }
+
+void *rsm_ptr(const void *sym, int pe) {
+  Runtime *rt = Runtime::get();
+  return rt ? rt->translate(sym, pe) : nullptr;
+}
+
+void *rsm_heap_base(int pe) {
+  Runtime *rt = Runtime::get();
+  if (!rt || pe < 0 || pe >= rt->num_pes()) return nullptr;
+  return rt->slice_base(pe);
+}
+
+int rsm_take_status(void) {
+  RSM_NEED_RT(rt);
+  return static_cast<int>(rt->take_status());
+}
+
+uint64_t rsm_team_world(void) {
+  Runtime *rt = Runtime::get();
+  return rt ? reinterpret_cast<uint64_t>(rt->team_world()) : 0;
+}
+
+int rsm_team_split_strided(uint64_t parent, int start, int stride, int size, uint64_t *new_team) {
+  RSM_NEED_RT(rt);
+  if (!new_team) return rsm::fail("new_team is NULL");
+  detail::Team *out = nullptr;
+  int rc = rt->team_split(reinterpret_cast<detail::Team *>(parent), start, stride, size, &out);
+  *new_team = reinterpret_cast<uint64_t>(out);
+  if (rc != 0) return rsm::fail("team_split_strided: invalid arguments");
+  return 0;
+}
+
+int rsm_team_destroy(uint64_t team) {
+  RSM_NEED_RT(rt);
+  (void)hipDeviceSynchronize();
+  rt->team_destroy(reinterpret_cast<detail::Team *>(team));
+  return 0;
+}
+
+int rsm_team_n_pes(uint64_t team) {
+  return rocshmem::roc_shmem_team_n_pes(reinterpret_cast<rocshmem::roc_shmem_team_t>(team));
+}
+
+int rsm_team_translate_pe(uint64_t src_team, int src_pe, uint64_t dst_team) {
+  if (!Runtime::get()) return -1;
+  return rocshmem::roc_shmem_team_translate_pe(
+      reinterpret_cast<rocshmem::roc_shmem_team_t>(src_team), src_pe,
+      reinterpret_cast<rocshmem::roc_shmem_team_t>(dst_team));
+}
+
+int rsm_copy_to_device(void *dst, const void *host_src, size_t bytes) {
+  RSM_HIP(hipMemcpy(dst, host_src, bytes, hipMemcpyHostToDevice));
+  return 0;
+}
+int rsm_copy_to_host(void *host_dst, const void *src, size_t bytes) {
+  RSM_HIP(hipMemcpy(host_dst, src, bytes, hipMemcpyDeviceToHost));
+  return 0;
+}
+int rsm_fill(void *dst, int byte_value, size_t bytes) {
+  RSM_HIP(hipMemset(dst, byte_value, bytes));
+  return 0;
+}
+int rsm_synchronize(void) {
+  RSM_HIP(hipDeviceSynchronize());
+  return 0;
+}
+void *rsm_device_alloc(size_t bytes) {
+  void *p = nullptr;
+  if (hipMalloc(&p, bytes) != hipSuccess) {
+    rsm::fail("hipMalloc failed");
+    return nullptr;
+  }
+  return p;
+}
+int rsm_device_free(void *ptr) {
+  RSM_HIP(hipFree(ptr));
+  return 0;
+}
+void *rsm_stream_create(void) {
+  hipStream_t s = nullptr;
+  if (hipStreamCreate(&s) != hipSuccess) {
+    rsm::fail("hipStreamCreate failed");
+    return nullptr;
+  }
+  return s;
+}
+int rsm_stream_destroy(void *stream) {
+  RSM_HIP(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+  return 0;
+}
+void *rsm_event_create(void) {
+  hipEvent_t e = nullptr;
+  if (hipEventCreate(&e) != hipSuccess) {
+    rsm::fail("hipEventCreate failed");
+    return nullptr;
+  }
+  return e;
+}
+int rsm_event_destroy(void *event) {
+  RSM_HIP(hipEventDestroy(static_cast<hipEvent_t>(event)));
+  return 0;
+}
+int rsm_event_record(void *event, void *stream) {
+  RSM_HIP(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
+  return 0;
+}
+int rsm_event_elapsed_ms(void *start, void *stop, float *ms) {
+  RSM_HIP(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
+  RSM_HIP(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+  return 0;
+}
+
+// ---- send-queue inspection ---------------------------------------------------
+
+static bool sq_args_ok(Runtime *rt, int pe, int block) {
+  return pe >= 0 && pe < rt->num_pes() && block >= 0 && block < rt->options().num_blocks;
+}
+
+int rsm_sq_reset(void) {
+  RSM_NEED_RT(rt);
+  RSM_HIP(hipDeviceSynchronize());
+  rt->reset_queues(nullptr);
+  RSM_HIP(hipDeviceSynchronize());
+  return 0;
+}
+
+int rsm_sq_read(int pe, int block, unsigned index, uint64_t out_words[8]) {
+  RSM_NEED_RT(rt);
+  if (!sq_args_ok(rt, pe, block) || index >= rt->options().sq_size)
+    return rsm::fail("rsm_sq_read: arguments out of range");
+  RSM_HIP(hipDeviceSynchronize());
+  RSM_HIP(hipMemcpy(out_words, rt->ctx_image(pe, block).ring.sq + 8ull * index, 64,
+                    hipMemcpyDeviceToHost));
+  return 0;
+}
+
+int rsm_sq_image(int pe, int block, void *host_out, size_t bytes) {
+  RSM_NEED_RT(rt);
+  if (!sq_args_ok(rt, pe, block) || bytes > 64ull * rt->options().sq_size)
+    return rsm::fail("rsm_sq_image: arguments out of range");
+  RSM_HIP(hipDeviceSynchronize());
+  RSM_HIP(hipMemcpy(host_out, rt->ctx_image(pe, block).ring.sq, bytes, hipMemcpyDeviceToHost));
+  return 0;
+}
+
+int rsm_sq_state(int pe, int block, uint32_t *sq_counter, uint32_t *published,
+                 uint32_t *atomic_counter, uint64_t mailbox[2]) {
+  RSM_NEED_RT(rt);
+  if (!sq_args_ok(rt, pe, block)) return rsm::fail("rsm_sq_state: arguments out of range");
+  RSM_HIP(hipDeviceSynchronize());
+  detail::SqCounters c;
+  const detail::DeviceCtx &ctx = rt->ctx_image(pe, block);
+  RSM_HIP(hipMemcpy(&c, ctx.counters, sizeof(c), hipMemcpyDeviceToHost));
+  if (sq_counter) *sq_counter = c.sq_counter;
+  if (published) *published = c.published;
+  if (atomic_counter) *atomic_counter = c.atomic_counter;
+  if (mailbox) RSM_HIP(hipMemcpy(mailbox, ctx.ring.mailbox, 16, hipMemcpyDeviceToHost));
+  return 0;
+}
+
+int rsm_sq_constants(int pe, int block, uint32_t *ctrl_qp_sq, uint64_t *ctrl_sig, uint32_t *lkey,
+                     uint32_t *atomic_lkey, uint64_t *atomic_ret_base, uint32_t *max_nwqe) {
+  RSM_NEED_RT(rt);
+  if (!sq_args_ok(rt, pe, block)) return rsm::fail("rsm_sq_constants: arguments out of range");
+  const detail::SqRing &r = rt->ctx_image(pe, block).ring;
+  if (ctrl_qp_sq) *ctrl_qp_sq = r.ctrl_qp_sq;
+  if (ctrl_sig) *ctrl_sig = r.ctrl_sig;
+  if (lkey) *lkey = r.lkey;
+  if (atomic_lkey) *atomic_lkey = r.atomic_lkey;
+  if (atomic_ret_base) *atomic_ret_base = r.atomic_ret_base;
+  if (max_nwqe) *max_nwqe = r.max_nwqe;
+  return 0;
+}
+
+int rsm_sq_rkey(int dest_pe, uint32_t *rkey) {
+  RSM_NEED_RT(rt);
+  if (dest_pe < 0 || dest_pe >= rt->num_pes() || !rkey)
+    return rsm::fail("rsm_sq_rkey: arguments out of range");
+  *rkey = __builtin_bswap32(0x1000u + dest_pe);
+  return 0;
+}
+
+}  // extern "C"

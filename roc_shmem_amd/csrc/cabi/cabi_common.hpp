@@ -1,0 +1,36 @@
+// Shared helpers of the C-ABI translation units.
+#ifndef ROCSHMEM_MI355X_CABI_COMMON_HPP
+#define ROCSHMEM_MI355X_CABI_COMMON_HPP
+
+#include <hip/hip_runtime.h>
+
+#include <string>
+
+#include "host/runtime.hpp"
+#include "rocshmem_mi355x.h"
+
+namespace rsm {
+
+int fail(const std::string &msg);   // records the message, returns -1
+void clear_error();
+
+struct Launch {
+  int wgs_per_pe;
+  int wg_size;
+  size_t tile;
+  hipStream_t stream;
+  unsigned grid;   // wgs_per_pe * num_pes
+};
+
+// Validates the runtime and the launch shape; false (with the error set) on failure.
+bool resolve_launch(const rsm_launch_t *in, Launch *out);
+
+// True when `p` is a symmetric address in PE 0's slice (or NULL when allowed).
+bool check_symmetric(const void *p, const char *what, bool allow_null = false);
+
+// hipGetLastError() after a launch, folded into the error convention.
+int after_launch(const char *what);
+
+}  // namespace rsm
+
+#endif

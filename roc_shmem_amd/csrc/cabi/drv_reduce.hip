@@ -1,0 +1,231 @@
+// C ABI: reductions.  The kernels below drive the device API the way the
+// reference's ReductionTest kernel does (clients/functional_tests/
+// reduction_tester.cpp:74-104), for every PE of the job in one grid.
+#include "cabi_common.hpp"
+#include "roc_shmem.hpp"
+
+using namespace rocshmem;
+
+namespace {
+
+template <typename T, ROC_SHMEM_OP Op>
+struct ToAll;
+
+#define RSM_TO_ALL(T, TNAME, OPNAME, OP)                                                      \
+  template <>                                                                                 \
+  struct ToAll<T, OP> {                                                                       \
+    static __device__ __forceinline__ void active_set(roc_shmem_ctx_t ctx, T *dest,           \
+                                                      const T *source, int n, int pe_start,   \
+                                                      int log_stride, int pe_size, T *pWrk,   \
+                                                      long *pSync) {                          \
+      roc_shmem_ctx_##TNAME##_##OPNAME##_wg_to_all(ctx, dest, source, n, pe_start,            \
+                                                   log_stride, pe_size, pWrk, pSync);         \
+    }                                                                                         \
+    static __device__ __forceinline__ void team(roc_shmem_ctx_t ctx, roc_shmem_team_t team,   \
+                                                T *dest, const T *source, int n) {            \
+      roc_shmem_ctx_##TNAME##_##OPNAME##_wg_to_all(ctx, team, dest, source, n);               \
+    }                                                                                         \
+  };
+#define RSM_TO_ALL_ARITH(T, TNAME)            \
+  RSM_TO_ALL(T, TNAME, sum, ROC_SHMEM_SUM)    \
+  RSM_TO_ALL(T, TNAME, max, ROC_SHMEM_MAX)    \
+  RSM_TO_ALL(T, TNAME, min, ROC_SHMEM_MIN)    \
+  RSM_TO_ALL(T, TNAME, prod, ROC_SHMEM_PROD)
+#define RSM_TO_ALL_BITS(T, TNAME)             \
+  RSM_TO_ALL(T, TNAME, and, ROC_SHMEM_AND)    \
+  RSM_TO_ALL(T, TNAME, or, ROC_SHMEM_OR)      \
+  RSM_TO_ALL(T, TNAME, xor, ROC_SHMEM_XOR)
+RSM_TO_ALL_ARITH(short, short)
+RSM_TO_ALL_BITS(short, short)
+RSM_TO_ALL_ARITH(int, int)
+RSM_TO_ALL_BITS(int, int)
+RSM_TO_ALL_ARITH(long, long)
+RSM_TO_ALL_BITS(long, long)
+RSM_TO_ALL_ARITH(long long, longlong)
+RSM_TO_ALL_BITS(long long, longlong)
+RSM_TO_ALL_ARITH(float, float)
+RSM_TO_ALL_ARITH(double, double)
+RSM_TO_ALL(__hip_bfloat16, bf16, sum, ROC_SHMEM_SUM)
+RSM_TO_ALL(__hip_bfloat16, bf16, max, ROC_SHMEM_MAX)
+RSM_TO_ALL(__hip_bfloat16, bf16, min, ROC_SHMEM_MIN)
+
+template <typename T, ROC_SHMEM_OP Op>
+__global__ void __launch_bounds__(1024)
+    to_all_kernel(T *dest0, const T *source0, size_t n, size_t tile, int pe_start, int log_stride,
+                  int pe_size, T *pWrk0, long *pSync0) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  const int me = roc_shmem_ctx_my_pe(ctx);
+  const int npes = roc_shmem_ctx_n_pes(ctx);
+  const size_t w = blockIdx.x / npes;
+  const size_t nw = gridDim.x / npes;
+  const int rel = me - pe_start;
+  const bool member = rel >= 0 && (rel & ((1 << log_stride) - 1)) == 0 &&
+                      (rel >> log_stride) < pe_size;
+  if (member) {
+    T *dest = roc_shmemx_my_addr(dest0);
+    const T *source = roc_shmemx_my_addr(source0);
+    T *pWrk = roc_shmemx_my_addr(pWrk0);
+    long *pSync = roc_shmemx_my_addr(pSync0) + w * ROC_SHMEM_REDUCE_SYNC_SIZE;
+    for (size_t off = w * tile; off < n; off += nw * tile) {
+      size_t cnt = n - off < tile ? n - off : tile;
+      ToAll<T, Op>::active_set(ctx, dest + off, source + off, static_cast<int>(cnt), pe_start,
+                               log_stride, pe_size, pWrk, pSync);
+    }
+  }
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+template <typename T, ROC_SHMEM_OP Op>
+__global__ void __launch_bounds__(1024)
+    to_all_team_kernel(roc_shmem_team_t team, T *dest0, const T *source0, size_t n, size_t tile,
+                       int pe_start, int stride, int pe_size) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_team_create_ctx(team, ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  const int me = roc_shmem_ctx_my_pe(ctx);
+  const int npes = roc_shmem_ctx_n_pes(ctx);
+  const size_t w = blockIdx.x / npes;
+  const size_t nw = gridDim.x / npes;
+  const int rel = me - pe_start;
+  const bool member = rel >= 0 && rel % stride == 0 && rel / stride < pe_size;
+  if (member) {
+    T *dest = roc_shmemx_my_addr(dest0);
+    const T *source = roc_shmemx_my_addr(source0);
+    for (size_t off = w * tile; off < n; off += nw * tile) {
+      size_t cnt = n - off < tile ? n - off : tile;
+      ToAll<T, Op>::team(ctx, team, dest + off, source + off, static_cast<int>(cnt));
+    }
+  }
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+struct ReduceArgs {
+  void *dest;
+  const void *source;
+  size_t n;
+  size_t tile;
+  int pe_start, log_stride, pe_size;
+  void *pWrk;
+  long *pSync;
+  roc_shmem_team_t team;
+  int stride;
+};
+
+template <typename T, ROC_SHMEM_OP Op>
+void launch_one(const rsm::Launch &l, const ReduceArgs &a) {
+  if (a.team) {
+    hipLaunchKernelGGL((to_all_team_kernel<T, Op>), dim3(l.grid), dim3(l.wg_size), 0, l.stream,
+                       a.team, static_cast<T *>(a.dest), static_cast<const T *>(a.source), a.n,
+                       a.tile, a.pe_start, a.stride, a.pe_size);
+  } else {
+    hipLaunchKernelGGL((to_all_kernel<T, Op>), dim3(l.grid), dim3(l.wg_size), 0, l.stream,
+                       static_cast<T *>(a.dest), static_cast<const T *>(a.source), a.n, a.tile,
+                       a.pe_start, a.log_stride, a.pe_size, static_cast<T *>(a.pWrk), a.pSync);
+  }
+}
+
+template <typename T>
+bool launch_arith(int op, const rsm::Launch &l, const ReduceArgs &a) {
+  switch (op) {
+    case RSM_SUM: launch_one<T, ROC_SHMEM_SUM>(l, a); return true;
+    case RSM_MAX: launch_one<T, ROC_SHMEM_MAX>(l, a); return true;
+    case RSM_MIN: launch_one<T, ROC_SHMEM_MIN>(l, a); return true;
+    case RSM_PROD: launch_one<T, ROC_SHMEM_PROD>(l, a); return true;
+    default: return false;
+  }
+}
+
+template <typename T>
+bool launch_int(int op, const rsm::Launch &l, const ReduceArgs &a) {
+  switch (op) {
+    case RSM_AND: launch_one<T, ROC_SHMEM_AND>(l, a); return true;
+    case RSM_OR: launch_one<T, ROC_SHMEM_OR>(l, a); return true;
+    case RSM_XOR: launch_one<T, ROC_SHMEM_XOR>(l, a); return true;
+    default: return launch_arith<T>(op, l, a);
+  }
+}
+
+bool launch_bf16(int op, const rsm::Launch &l, const ReduceArgs &a) {
+  switch (op) {
+    case RSM_SUM: launch_one<__hip_bfloat16, ROC_SHMEM_SUM>(l, a); return true;
+    case RSM_MAX: launch_one<__hip_bfloat16, ROC_SHMEM_MAX>(l, a); return true;
+    case RSM_MIN: launch_one<__hip_bfloat16, ROC_SHMEM_MIN>(l, a); return true;
+    default: return false;
+  }
+}
+
+size_t dtype_size(int dtype) {
+  switch (dtype) {
+    case RSM_SHORT: case RSM_BF16: return 2;
+    case RSM_INT: case RSM_FLOAT: return 4;
+    case RSM_LONG: case RSM_LONGLONG: case RSM_DOUBLE: return 8;
+    default: return 0;
+  }
+}
+
+int run(int dtype, int op, const rsm::Launch &l, ReduceArgs a) {
+  const size_t es = dtype_size(dtype);
+  if (!es) return rsm::fail("to_all: unknown dtype");
+  if (a.n == 0) return 0;  // zero-element reductions are no-ops (context_tmpl_device.hpp:68-70)
+  if (a.tile == 0) {
+    size_t t = (a.n + l.wgs_per_pe - 1) / l.wgs_per_pe;
+    a.tile = (t + 1023) / 1024 * 1024;
+  }
+  if (a.tile > 0x7fffffffull) return rsm::fail("to_all: tile does not fit the API's int nreduce");
+  bool ok = false;
+  switch (dtype) {
+    case RSM_SHORT: ok = launch_int<short>(op, l, a); break;
+    case RSM_INT: ok = launch_int<int>(op, l, a); break;
+    case RSM_LONG: ok = launch_int<long>(op, l, a); break;
+    case RSM_LONGLONG: ok = launch_int<long long>(op, l, a); break;
+    case RSM_FLOAT: ok = launch_arith<float>(op, l, a); break;
+    case RSM_DOUBLE: ok = launch_arith<double>(op, l, a); break;
+    case RSM_BF16: ok = launch_bf16(op, l, a); break;
+  }
+  if (!ok) return rsm::fail("to_all: operator not defined for this dtype");
+  return rsm::after_launch("to_all");
+}
+
+}  // namespace
+
+extern "C" {
+
+int rsm_to_all(int dtype, int op, void *dest, const void *source, size_t nreduce, int pe_start,
+               int log_pe_stride, int pe_size, void *pWrk, long *pSync,
+               const rsm_launch_t *launch) {
+  rsm::Launch l;
+  if (!rsm::resolve_launch(launch, &l)) return -1;
+  host::Runtime *rt = host::Runtime::get();
+  if (!rsm::check_symmetric(dest, "dest") || !rsm::check_symmetric(source, "source") ||
+      !rsm::check_symmetric(pSync, "pSync") || !rsm::check_symmetric(pWrk, "pWrk", true))
+    return -1;
+  if (pe_start < 0 || log_pe_stride < 0 || log_pe_stride > 30 || pe_size < 1 ||
+      pe_size > detail::kMaxPes ||
+      pe_start + ((pe_size - 1) << log_pe_stride) >= rt->num_pes())
+    return rsm::fail("to_all: active set out of range");
+  ReduceArgs a{dest, source, nreduce, l.tile, pe_start, log_pe_stride, pe_size, pWrk, pSync,
+               nullptr, 1 << log_pe_stride};
+  return run(dtype, op, l, a);
+}
+
+int rsm_to_all_team(int dtype, int op, uint64_t team, void *dest, const void *source,
+                    size_t nreduce, const rsm_launch_t *launch) {
+  rsm::Launch l;
+  if (!rsm::resolve_launch(launch, &l)) return -1;
+  host::Runtime *rt = host::Runtime::get();
+  if (!rsm::check_symmetric(dest, "dest") || !rsm::check_symmetric(source, "source")) return -1;
+  const host::TeamRecord *rec = rt->team_record(reinterpret_cast<detail::Team *>(team));
+  if (!rec) return rsm::fail("to_all_team: invalid team");
+  if (l.wgs_per_pe > rt->options().num_blocks)
+    return rsm::fail("to_all_team: wgs_per_pe exceeds the contexts per PE (team pSync slices)");
+  const detail::TeamInfo &ti = rec->image.wrt_world;
+  ReduceArgs a{dest, source, nreduce, l.tile, ti.pe_start, ti.log_stride, ti.size, nullptr,
+               nullptr, reinterpret_cast<roc_shmem_team_t>(team), ti.stride};
+  return run(dtype, op, l, a);
+}
+
+}  // extern "C"

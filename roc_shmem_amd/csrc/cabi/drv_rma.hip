@@ -1,0 +1,90 @@
+// C ABI: workgroup-, wavefront- and thread-level put/get.  The kernel mirrors
+// the reference's ExtendedPrimitiveTest / PrimitiveTest kernels
+// (clients/functional_tests/extended_primitives.cpp:33-76,
+// primitive_tester.cpp:32-82), with every PE of the job in one grid.
+#include "cabi_common.hpp"
+#include "roc_shmem.hpp"
+
+using namespace rocshmem;
+
+namespace {
+
+__global__ void __launch_bounds__(1024)
+    rma_kernel(int kind, int granularity, char *dest0, const char *source0, size_t msg_bytes,
+               size_t n_msgs, size_t dst_stride, size_t src_stride, int pe_shift) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  const int me = roc_shmem_ctx_my_pe(ctx);
+  const int npes = roc_shmem_ctx_n_pes(ctx);
+  const int target = (me + pe_shift) % npes;
+  const size_t w = blockIdx.x / npes;
+  const size_t nw = gridDim.x / npes;
+  char *dest = roc_shmemx_my_addr(dest0);
+  const char *source = roc_shmemx_my_addr(source0);
+
+  if (granularity == RSM_WG) {
+    for (size_t m = w; m < n_msgs; m += nw) {
+      char *d = dest + m * dst_stride;
+      const char *s = source + m * src_stride;
+      switch (kind) {
+        case RSM_PUT: roc_shmemx_ctx_putmem_wg(ctx, d, s, msg_bytes, target); break;
+        case RSM_GET: roc_shmemx_ctx_getmem_wg(ctx, d, s, msg_bytes, target); break;
+        case RSM_PUT_NBI: roc_shmemx_ctx_putmem_nbi_wg(ctx, d, s, msg_bytes, target); break;
+        default: roc_shmemx_ctx_getmem_nbi_wg(ctx, d, s, msg_bytes, target); break;
+      }
+    }
+  } else if (granularity == RSM_WAVE) {
+    const size_t waves_per_wg = blockDim.x / 64;
+    const size_t wave = w * waves_per_wg + threadIdx.x / 64;
+    const size_t n_waves = nw * waves_per_wg;
+    for (size_t m = wave; m < n_msgs; m += n_waves) {
+      char *d = dest + m * dst_stride;
+      const char *s = source + m * src_stride;
+      switch (kind) {
+        case RSM_PUT: roc_shmemx_ctx_putmem_wave(ctx, d, s, msg_bytes, target); break;
+        case RSM_GET: roc_shmemx_ctx_getmem_wave(ctx, d, s, msg_bytes, target); break;
+        case RSM_PUT_NBI: roc_shmemx_ctx_putmem_nbi_wave(ctx, d, s, msg_bytes, target); break;
+        default: roc_shmemx_ctx_getmem_nbi_wave(ctx, d, s, msg_bytes, target); break;
+      }
+    }
+  } else {
+    const size_t thread = w * blockDim.x + threadIdx.x;
+    const size_t n_threads = nw * blockDim.x;
+    for (size_t m = thread; m < n_msgs; m += n_threads) {
+      char *d = dest + m * dst_stride;
+      const char *s = source + m * src_stride;
+      switch (kind) {
+        case RSM_PUT: roc_shmem_ctx_putmem(ctx, d, s, msg_bytes, target); break;
+        case RSM_GET: roc_shmem_ctx_getmem(ctx, d, s, msg_bytes, target); break;
+        case RSM_PUT_NBI: roc_shmem_ctx_putmem_nbi(ctx, d, s, msg_bytes, target); break;
+        default: roc_shmem_ctx_getmem_nbi(ctx, d, s, msg_bytes, target); break;
+      }
+    }
+  }
+  roc_shmem_ctx_quiet(ctx);
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+}  // namespace
+
+extern "C" int rsm_rma(int kind, int granularity, void *dest, const void *source,
+                       size_t msg_bytes, size_t n_msgs, size_t dst_stride, size_t src_stride,
+                       int pe_shift, const rsm_launch_t *launch) {
+  rsm::Launch l;
+  if (!rsm::resolve_launch(launch, &l)) return -1;
+  if (kind < RSM_PUT || kind > RSM_GET_NBI) return rsm::fail("rma: unknown kind");
+  if (granularity < RSM_THREAD || granularity > RSM_WG) return rsm::fail("rma: unknown granularity");
+  if (!dest || !source) return rsm::fail("rma: NULL buffer");
+  host::Runtime *rt = host::Runtime::get();
+  // The remote side of the transfer must be symmetric.
+  const void *remote = (kind == RSM_PUT || kind == RSM_PUT_NBI) ? dest : source;
+  if (rt->pe_of(remote) != 0) return rsm::fail("rma: the remote buffer is not a symmetric address of PE 0");
+  if (pe_shift < 0) return rsm::fail("rma: pe_shift must be non-negative");
+  if (n_msgs == 0) return 0;
+  hipLaunchKernelGGL(rma_kernel, dim3(l.grid), dim3(l.wg_size), 0, l.stream, kind, granularity,
+                     static_cast<char *>(dest), static_cast<const char *>(source), msg_bytes,
+                     n_msgs, dst_stride, src_stride, pe_shift);
+  return rsm::after_launch("rma");
+}

@@ -1,0 +1,397 @@
+#include "runtime.hpp"
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <sstream>
+
+namespace rocshmem {
+namespace host {
+
+// ---------------------------------------------------------------------------
+// Pow2Allocator
+// ---------------------------------------------------------------------------
+
+static size_t round_up_pow2(size_t v) {
+  size_t p = Pow2Allocator::kMinBlock;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+Pow2Allocator::Pow2Allocator(size_t heap_bytes) : heap_bytes_(heap_bytes) {
+  // One bin per power of two from the floor up to the largest power of two
+  // that fits; the heap is handed to the bins as its binary decomposition,
+  // largest block at the lowest address.
+  size_t top = kMinBlock;
+  while ((top << 1) <= heap_bytes && (top << 1) != 0) top <<= 1;
+  for (size_t s = kMinBlock; s <= top; s <<= 1) bins_[s];
+  size_t offset = 0;
+  for (size_t s = top; s >= kMinBlock; s >>= 1) {
+    if (heap_bytes - offset >= s) {
+      bins_[s].push_back(offset);
+      offset += s;
+    }
+  }
+}
+
+bool Pow2Allocator::refill(std::map<size_t, std::vector<size_t>>::iterator it) {
+  auto next = std::next(it);
+  if (next == bins_.end()) return false;
+  if (next->second.empty() && !refill(next)) return false;
+  size_t block = next->second.back();
+  next->second.pop_back();
+  // Upper half goes in first so that the lower half is handed out first.
+  it->second.push_back(block + it->first);
+  it->second.push_back(block);
+  return true;
+}
+
+size_t Pow2Allocator::alloc(size_t request) {
+  if (request == 0) return kNoOffset;
+  size_t want = round_up_pow2(request);
+  auto it = bins_.find(want);
+  if (it == bins_.end()) return kNoOffset;
+  if (it->second.empty() && !refill(it)) return kNoOffset;
+  size_t off = it->second.back();
+  it->second.pop_back();
+  outstanding_[off] = want;
+  return off;
+}
+
+bool Pow2Allocator::free(size_t offset) {
+  auto it = outstanding_.find(offset);
+  if (it == outstanding_.end()) return false;
+  bins_[it->second].push_back(offset);
+  outstanding_.erase(it);
+  return true;
+}
+
+size_t Pow2Allocator::bytes_in_use() const {
+  size_t total = 0;
+  for (const auto &kv : outstanding_) total += kv.second;
+  return total;
+}
+
+// ---------------------------------------------------------------------------
+// Options
+// ---------------------------------------------------------------------------
+
+static bool env_u64(const char *name, unsigned long long *out) {
+  const char *s = getenv(name);
+  if (!s || !*s) return false;
+  char *end = nullptr;
+  unsigned long long v = strtoull(s, &end, 0);
+  if (end == s) return false;
+  *out = v;
+  return true;
+}
+
+Options Options::from_env() {
+  Options o;
+  unsigned long long v;
+  if (env_u64("ROC_SHMEM_NUM_PES", &v)) o.num_pes = static_cast<int>(v);
+  if (env_u64("ROC_SHMEM_HEAP_SIZE", &v)) o.heap_size = static_cast<size_t>(v);
+  if (env_u64("ROC_SHMEM_NUM_BLOCKS", &v)) o.num_blocks = static_cast<int>(v);
+  if (env_u64("ROC_SHMEM_SQ_SIZE", &v)) o.sq_size = static_cast<uint32_t>(v);
+  if (env_u64("ROC_SHMEM_SLICE_PAD", &v)) o.slice_pad = static_cast<size_t>(v);
+  if (const char *s = getenv("ROC_SHMEM_WAIT_LIMIT_S")) {
+    double d = atof(s);
+    if (d > 0) o.wait_limit_s = d;
+  }
+  return o;
+}
+
+// ---------------------------------------------------------------------------
+// Runtime
+// ---------------------------------------------------------------------------
+
+Runtime *Runtime::instance_ = nullptr;
+
+#define RT_HIP(expr)                                                             \
+  do {                                                                           \
+    hipError_t e_ = (expr);                                                      \
+    if (e_ != hipSuccess) {                                                      \
+      std::ostringstream os_;                                                    \
+      os_ << #expr << " failed: " << hipGetErrorString(e_);                      \
+      return os_.str();                                                          \
+    }                                                                            \
+  } while (0)
+
+std::string Runtime::create(const Options &opt) {
+  if (instance_) return "runtime already initialised";
+  Runtime *rt = new Runtime();
+  std::string err = rt->init(opt);
+  if (!err.empty()) {
+    rt->teardown();
+    delete rt;
+    return err;
+  }
+  instance_ = rt;
+  return "";
+}
+
+void Runtime::destroy() {
+  if (!instance_) return;
+  instance_->teardown();
+  delete instance_;
+  instance_ = nullptr;
+}
+
+static uint32_t bswap32(uint32_t v) { return __builtin_bswap32(v); }
+
+std::string Runtime::init(const Options &opt) {
+  opt_ = opt;
+  if (opt_.num_pes < 1 || opt_.num_pes > detail::kMaxPes)
+    return "ROC_SHMEM_NUM_PES must be in [1, 128]";
+  if (opt_.num_blocks < 1) return "ROC_SHMEM_NUM_BLOCKS must be positive";
+  if (opt_.sq_size < 2 || (opt_.sq_size & (opt_.sq_size - 1)))
+    return "ROC_SHMEM_SQ_SIZE must be a power of two";
+  if (opt_.heap_size < (1u << 20) || (opt_.heap_size & 4095))
+    return "ROC_SHMEM_HEAP_SIZE must be a multiple of 4096 and at least 1 MiB";
+  if (opt_.slice_pad & 4095) return "ROC_SHMEM_SLICE_PAD must be a multiple of 4096";
+
+  const int P = opt_.num_pes;
+  const int B = opt_.num_blocks;
+  stride_ = opt_.heap_size + opt_.slice_pad;
+  RT_HIP(hipMalloc(reinterpret_cast<void **>(&arena_), stride_ * P));
+  alloc_ = Pow2Allocator(opt_.heap_size);
+
+  // Slice base table (reference: RemoteHeapInfo's base_heap[], remote_heap_info.hpp:142-152).
+  std::vector<char *> bases(P);
+  for (int p = 0; p < P; ++p) bases[p] = slice_base(p);
+  RT_HIP(hipMalloc(reinterpret_cast<void **>(&base_heap_dev_), sizeof(char *) * P));
+  RT_HIP(hipMemcpy(base_heap_dev_, bases.data(), sizeof(char *) * P, hipMemcpyHostToDevice));
+
+  // Send queues.  Per ring: sq_size 64-byte slots, a 64-byte mailbox
+  // (doorbell record + doorbell value) and the AMO return window.
+  const size_t ring_bytes = static_cast<size_t>(opt_.sq_size) * 64 + 64 +
+                            static_cast<size_t>(detail::kAtomicRetSlots) * 8;
+  const size_t rings = static_cast<size_t>(P) * B;
+  queue_mem_bytes_ = ring_bytes * rings;
+  RT_HIP(hipMalloc(reinterpret_cast<void **>(&queue_mem_), queue_mem_bytes_));
+  RT_HIP(hipMemset(queue_mem_, 0, queue_mem_bytes_));
+  RT_HIP(hipMalloc(reinterpret_cast<void **>(&counters_dev_), sizeof(detail::SqCounters) * rings));
+  RT_HIP(hipMemset(counters_dev_, 0, sizeof(detail::SqCounters) * rings));
+
+  // Synthetic queue-pair constants standing in for what the reference
+  // harvests from a NIC-built template WQE (connection.cpp:379-391).
+  std::vector<uint32_t> rkeys(P);
+  for (int p = 0; p < P; ++p) rkeys[p] = bswap32(0x1000u + p);
+  RT_HIP(hipMalloc(reinterpret_cast<void **>(&rkeys_dev_), sizeof(uint32_t) * P));
+  RT_HIP(hipMemcpy(rkeys_dev_, rkeys.data(), sizeof(uint32_t) * P, hipMemcpyHostToDevice));
+
+  ctx_images_.resize(rings);
+  for (int p = 0; p < P; ++p) {
+    for (int b = 0; b < B; ++b) {
+      const size_t r = static_cast<size_t>(p) * B + b;
+      detail::DeviceCtx &c = ctx_images_[r];
+      c.my_pe = p;
+      c.num_pes = P;
+      c.block_id = b;
+      c.options = 0;
+      char *base = queue_mem_ + ring_bytes * r;
+      c.ring.sq = reinterpret_cast<uint64_t *>(base);
+      c.ring.mailbox = reinterpret_cast<uint64_t *>(base + static_cast<size_t>(opt_.sq_size) * 64);
+      c.ring.atomic_ret_base =
+          reinterpret_cast<uint64_t>(base + static_cast<size_t>(opt_.sq_size) * 64 + 64);
+      c.ring.rkey_by_pe = rkeys_dev_;
+      c.ring.ctrl_sig = 0;
+      // Queue-pair number 0x000100 + ring index, laid out as the three
+      // big-endian bytes that follow the opcode word of a WQE.
+      c.ring.ctrl_qp_sq = bswap32((0x000100u + static_cast<uint32_t>(r)) << 8) & 0xffffffu;
+      c.ring.lkey = bswap32(0x2000u);
+      c.ring.atomic_lkey = bswap32(0x3000u);
+      c.ring.max_nwqe = opt_.sq_size;
+      c.counters = counters_dev_ + r;
+    }
+  }
+  RT_HIP(hipMalloc(reinterpret_cast<void **>(&ctx_table_dev_), sizeof(detail::DeviceCtx) * rings));
+  RT_HIP(hipMemcpy(ctx_table_dev_, ctx_images_.data(), sizeof(detail::DeviceCtx) * rings,
+                   hipMemcpyHostToDevice));
+
+  RT_HIP(hipMalloc(reinterpret_cast<void **>(&status_dev_), 64));
+  RT_HIP(hipMemset(status_dev_, 0, 64));
+
+  RT_HIP(hipMalloc(reinterpret_cast<void **>(&teams_dev_), sizeof(detail::Team) * kMaxTeams));
+  RT_HIP(hipMemset(teams_dev_, 0, sizeof(detail::Team) * kMaxTeams));
+  for (int i = kMaxTeams - 1; i >= 0; --i) free_team_slots_.push_back(i);
+
+  detail::TeamInfo world_info{0, 1, 0, P};
+  world_ = make_team(world_info);
+  if (!world_) return "could not allocate the world team's pSync pools";
+
+  state_.heap_base0 = arena_;
+  state_.slice_stride = stride_;
+  state_.heap_size = opt_.heap_size;
+  state_.num_pes = P;
+  state_.num_blocks = B;
+  state_.ctx_table = ctx_table_dev_;
+  state_.base_heap = base_heap_dev_;
+  state_.team_world = world_->device;
+  state_.status = status_dev_;
+  state_.wait_limit_ticks = static_cast<uint64_t>(opt_.wait_limit_s * 100e6);  // 100 MHz clock
+  upload_state_everywhere(state_);
+  RT_HIP(hipDeviceSynchronize());
+  return "";
+}
+
+void Runtime::teardown() {
+  (void)hipDeviceSynchronize();
+  if (teams_dev_) (void)hipFree(teams_dev_);
+  if (status_dev_) (void)hipFree(status_dev_);
+  if (ctx_table_dev_) (void)hipFree(ctx_table_dev_);
+  if (rkeys_dev_) (void)hipFree(rkeys_dev_);
+  if (counters_dev_) (void)hipFree(counters_dev_);
+  if (queue_mem_) (void)hipFree(queue_mem_);
+  if (base_heap_dev_) (void)hipFree(base_heap_dev_);
+  if (arena_) (void)hipFree(arena_);
+  teams_dev_ = nullptr;
+  status_dev_ = nullptr;
+  ctx_table_dev_ = nullptr;
+  rkeys_dev_ = nullptr;
+  counters_dev_ = nullptr;
+  queue_mem_ = nullptr;
+  base_heap_dev_ = nullptr;
+  arena_ = nullptr;
+  teams_.clear();
+  world_ = nullptr;
+  detail::DeviceState cleared{};
+  upload_state_everywhere(cleared);
+}
+
+bool Runtime::owns(const void *p) const {
+  const char *c = static_cast<const char *>(p);
+  return c >= arena_ && c < arena_ + stride_ * static_cast<size_t>(opt_.num_pes);
+}
+
+int Runtime::pe_of(const void *p) const {
+  if (!owns(p)) return -1;
+  return static_cast<int>((static_cast<const char *>(p) - arena_) / stride_);
+}
+
+void *Runtime::sym_malloc(size_t bytes) {
+  size_t off = alloc_.alloc(bytes);
+  if (off == Pow2Allocator::kNoOffset) return nullptr;
+  return slice_base(current_pe_) + off;
+}
+
+bool Runtime::sym_free(void *ptr) {
+  if (!ptr || !owns(ptr)) return false;
+  size_t off = (static_cast<char *>(ptr) - arena_) % stride_;
+  return alloc_.free(off);
+}
+
+void *Runtime::translate(const void *ptr, int pe) const {
+  if (!owns(ptr) || pe < 0 || pe >= opt_.num_pes) return nullptr;
+  size_t off = (static_cast<const char *>(ptr) - arena_) % stride_;
+  return slice_base(pe) + off;
+}
+
+TeamRecord *Runtime::make_team(const detail::TeamInfo &info) {
+  if (free_team_slots_.empty()) return nullptr;
+  // Four pSync pools, one kSyncSlots-long slice per context block each
+  // (reference: per-team pool slices, gpu_ib_team.cpp:30-52, backend_ib.cpp:335-381).
+  const size_t pool_bytes = static_cast<size_t>(opt_.num_blocks) * detail::kSyncSlots * sizeof(long);
+  size_t off = alloc_.alloc(4 * pool_bytes);
+  if (off == Pow2Allocator::kNoOffset) return nullptr;
+  for (int p = 0; p < opt_.num_pes; ++p) {
+    if (hipMemset(slice_base(p) + off, 0, 4 * pool_bytes) != hipSuccess) return nullptr;
+  }
+  int slot = free_team_slots_.back();
+  free_team_slots_.pop_back();
+  TeamRecord rec;
+  rec.image.wrt_world = info;
+  rec.image.valid = 1;
+  rec.image.pad_ = 0;
+  rec.image.barrier_psync_off = off;
+  rec.image.reduce_psync_off = off + pool_bytes;
+  rec.image.bcast_psync_off = off + 2 * pool_bytes;
+  rec.image.alltoall_psync_off = off + 3 * pool_bytes;
+  rec.device = teams_dev_ + slot;
+  rec.pool_offset = off;
+  if (hipMemcpy(rec.device, &rec.image, sizeof(detail::Team), hipMemcpyHostToDevice) !=
+      hipSuccess)
+    return nullptr;
+  auto ins = teams_.emplace(rec.device, rec);
+  return &ins.first->second;
+}
+
+int Runtime::team_split(detail::Team *parent, int start, int stride, int size,
+                        detail::Team **out) {
+  *out = nullptr;
+  if (!parent) return 0;  // reference: splitting an invalid team yields an invalid team, returns 0
+  const TeamRecord *prec = team_record(parent);
+  if (!prec) return -1;
+  const detail::TeamInfo &pi = prec->image.wrt_world;
+  // reference: sanity checks of roc_shmem_team_split_strided, roc_shmem.cpp:237-252
+  if (start < 0 || start >= pi.size || size < 1 || size > pi.size || stride < 1) return -1;
+  int start_world = pi.pe_start + pi.stride * start;
+  int stride_world = stride * pi.stride;
+  int end_world = start_world + stride_world * (size - 1);
+  if (end_world >= opt_.num_pes) return -1;
+  if (stride_world & (stride_world - 1)) return -1;  // collectives address members by log2 stride
+  int log_stride = 0;
+  while ((1 << log_stride) < stride_world) ++log_stride;
+  if (static_cast<int>(teams_.size()) >= kMaxTeams - 1) {
+    fprintf(stderr, "rocshmem: too many teams (limit %d)\n", kMaxTeams);
+    abort();  // reference: roc_shmem.cpp:224-228
+  }
+  detail::TeamInfo info{start_world, stride_world, log_stride, size};
+  TeamRecord *rec = make_team(info);
+  if (!rec) return -1;
+  *out = rec->device;
+  return 0;
+}
+
+void Runtime::team_destroy(detail::Team *team) {
+  auto it = teams_.find(team);
+  if (it == teams_.end() || &it->second == world_) return;
+  alloc_.free(it->second.pool_offset);
+  free_team_slots_.push_back(static_cast<int>(it->second.device - teams_dev_));
+  teams_.erase(it);
+}
+
+const TeamRecord *Runtime::team_record(const detail::Team *team) const {
+  auto it = teams_.find(team);
+  return it == teams_.end() ? nullptr : &it->second;
+}
+
+void Runtime::reset_queues(hipStream_t stream) {
+  (void)hipMemsetAsync(queue_mem_, 0, queue_mem_bytes_, stream);
+  (void)hipMemsetAsync(counters_dev_, 0,
+                       sizeof(detail::SqCounters) * static_cast<size_t>(opt_.num_pes) *
+                           opt_.num_blocks,
+                       stream);
+}
+
+uint32_t Runtime::take_status() {
+  uint32_t v = 0;
+  (void)hipDeviceSynchronize();
+  (void)hipMemcpy(&v, status_dev_, sizeof(v), hipMemcpyDeviceToHost);
+  if (v) (void)hipMemset(status_dev_, 0, sizeof(v));
+  return v;
+}
+
+// ---------------------------------------------------------------------------
+// State upload registry
+// ---------------------------------------------------------------------------
+
+typedef void (*UploadFn)(const detail::DeviceState *);
+static std::vector<UploadFn> &registry() {
+  static std::vector<UploadFn> fns;
+  return fns;
+}
+
+void upload_state_everywhere(const detail::DeviceState &state) {
+  for (UploadFn fn : registry()) fn(&state);
+}
+
+}  // namespace host
+
+namespace detail {
+typedef void (*StateUploadFn)(const DeviceState *);
+void register_state_upload(StateUploadFn fn) { host::registry().push_back(fn); }
+}  // namespace detail
+
+}  // namespace rocshmem

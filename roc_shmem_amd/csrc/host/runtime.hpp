@@ -1,0 +1,141 @@
+// Host-side runtime of the MI355X data path: the HBM arena that holds every
+// PE's symmetric-heap slice, the symmetric allocator, context and send-queue
+// tables, and teams.  Plain C++ over the HIP runtime, nothing else.
+#ifndef ROCSHMEM_MI355X_HOST_RUNTIME_HPP
+#define ROCSHMEM_MI355X_HOST_RUNTIME_HPP
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "rocshmem_device/state.hpp"
+
+namespace rocshmem {
+namespace host {
+
+// Symmetric-heap allocator handing out slice-relative offsets.  Observable
+// behaviour follows the reference's Pow2Bins strategy
+// (library/src/memory/pow2_bins.hpp:90-125,264-287, binner.hpp:109-134):
+// requests round up to a power of two with a 128-byte floor; an empty bin is
+// refilled by halving a block of the next non-empty larger bin, lower half
+// handed out first; freed blocks go back on top of their bin and are never
+// merged; a zero-byte request yields nothing.
+class Pow2Allocator {
+ public:
+  static constexpr size_t kMinBlock = 128;  // reference: ALIGNMENT, constants.hpp:39
+  static constexpr size_t kNoOffset = ~size_t(0);
+
+  Pow2Allocator() = default;
+  explicit Pow2Allocator(size_t heap_bytes);
+
+  size_t alloc(size_t request);  // kNoOffset when nothing fits (or request == 0)
+  bool free(size_t offset);      // false when `offset` is not an outstanding allocation
+  size_t bytes_in_use() const;
+  size_t heap_bytes() const { return heap_bytes_; }
+
+ private:
+  bool refill(std::map<size_t, std::vector<size_t>>::iterator it);
+  size_t heap_bytes_ = 0;
+  std::map<size_t, std::vector<size_t>> bins_;  // block size -> LIFO stack of offsets
+  std::map<size_t, size_t> outstanding_;        // offset -> block size
+};
+
+struct Options {
+  int num_pes = 8;                 // ROC_SHMEM_NUM_PES
+  size_t heap_size = 1ull << 30;   // ROC_SHMEM_HEAP_SIZE, per PE (reference: heap_memory.hpp:114)
+  int num_blocks = 64;             // ROC_SHMEM_NUM_BLOCKS, contexts per PE
+  uint32_t sq_size = 1024;         // ROC_SHMEM_SQ_SIZE (reference: connection.hpp:225)
+  size_t slice_pad = 0;            // ROC_SHMEM_SLICE_PAD, extra bytes between slices
+  double wait_limit_s = 2.0;       // ROC_SHMEM_WAIT_LIMIT_S, bound of a device flag wait
+  static Options from_env();
+};
+
+struct TeamRecord {
+  detail::Team image;      // host copy of the device object
+  detail::Team *device;    // the handle a roc_shmem_team_t points at
+  size_t pool_offset;      // symmetric offset of the pSync pools
+};
+
+class Runtime {
+ public:
+  // Returns an empty string on success, an error message otherwise.
+  static std::string create(const Options &opt);
+  static void destroy();
+  static Runtime *get() { return instance_; }
+
+  const Options &options() const { return opt_; }
+  int num_pes() const { return opt_.num_pes; }
+  size_t slice_stride() const { return stride_; }
+  char *slice_base(int pe) const { return arena_ + stride_ * static_cast<size_t>(pe); }
+  bool owns(const void *p) const;
+  int pe_of(const void *p) const;
+
+  int current_pe() const { return current_pe_; }
+  void set_current_pe(int pe) { current_pe_ = pe; }
+
+  void *sym_malloc(size_t bytes);   // address in the current PE's slice, nullptr on failure
+  bool sym_free(void *ptr);
+  void *translate(const void *ptr, int pe) const;
+  size_t bytes_in_use() const { return alloc_.bytes_in_use(); }
+
+  detail::Team *team_world() const { return world_->device; }
+  // 0 on success (handle in *out, nullptr if arguments describe no team), -1 on bad arguments.
+  int team_split(detail::Team *parent, int start, int stride, int size, detail::Team **out);
+  void team_destroy(detail::Team *team);
+  const TeamRecord *team_record(const detail::Team *team) const;
+  int live_teams() const { return static_cast<int>(teams_.size()); }
+
+  detail::DeviceCtx *ctx_device(int pe, int block) const {
+    return ctx_table_dev_ + static_cast<size_t>(pe) * opt_.num_blocks + block;
+  }
+  const detail::DeviceCtx &ctx_image(int pe, int block) const {
+    return ctx_images_[static_cast<size_t>(pe) * opt_.num_blocks + block];
+  }
+  // Zero every ring, mailbox and producer index.
+  void reset_queues(hipStream_t stream);
+
+  // Reads and clears the sticky device status word.
+  uint32_t take_status();
+
+  static constexpr int kMaxTeams = 40;  // reference: team_tracker.hpp:125
+
+ private:
+  Runtime() = default;
+  std::string init(const Options &opt);
+  void teardown();
+  TeamRecord *make_team(const detail::TeamInfo &info);
+
+  static Runtime *instance_;
+  Options opt_;
+  size_t stride_ = 0;
+  char *arena_ = nullptr;
+  Pow2Allocator alloc_;
+  int current_pe_ = 0;
+
+  char **base_heap_dev_ = nullptr;
+  detail::DeviceCtx *ctx_table_dev_ = nullptr;
+  std::vector<detail::DeviceCtx> ctx_images_;
+  char *queue_mem_ = nullptr;   // rings + mailboxes + atomic-return windows
+  size_t queue_mem_bytes_ = 0;
+  detail::SqCounters *counters_dev_ = nullptr;
+  uint32_t *rkeys_dev_ = nullptr;
+  uint32_t *status_dev_ = nullptr;
+  detail::Team *teams_dev_ = nullptr;   // kMaxTeams objects
+  std::vector<int> free_team_slots_;
+  std::map<const detail::Team *, TeamRecord> teams_;
+  TeamRecord *world_ = nullptr;
+  detail::DeviceState state_{};
+};
+
+// Every translation unit that contains kernels registers a function that
+// copies the device state into its own __constant__ instance.
+void upload_state_everywhere(const detail::DeviceState &state);
+
+}  // namespace host
+}  // namespace rocshmem
+
+#endif

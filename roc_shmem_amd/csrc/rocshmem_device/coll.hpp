@@ -1,0 +1,201 @@
+// Workgroup-collective data movement between the slices of an active set:
+// broadcast, alltoall, fcollect, and the barrier/sync family.
+//
+// Each collective is entered by one workgroup per member PE with identical
+// arguments (reference: GPUIBContext::broadcast / alltoall_broadcast /
+// fcollect_broadcast, library/src/gpu_ib/context_ib_tmpl_device.hpp:455-558,
+// 845-876; internal_sync, context_ib_device_coll.cpp:30-89).  Because every
+// slice is addressable, the work of one call is split over its member
+// workgroups by byte range rather than by peer: member k moves the k-th share
+// of the payload for all peers, reading each source byte once.  Every call is
+// bracketed by two flag barriers on distinct halves of the pSync slice, which
+// also makes back-to-back calls on the same pSync safe.
+//
+// A `shard`/`nshards` pair restricts a call to one equal part of every block,
+// so that several workgroups of a PE (each with its own pSync slice) can
+// share one large collective.
+#ifndef ROCSHMEM_MI355X_DEVICE_COLL_HPP
+#define ROCSHMEM_MI355X_DEVICE_COLL_HPP
+
+#include "copy.hpp"
+#include "reduce.hpp"
+#include "sync.hpp"
+
+namespace rocshmem {
+namespace detail {
+
+// Split [0, n) into `parts` contiguous shares whose interior boundaries are
+// multiples of `quantum`; returns share `idx`.
+__device__ __forceinline__ void split_range(size_t n, int parts, int idx, size_t quantum,
+                                            size_t &begin, size_t &end) {
+  size_t share = (n + parts - 1) / parts;
+  share = (share + quantum - 1) / quantum * quantum;
+  begin = share * static_cast<size_t>(idx);
+  end = begin + share;
+  if (begin > n) begin = n;
+  if (end > n) end = n;
+}
+
+// Copy `n` bytes from `src` into the same symmetric address `dst_mine` of
+// every member for which `skip_idx != member index`, loading each source
+// vector once when all addresses are mutually 16-byte aligned.
+__device__ __forceinline__ void wg_copy_to_members(char *dst_mine, const char *src, size_t n,
+                                                   const ActiveSet &as, int my_pe, int skip_idx,
+                                                   uint32_t tid, uint32_t nthr) {
+  if (n == 0) return;
+  const int64_t stride = static_cast<int64_t>(g_state.slice_stride);
+  char *dst0 = dst_mine + (static_cast<int64_t>(as.pe_start) - my_pe) * stride;
+  const int64_t member_step = stride << as.log_stride;
+  const bool coaligned =
+      ((reinterpret_cast<uintptr_t>(dst_mine) ^ reinterpret_cast<uintptr_t>(src)) & 15u) == 0;
+  if (!coaligned || n < 256) {
+    for (int m = 0; m < as.size; ++m) {
+      if (m == skip_idx) continue;
+      group_copy(dst0 + m * member_step, src, n, tid, nthr);
+    }
+    return;
+  }
+  size_t head = (16u - (reinterpret_cast<uintptr_t>(src) & 15u)) & 15u;
+  size_t nvec = (n - head) / 16;
+  size_t tail = n - head - nvec * 16;
+  if (tid < head) {
+    char b = src[tid];
+    for (int m = 0; m < as.size; ++m)
+      if (m != skip_idx) dst0[m * member_step + tid] = b;
+  }
+  if (tid < tail) {
+    size_t off = head + nvec * 16 + tid;
+    char b = src[off];
+    for (int m = 0; m < as.size; ++m)
+      if (m != skip_idx) dst0[m * member_step + off] = b;
+  }
+  const u32x4 *sv = reinterpret_cast<const u32x4 *>(src + head);
+  char *dv0 = dst0 + head;
+  constexpr int U = kCopyUnroll;
+  size_t i = tid;
+  const size_t step = nthr;
+  for (; i + (U - 1) * step < nvec; i += U * step) {
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(&sv[i + u * step]);
+    for (int m = 0; m < as.size; ++m) {
+      if (m == skip_idx) continue;
+      u32x4 *d = reinterpret_cast<u32x4 *>(dv0 + m * member_step);
+#pragma unroll
+      for (int u = 0; u < U; ++u) __builtin_nontemporal_store(v[u], &d[i + u * step]);
+    }
+  }
+  for (; i < nvec; i += step) {
+    u32x4 v = __builtin_nontemporal_load(&sv[i]);
+    for (int m = 0; m < as.size; ++m) {
+      if (m == skip_idx) continue;
+      __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dv0 + m * member_step) + i);
+    }
+  }
+}
+
+// Broadcast `nbytes` from the root member's `source` to every other member's
+// `dest`; the root's `dest` is not written (reference: internal_put_broadcast
+// / internal_get_broadcast, context_ib_tmpl_device.hpp:455-478).  `root_idx`
+// is the root's ordinal within the active set.
+__device__ __forceinline__ void wg_broadcast_bytes(int my_pe, void *dest, const void *source,
+                                                   size_t nbytes, int root_idx, int pe_start,
+                                                   int log_stride, int pe_size, long *psync) {
+  if (nbytes == 0) return;
+  if (pe_size > kMaxPes || pe_size <= 0 || root_idx < 0 || root_idx >= pe_size) {
+    status_raise(kStatusBadArgument);
+    return;
+  }
+  const ActiveSet as{pe_start, log_stride, pe_size};
+  const int my_idx = (my_pe - pe_start) >> log_stride;
+  const uint32_t tid = flat_thread_id();
+  const uint32_t nthr = flat_block_size();
+
+  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, log_stride, pe_size);
+
+  size_t b, e;
+  split_range(nbytes, pe_size, my_idx, 256, b, e);
+  const char *root_src = translate(static_cast<const char *>(source), my_pe, as.pe_at(root_idx));
+  wg_copy_to_members(static_cast<char *>(dest) + b, root_src + b, e - b, as, my_pe, root_idx,
+                     tid, nthr);
+
+  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, log_stride, pe_size);
+}
+
+// Alltoall block exchange: member i's block j goes to member j's block i,
+// self block included (reference: alltoall_broadcast,
+// context_ib_tmpl_device.hpp:528-558).  `block_bytes` is the size of one
+// block; only bytes [shard_begin, shard_end) of every block are moved.
+__device__ __forceinline__ void wg_alltoall_bytes(int my_pe, void *dest, const void *source,
+                                                  size_t block_bytes, size_t shard_begin,
+                                                  size_t shard_end, int pe_start, int log_stride,
+                                                  int pe_size, long *psync) {
+  if (block_bytes == 0) return;
+  if (pe_size > kMaxPes || pe_size <= 0) {
+    status_raise(kStatusBadArgument);
+    return;
+  }
+  const ActiveSet as{pe_start, log_stride, pe_size};
+  const int my_idx = (my_pe - pe_start) >> log_stride;
+  const uint32_t tid = flat_thread_id();
+  const uint32_t nthr = flat_block_size();
+
+  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, log_stride, pe_size);
+
+  const size_t len = shard_end - shard_begin;
+  char *dst_mine = static_cast<char *>(dest) + static_cast<size_t>(my_idx) * block_bytes +
+                   shard_begin;
+  const char *src = static_cast<const char *>(source) + shard_begin;
+  for (int jj = 0; jj < pe_size; ++jj) {
+    // Start at the own index so that concurrent members hit different slices.
+    int j = my_idx + jj;
+    if (j >= pe_size) j -= pe_size;
+    group_copy(translate(dst_mine, my_pe, as.pe_at(j)), src + static_cast<size_t>(j) * block_bytes,
+               len, tid, nthr);
+  }
+
+  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, log_stride, pe_size);
+}
+
+// Fcollect: member i's `block_bytes` land in block i of every member's dest
+// (reference: fcollect_broadcast, context_ib_tmpl_device.hpp:845-876).
+__device__ __forceinline__ void wg_fcollect_bytes(int my_pe, void *dest, const void *source,
+                                                  size_t block_bytes, size_t shard_begin,
+                                                  size_t shard_end, int pe_start, int log_stride,
+                                                  int pe_size, long *psync) {
+  if (block_bytes == 0) return;
+  if (pe_size > kMaxPes || pe_size <= 0) {
+    status_raise(kStatusBadArgument);
+    return;
+  }
+  const ActiveSet as{pe_start, log_stride, pe_size};
+  const int my_idx = (my_pe - pe_start) >> log_stride;
+
+  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, log_stride, pe_size);
+
+  char *dst_mine = static_cast<char *>(dest) + static_cast<size_t>(my_idx) * block_bytes +
+                   shard_begin;
+  wg_copy_to_members(dst_mine, static_cast<const char *>(source) + shard_begin,
+                     shard_end - shard_begin, as, my_pe, -1, flat_thread_id(),
+                     flat_block_size());
+
+  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, log_stride, pe_size);
+}
+
+// Barrier among the member workgroups (reference: internal_sync,
+// context_ib_device_coll.cpp:67-89).
+__device__ __forceinline__ void wg_sync_members(int my_pe, int pe_start, int log_stride,
+                                                int pe_size, long *psync) {
+  if (pe_size > kMaxPes || pe_size <= 0) {
+    status_raise(kStatusBadArgument);
+    return;
+  }
+  const int my_idx = (my_pe - pe_start) >> log_stride;
+  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, log_stride, pe_size);
+  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, log_stride, pe_size);
+}
+
+}  // namespace detail
+}  // namespace rocshmem
+
+#endif

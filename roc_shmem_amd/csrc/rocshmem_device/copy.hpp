@@ -1,0 +1,162 @@
+// HBM-to-HBM byte copy shared by put/get/broadcast/alltoall at workgroup,
+// wavefront and single-lane granularity.
+//
+// The reference moves 8 bytes per lane per step through uncached stores
+// (memcpy_wg / memcpy_wave / memcpy, library/src/util.hpp:248-325).  Here a
+// group of `nthr` lanes moves 16 bytes per lane per access, four accesses in
+// flight per lane: destination-aligned global_store_dwordx4, sources read as
+// dwordx4 at whatever 4-byte alignment they have, and byte-misaligned
+// sources re-aligned in registers with v_alignbyte_b32.  Semantics are exactly
+// memcpy(dst, src, n) for non-overlapping ranges.
+#ifndef ROCSHMEM_MI355X_DEVICE_COPY_HPP
+#define ROCSHMEM_MI355X_DEVICE_COPY_HPP
+
+#include "state.hpp"
+#include "wave.hpp"
+
+namespace rocshmem {
+namespace detail {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
+
+constexpr int kCopyUnroll = 4;
+// Copies at least this large bypass cache allocation (nt loads and stores):
+// the payload is touched once and is larger than what the L2 would keep.
+constexpr size_t kNonTemporalBytes = 256 * 1024;
+
+template <bool kNt>
+__device__ __forceinline__ u32x4 load_vec(const u32x4 *p) {
+  if constexpr (kNt) return __builtin_nontemporal_load(p);
+  return *p;
+}
+template <bool kNt>
+__device__ __forceinline__ void store_vec(u32x4 v, u32x4 *p) {
+  if constexpr (kNt) {
+    __builtin_nontemporal_store(v, p);
+  } else {
+    *p = v;
+  }
+}
+
+// dst and src both 16-byte aligned.
+template <bool kNt>
+__device__ __forceinline__ void copy_vec_aligned(u32x4 *__restrict__ d,
+                                                 const u32x4 *__restrict__ s, size_t nvec,
+                                                 uint32_t tid, uint32_t nthr) {
+  size_t i = tid;
+  const size_t step = nthr;
+  for (; i + (kCopyUnroll - 1) * step < nvec; i += kCopyUnroll * step) {
+    u32x4 v[kCopyUnroll];
+#pragma unroll
+    for (int k = 0; k < kCopyUnroll; ++k) v[k] = load_vec<kNt>(&s[i + k * step]);
+#pragma unroll
+    for (int k = 0; k < kCopyUnroll; ++k) store_vec<kNt>(v[k], &d[i + k * step]);
+  }
+  for (; i < nvec; i += step) store_vec<kNt>(load_vec<kNt>(&s[i]), &d[i]);
+}
+
+// dst 16-byte aligned, src 4-byte aligned.
+__device__ __forceinline__ void copy_vec_src_dword(u32x4 *__restrict__ d,
+                                                   const char *__restrict__ s, size_t nvec,
+                                                   uint32_t tid, uint32_t nthr) {
+  const u32x4_a4 *sv = reinterpret_cast<const u32x4_a4 *>(s);
+  size_t i = tid;
+  const size_t step = nthr;
+  for (; i + (kCopyUnroll - 1) * step < nvec; i += kCopyUnroll * step) {
+    u32x4 v[kCopyUnroll];
+#pragma unroll
+    for (int k = 0; k < kCopyUnroll; ++k) v[k] = sv[i + k * step];
+#pragma unroll
+    for (int k = 0; k < kCopyUnroll; ++k) d[i + k * step] = v[k];
+  }
+  for (; i < nvec; i += step) d[i] = sv[i];
+}
+
+// dst 16-byte aligned, src at byte offset `shift` (1..3) past a 4-byte
+// boundary.  Each lane reads the five aligned dwords that cover its 16
+// destination bytes and funnels them together.  The caller guarantees that
+// the dword holding the last source byte of every vector lies inside the
+// source range's enclosing aligned dwords (true for any in-bounds source:
+// the fifth dword always contains at least one requested byte).
+__device__ __forceinline__ void copy_vec_src_bytes(u32x4 *__restrict__ d,
+                                                   const char *__restrict__ s, size_t nvec,
+                                                   uint32_t tid, uint32_t nthr) {
+  const uint32_t shift = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(s) & 3u);
+  const uint32_t *sw = reinterpret_cast<const uint32_t *>(s - shift);
+  for (size_t i = tid; i < nvec; i += nthr) {
+    const u32x4_a4 *lo = reinterpret_cast<const u32x4_a4 *>(sw + 4 * i);
+    u32x4 w = *lo;
+    uint32_t w4 = sw[4 * i + 4];
+    u32x4 o;
+    o.x = __builtin_amdgcn_alignbyte(w.y, w.x, shift);
+    o.y = __builtin_amdgcn_alignbyte(w.z, w.y, shift);
+    o.z = __builtin_amdgcn_alignbyte(w.w, w.z, shift);
+    o.w = __builtin_amdgcn_alignbyte(w4, w.w, shift);
+    d[i] = o;
+  }
+}
+
+// memcpy(dst, src, n) executed cooperatively by lanes tid = 0..nthr-1.
+// No barrier inside: the caller synchronises the group afterwards.
+__device__ __forceinline__ void group_copy(void *dst, const void *src, size_t n, uint32_t tid,
+                                           uint32_t nthr) {
+  char *d = static_cast<char *>(dst);
+  const char *s = static_cast<const char *>(src);
+  if (n < 64) {
+    for (size_t i = tid; i < n; i += nthr) d[i] = s[i];
+    return;
+  }
+  // Head: bring the destination to a 16-byte boundary.
+  size_t head = (16u - (reinterpret_cast<uintptr_t>(d) & 15u)) & 15u;
+  if (tid < head) d[tid] = s[tid];
+  d += head;
+  s += head;
+  n -= head;
+
+  size_t nvec = n / 16;
+  size_t body = nvec * 16;
+  uintptr_t smis = reinterpret_cast<uintptr_t>(s) & 15u;
+  u32x4 *dv = reinterpret_cast<u32x4 *>(d);
+  if (smis == 0) {
+    if (body >= kNonTemporalBytes) {
+      copy_vec_aligned<true>(dv, reinterpret_cast<const u32x4 *>(s), nvec, tid, nthr);
+    } else {
+      copy_vec_aligned<false>(dv, reinterpret_cast<const u32x4 *>(s), nvec, tid, nthr);
+    }
+  } else if ((smis & 3u) == 0) {
+    copy_vec_src_dword(dv, s, nvec, tid, nthr);
+  } else {
+    copy_vec_src_bytes(dv, s, nvec, tid, nthr);
+  }
+  // Tail: fewer than 16 bytes.
+  size_t tail = n - body;
+  if (tid < tail) d[body + tid] = s[body + tid];
+}
+
+__device__ __forceinline__ void wg_copy(void *dst, const void *src, size_t n) {
+  group_copy(dst, src, n, flat_thread_id(), flat_block_size());
+}
+
+__device__ __forceinline__ void wave_copy(void *dst, const void *src, size_t n) {
+  // All lanes of the calling wave take part (wave-collective call).
+  group_copy(dst, src, n, lane_id(), kWaveSize);
+}
+
+// Single-lane copy used by the thread-level put/get: the common 4- and 8-byte
+// naturally aligned messages are a single store.
+__device__ __forceinline__ void lane_copy(void *dst, const void *src, size_t n) {
+  uintptr_t both = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src);
+  if (n == 8 && (both & 7u) == 0) {
+    *static_cast<uint64_t *>(dst) = *static_cast<const uint64_t *>(src);
+  } else if (n == 4 && (both & 3u) == 0) {
+    *static_cast<uint32_t *>(dst) = *static_cast<const uint32_t *>(src);
+  } else {
+    group_copy(dst, src, n, 0u, 1u);
+  }
+}
+
+}  // namespace detail
+}  // namespace rocshmem
+
+#endif

@@ -1,0 +1,100 @@
+// Device-visible runtime state of the MI355X data path.
+//
+// One process hosts every PE.  PE p owns the symmetric-heap slice
+//   [heap_base0 + p*slice_stride, heap_base0 + p*slice_stride + heap_size)
+// of a single HBM arena, so the reference's address translation
+//   base_heap[pe] + (ptr - base_heap[my_pe])
+// (library/src/gpu_ib/context_ib_device.cpp:86,99,222) becomes one multiply-add.
+#ifndef ROCSHMEM_MI355X_DEVICE_STATE_HPP
+#define ROCSHMEM_MI355X_DEVICE_STATE_HPP
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rocshmem {
+namespace detail {
+
+constexpr int kWaveSize = 64;      // reference: WF_SIZE, library/src/constants.hpp:56
+constexpr int kMaxPes = 128;       // two flag sets of kMaxPes fit ROC_SHMEM_*_SYNC_SIZE (256)
+constexpr int kSyncSlots = 256;    // longs per pSync slice
+constexpr int kAtomicRetSlots = 4096;  // reference: atomic_return.hpp:34-40
+
+// Sticky status codes written to DeviceState::status[0].
+enum : uint32_t {
+  kStatusOk = 0,
+  kStatusWaitTimeout = 1,   // a bounded flag wait gave up
+  kStatusBadArgument = 2,   // e.g. active set larger than kMaxPes
+};
+
+// Active-set description relative to the world (reference: TeamInfo,
+// library/src/team.hpp:38-75; log_stride is kept integral here).
+struct TeamInfo {
+  int pe_start;
+  int stride;
+  int log_stride;
+  int size;
+};
+
+// Device-side team object (reference: GPUIBTeam, library/src/gpu_ib/gpu_ib_team.hpp).
+// The pSync pools are symmetric-heap offsets valid in every slice; each
+// context block owns a private kSyncSlots-long slice of each pool so that
+// several workgroups of one PE can run team collectives concurrently.
+struct Team {
+  TeamInfo wrt_world;
+  int valid;
+  int pad_;
+  uint64_t barrier_psync_off;
+  uint64_t reduce_psync_off;
+  uint64_t bcast_psync_off;
+  uint64_t alltoall_psync_off;
+};
+
+// Send-queue ring of one context (reference: QueuePair, queue_pair.hpp:337-418).
+struct SqRing {
+  uint64_t *sq;             // max_nwqe slots of 8 x u64 (64 B each)
+  uint64_t *mailbox;        // [0] doorbell record (BE32 in the low word), [1] doorbell value
+  const uint32_t *rkey_by_pe;  // remote key per destination PE, stored as the NIC would read it
+  uint64_t atomic_ret_base; // address AMO results would be DMA'd to (never written here)
+  uint64_t ctrl_sig;
+  uint32_t ctrl_qp_sq;
+  uint32_t lkey;
+  uint32_t atomic_lkey;
+  uint32_t max_nwqe;
+};
+
+// Mutable producer indices of a ring, on their own cache line.
+struct alignas(64) SqCounters {
+  uint32_t sq_counter;      // free-running WQE index (reference: queue_pair.hpp:378)
+  uint32_t published;       // every WQE below this index is complete in memory
+  uint32_t atomic_counter;  // free-running AMO return-slot index
+  uint32_t pad_[13];
+};
+
+// One context = one (PE, block) pair (reference: GPUIBContext members,
+// context_ib_device.hpp:278-299, minus all NIC state).
+struct DeviceCtx {
+  int my_pe;
+  int num_pes;
+  int block_id;
+  int options;
+  SqRing ring;
+  SqCounters *counters;
+};
+
+struct DeviceState {
+  char *heap_base0;
+  uint64_t slice_stride;
+  uint64_t heap_size;
+  int num_pes;
+  int num_blocks;
+  DeviceCtx *ctx_table;        // [num_pes * num_blocks]
+  char *const *base_heap;      // slice base per PE (reference: base_heap[])
+  Team *team_world;
+  uint32_t *status;
+  uint64_t wait_limit_ticks;   // wall_clock64() ticks a flag wait may take
+};
+
+}  // namespace detail
+}  // namespace rocshmem
+
+#endif

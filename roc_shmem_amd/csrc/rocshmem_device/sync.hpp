@@ -1,0 +1,130 @@
+// Agent-scope synchronisation between the workgroups that stand for the PEs
+// of one collective: bounded flag waits and an all-to-all flag barrier on
+// the caller's (or the team's) pSync array.
+//
+// Every wait is bounded by DeviceState::wait_limit_ticks of the 100 MHz
+// constant clock; a wait that gives up records kStatusWaitTimeout in the
+// sticky status word, after which every later wait returns at once, so a
+// mis-launched grid drains instead of hanging the device.
+#ifndef ROCSHMEM_MI355X_DEVICE_SYNC_HPP
+#define ROCSHMEM_MI355X_DEVICE_SYNC_HPP
+
+#include "state.hpp"
+#include "wave.hpp"
+
+namespace rocshmem {
+namespace detail {
+
+// Per translation unit copy of the runtime state; the host library uploads it
+// into every registered translation unit during roc_shmem_init().
+static __constant__ DeviceState g_state;
+
+__device__ __forceinline__ void fence_release_agent() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+}
+__device__ __forceinline__ void fence_acquire_agent() {
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+}
+__device__ __forceinline__ void fence_acq_rel_agent() {
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "agent");
+}
+
+__device__ __forceinline__ bool status_failed() {
+  return __hip_atomic_load(g_state.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) !=
+         kStatusOk;
+}
+
+__device__ __forceinline__ void status_raise(uint32_t code) {
+  uint32_t expected = kStatusOk;
+  __hip_atomic_compare_exchange_strong(g_state.status, &expected, code, __ATOMIC_RELAXED,
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Translate a symmetric address of PE `from_pe` into the slice of PE `to_pe`.
+template <typename T>
+__device__ __forceinline__ T *translate(T *ptr, int from_pe, int to_pe) {
+  int64_t delta = (static_cast<int64_t>(to_pe) - from_pe) *
+                  static_cast<int64_t>(g_state.slice_stride);
+  return reinterpret_cast<T *>(
+      reinterpret_cast<uintptr_t>(ptr) + static_cast<uintptr_t>(delta));
+}
+
+enum WaitCmp { kWaitEq, kWaitNe, kWaitGt, kWaitGe, kWaitLt, kWaitLe };
+
+template <typename T>
+__device__ __forceinline__ bool compare_for_wait(T have, int cmp, T want) {
+  switch (cmp) {
+    case kWaitEq: return have == want;
+    case kWaitNe: return have != want;
+    case kWaitGt: return have > want;
+    case kWaitGe: return have >= want;
+    case kWaitLt: return have < want;
+    default: return have <= want;
+  }
+}
+
+// Spin until `*ptr cmp want` holds, reading through agent-scope atomic loads
+// (the reference polls with uncached loads, context_tmpl_device.hpp:199-246).
+// Returns false on timeout or when the status word is already raised.
+template <typename T>
+__device__ __forceinline__ bool bounded_wait(const T *ptr, int cmp, T want) {
+  using Word = typename std::conditional<sizeof(T) == 8, uint64_t, uint32_t>::type;
+  static_assert(sizeof(T) == 4 || sizeof(T) == 8, "wait on 4- or 8-byte words");
+  const Word *wptr = reinterpret_cast<const Word *>(ptr);
+  uint64_t start = wall_clock64();
+  uint32_t spins = 0;
+  for (;;) {
+    Word raw = __hip_atomic_load(wptr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    T have;
+    __builtin_memcpy(&have, &raw, sizeof(T));
+    if (compare_for_wait(have, cmp, want)) return true;
+    __builtin_amdgcn_s_sleep(1);
+    if ((++spins & 63u) == 0) {
+      if (status_failed()) return false;
+      if (wall_clock64() - start > g_state.wait_limit_ticks) {
+        status_raise(kStatusWaitTimeout);
+        return false;
+      }
+    }
+  }
+}
+
+// All-to-all flag barrier among the `n_pes` workgroups (one per PE of the
+// active set) that share one collective call.  `psync` is this PE's copy of
+// the symmetric pSync slice, `set` selects slots [set*n_pes, (set+1)*n_pes).
+//
+// Arrival: thread t < n_pes publishes everything this workgroup wrote and
+// sets slot `my_idx` in the copy owned by member t.  Completion: thread t
+// waits for slot t of the own copy, then clears it, so the array is all
+// ROC_SHMEM_SYNC_VALUE again on return (the reference restores it the same
+// way, context_ib_tmpl_device.hpp:178-180,231-233).  Two consecutive barriers
+// must use different sets; the same set may be reused once a barrier on the
+// other set has completed in between.
+//
+// Must be called by every thread of the workgroup.
+__device__ __forceinline__ void wg_flag_barrier(long *psync, int set, int my_pe, int my_idx,
+                                                int pe_start, int log_stride, int n_pes) {
+  __syncthreads();
+  const uint32_t tid = flat_thread_id();
+  const uint32_t nthr = flat_block_size();
+  if (tid < static_cast<uint32_t>(n_pes)) fence_release_agent();
+  for (uint32_t t = tid; t < static_cast<uint32_t>(n_pes); t += nthr) {
+    int peer = pe_start + (static_cast<int>(t) << log_stride);
+    unsigned long long *slot = reinterpret_cast<unsigned long long *>(
+        translate(psync, my_pe, peer) + set * n_pes + my_idx);
+    __hip_atomic_store(slot, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  for (uint32_t t = tid; t < static_cast<uint32_t>(n_pes); t += nthr) {
+    unsigned long long *mine =
+        reinterpret_cast<unsigned long long *>(psync + set * n_pes + static_cast<int>(t));
+    bounded_wait<unsigned long long>(mine, kWaitEq, 1ull);
+    __hip_atomic_store(mine, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  fence_acquire_agent();
+}
+
+}  // namespace detail
+}  // namespace rocshmem
+
+#endif

@@ -1,0 +1,174 @@
+// GPU-built 64-byte work-queue entries in a send-queue ring.
+//
+// Byte layout, opcodes and field encodings follow what the reference writes
+// for the RC transport: SegmentBuilder (library/src/gpu_ib/segment_builder.cpp:
+// 29-128), QueuePair::update_posted_wqe_generic (queue_pair.cpp:205-273), the
+// completion flag and doorbell of the multi-thread post policy
+// (thread_policy.cpp:170-216, queue_pair.cpp:67-78) and the byte swaps of
+// endian.cpp:27-77.  A WQE is four 16-byte segments:
+//   0 control   : 00 | idx_hi idx_lo | opcode | qpn[3] | DS | sig | 00 00 | fm_ce_se | imm[4]
+//   1 remote    : BE64 raddr | rkey | 00000000
+//   2 data      : BE32 byte_count | lkey | BE64 laddr          (size > 8, or READ)
+//     inline    : BE32 (size | 0x80000000) | payload[size]      (WRITE, size <= 8)
+//     atomic    : BE64 swap_add | BE64 compare
+//   3 atomic only: BE32 8 | atomic_lkey | BE64 &atomic_ret[pos]
+// Bytes the reference never writes (inline padding, segment 3 of non-atomic
+// entries) are left as the ring holds them.
+//
+// What differs from the reference is how lanes get their slots.  The
+// reference serialises waves with a per-queue spin lock and lets every lane
+// call atomicAdd (thread_policy.cpp:218-323).  Here one wave reserves all the
+// slots its posting lanes need with a single atomic (ballot + v_mbcnt +
+// v_readlane), every posting lane assembles its entry in registers and
+// writes it with 16-byte stores, and completed ranges are published in index
+// order through SqCounters::published before the doorbell record moves.
+#ifndef ROCSHMEM_MI355X_DEVICE_WQE_HPP
+#define ROCSHMEM_MI355X_DEVICE_WQE_HPP
+
+#include "copy.hpp"
+#include "sync.hpp"
+#include "wave.hpp"
+
+namespace rocshmem {
+namespace detail {
+
+constexpr uint8_t kOpcodeRdmaWrite = 0x08;
+constexpr uint8_t kOpcodeRdmaRead = 0x10;
+constexpr uint8_t kOpcodeAtomicCs = 0x11;
+constexpr uint8_t kOpcodeAtomicFa = 0x12;
+constexpr uint32_t kInlineThreshold = 8;  // reference: queue_pair.hpp:324
+constexpr uint8_t kCqUpdate = 8;          // fm_ce_se value that requests a CQE
+
+__device__ __forceinline__ uint32_t be32(uint32_t v) { return __builtin_bswap32(v); }
+
+// A 64-bit value stored big-endian occupies two little-endian 32-bit words:
+// first the swapped high half, then the swapped low half.
+__device__ __forceinline__ uint32_t be64_first(uint64_t v) {
+  return __builtin_bswap32(static_cast<uint32_t>(v >> 32));
+}
+__device__ __forceinline__ uint32_t be64_second(uint64_t v) {
+  return __builtin_bswap32(static_cast<uint32_t>(v));
+}
+
+struct WqeRequest {
+  uint8_t opcode;
+  uint32_t size;         // bytes the entry covers (already merged by the coalescer)
+  uint64_t raddr;        // target address in the destination slice
+  uint64_t laddr;        // local buffer address (ignored for atomics)
+  uint64_t atomic_data;  // add / swap operand
+  uint64_t atomic_cmp;   // compare operand (0 for fetch-add)
+  uint64_t inline_data;  // payload bytes, little-endian packed, when size <= 8 and WRITE
+  int pe;
+};
+
+// Post one entry per lane that passes `sends == true`.  Called by every lane
+// that is active at the call site (senders and absorbed lanes alike).
+__device__ __forceinline__ void wave_post(DeviceCtx *ctx, bool sends, const WqeRequest &rq) {
+  const uint64_t send_mask = __ballot(sends);
+  if (send_mask == 0) return;
+  const uint32_t n = __popcll(send_mask);
+  const uint32_t rank = rank_in_mask(send_mask);
+  const uint32_t first = __builtin_ctzll(send_mask);
+  const bool is_atomic = rq.opcode == kOpcodeAtomicFa || rq.opcode == kOpcodeAtomicCs;
+  const uint64_t atomic_mask = __ballot(sends && is_atomic);
+
+  SqCounters *cnt = ctx->counters;
+  uint32_t base = 0, abase = 0;
+  if (sends && rank == 0) {
+    base = __hip_atomic_fetch_add(&cnt->sq_counter, n, __ATOMIC_RELAXED,
+                                  __HIP_MEMORY_SCOPE_AGENT);
+    if (atomic_mask) {
+      abase = __hip_atomic_fetch_add(&cnt->atomic_counter,
+                                     static_cast<uint32_t>(__popcll(atomic_mask)),
+                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  base = __builtin_amdgcn_readlane(base, first);
+  abase = __builtin_amdgcn_readlane(abase, first);
+
+  const SqRing &ring = ctx->ring;
+  const uint32_t my_counter = base + rank;
+  const bool last = sends && rank == n - 1;
+
+  uint32_t first8_lo = 0, first8_hi = 0;
+  if (sends) {
+    const uint32_t slot = my_counter & (ring.max_nwqe - 1);
+    u32x4 *seg = reinterpret_cast<u32x4 *>(ring.sq + 8ull * slot);
+    const uint16_t idx16 = static_cast<uint16_t>(my_counter);
+    const bool inl = rq.opcode == kOpcodeRdmaWrite && rq.size <= kInlineThreshold;
+
+    // Segment 0: control.
+    const uint32_t ds = is_atomic ? 4u : 3u;
+    u32x4 c;
+    c.x = (static_cast<uint32_t>(rq.opcode) << 24) |
+          (static_cast<uint32_t>(__builtin_bswap16(idx16)) << 8);
+    c.y = (ds << 24) | ring.ctrl_qp_sq;
+    const uint32_t fm_ce_se = last ? kCqUpdate : static_cast<uint32_t>((ring.ctrl_sig >> 24) & 0xffu);
+    c.z = static_cast<uint32_t>(ring.ctrl_sig & 0xffu) | (fm_ce_se << 24);
+    c.w = static_cast<uint32_t>(ring.ctrl_sig >> 32);
+    seg[0] = c;
+    first8_lo = c.x;
+    first8_hi = c.y;
+
+    // Segment 1: remote address and key.
+    u32x4 r;
+    r.x = be64_first(rq.raddr);
+      r.y = be64_second(rq.raddr);
+    r.z = ring.rkey_by_pe[rq.pe];
+    r.w = 0;
+    seg[1] = r;
+
+    if (is_atomic) {
+      u32x4 a;
+      a.x = be64_first(rq.atomic_data);
+      a.y = be64_second(rq.atomic_data);
+      a.z = be64_first(rq.atomic_cmp);
+      a.w = be64_second(rq.atomic_cmp);
+      seg[2] = a;
+      const uint32_t pos = (abase + rank_in_mask(atomic_mask)) % kAtomicRetSlots;
+      u32x4 d;
+      d.x = be32(8u);
+      d.y = ring.atomic_lkey;
+      d.z = be64_first(ring.atomic_ret_base + 8ull * pos);
+      d.w = be64_second(ring.atomic_ret_base + 8ull * pos);
+      seg[3] = d;
+    } else if (inl) {
+      uint32_t *w = reinterpret_cast<uint32_t *>(&seg[2]);
+      w[0] = be32((rq.size & 0x3ffu) | 0x80000000u);
+      if (rq.size == 8) {
+        w[1] = static_cast<uint32_t>(rq.inline_data);
+        w[2] = static_cast<uint32_t>(rq.inline_data >> 32);
+      } else if (rq.size == 4) {
+        w[1] = static_cast<uint32_t>(rq.inline_data);
+      } else {
+        uint8_t *b = reinterpret_cast<uint8_t *>(w + 1);
+        for (uint32_t i = 0; i < rq.size; ++i) b[i] = static_cast<uint8_t>(rq.inline_data >> (8 * i));
+      }
+    } else {
+      u32x4 d;
+      d.x = be32(rq.size & 0x7fffffffu);
+      d.y = ring.lkey;
+      d.z = be64_first(rq.laddr);
+      d.w = be64_second(rq.laddr);
+      seg[2] = d;
+    }
+  }
+
+  // Publish: entries become visible to a consumer in index order.  The last
+  // posting lane waits for every earlier range, then moves the doorbell
+  // record and writes the doorbell value (first 8 bytes of the wave's last
+  // entry, as the reference's finishPost does).
+  fence_release_agent();
+  if (last) {
+    bounded_wait<uint32_t>(&cnt->published, kWaitEq, base);
+    ring.mailbox[0] = be32(base + n);
+    ring.mailbox[1] = (static_cast<uint64_t>(first8_hi) << 32) | first8_lo;
+    fence_release_agent();
+    __hip_atomic_store(&cnt->published, base + n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+}  // namespace detail
+}  // namespace rocshmem
+
+#endif
