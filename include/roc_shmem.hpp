@@ -161,7 +161,7 @@ __host__ int roc_shmemx_take_status();
 
 namespace detail {
 // Registration of one translation unit's copy of the device state.
-typedef void (*StateUploadFn)(const DeviceState *);
+typedef bool (*StateUploadFn)(const DeviceState *);
 void register_state_upload(StateUploadFn fn);
 }  // namespace detail
 

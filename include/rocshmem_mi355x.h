@@ -110,6 +110,7 @@ int rsm_free(void *ptr);
 size_t rsm_heap_bytes_in_use(void);
 void *rsm_ptr(const void *sym, int pe);         /* roc_shmem_ptr: address of `sym` in PE `pe`'s slice */
 void *rsm_heap_base(int pe);                    /* first byte of PE `pe`'s slice (reference: base_heap[pe]) */
+int rsm_state_units(void);                      /* translation units holding a copy of the device state */
 int rsm_take_status(void);                      /* sticky device status word, cleared by the call */
 
 /* ---- teams (reference: roc_shmem.cpp:188-313, team.cpp:47-107) ------------ */

@@ -28,6 +28,7 @@ SIGNATURES = {
     "rsm_heap_bytes_in_use": (sz, []),
     "rsm_ptr": (vp, [vp, i32]),
     "rsm_heap_base": (vp, [i32]),
+    "rsm_state_units": (i32, []),
     "rsm_take_status": (i32, []),
     "rsm_team_world": (u64, []),
     "rsm_team_split_strided": (i32, [u64, i32, i32, i32, C.POINTER(u64)]),

@@ -155,6 +155,8 @@ void *rsm_heap_base(int pe) {
   return rt->slice_base(pe);
 }
 
+int rsm_state_units(void) { return rocshmem::host::registered_state_units(); }
+
 int rsm_take_status(void) {
   RSM_NEED_RT(rt);
   return static_cast<int>(rt->take_status());

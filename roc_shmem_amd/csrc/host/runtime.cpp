@@ -231,7 +231,8 @@ std::string Runtime::init(const Options &opt) {
   state_.team_world = world_->device;
   state_.status = status_dev_;
   state_.wait_limit_ticks = static_cast<uint64_t>(opt_.wait_limit_s * 100e6);  // 100 MHz clock
-  upload_state_everywhere(state_);
+  if (!upload_state_everywhere(state_))
+    return "could not upload the device state into every translation unit";
   RT_HIP(hipDeviceSynchronize());
   return "";
 }
@@ -257,7 +258,7 @@ void Runtime::teardown() {
   teams_.clear();
   world_ = nullptr;
   detail::DeviceState cleared{};
-  upload_state_everywhere(cleared);
+  (void)upload_state_everywhere(cleared);
 }
 
 bool Runtime::owns(const void *p) const {
@@ -377,20 +378,28 @@ uint32_t Runtime::take_status() {
 // State upload registry
 // ---------------------------------------------------------------------------
 
-typedef void (*UploadFn)(const detail::DeviceState *);
+typedef bool (*UploadFn)(const detail::DeviceState *);
 static std::vector<UploadFn> &registry() {
   static std::vector<UploadFn> fns;
   return fns;
 }
 
-void upload_state_everywhere(const detail::DeviceState &state) {
-  for (UploadFn fn : registry()) fn(&state);
+bool upload_state_everywhere(const detail::DeviceState &state) {
+  bool ok = true;
+  for (UploadFn fn : registry()) ok = fn(&state) && ok;
+  return ok;
+}
+
+int registered_state_units() {
+  std::vector<UploadFn> fns = registry();
+  std::sort(fns.begin(), fns.end());
+  return static_cast<int>(std::unique(fns.begin(), fns.end()) - fns.begin());
 }
 
 }  // namespace host
 
 namespace detail {
-typedef void (*StateUploadFn)(const DeviceState *);
+typedef bool (*StateUploadFn)(const DeviceState *);
 void register_state_upload(StateUploadFn fn) { host::registry().push_back(fn); }
 }  // namespace detail
 

@@ -133,7 +133,10 @@ class Runtime {
 
 // Every translation unit that contains kernels registers a function that
 // copies the device state into its own __constant__ instance.
-void upload_state_everywhere(const detail::DeviceState &state);
+// Returns false when any unit could not be updated and verified.
+bool upload_state_everywhere(const detail::DeviceState &state);
+// Number of distinct translation units registered for state uploads.
+int registered_state_units();
 
 }  // namespace host
 }  // namespace rocshmem

@@ -24,15 +24,28 @@ namespace rocshmem {
 
 namespace detail {
 
-// Per translation unit hook: uploads the runtime state into this unit's
-// __constant__ copy when the host library initialises.
-inline void upload_state_to_this_unit(const DeviceState *s) {
-  (void)hipMemcpyToSymbol(HIP_SYMBOL(g_state), s, sizeof(DeviceState), 0, hipMemcpyHostToDevice);
+// Per translation unit hook.  Every unit that includes this header owns a
+// private __constant__ copy of the runtime state; the hook below copies a new
+// state into this unit's copy and reads it back.  Both the function and the
+// registrar object have internal linkage on purpose: with external (inline)
+// linkage the linker would keep a single instance that refers to one unit's
+// copy only, and kernels of every other unit would run on a zeroed state.
+namespace {
+bool upload_state_to_this_unit(const DeviceState *s) {
+  if (hipMemcpyToSymbol(HIP_SYMBOL(g_state), s, sizeof(DeviceState), 0,
+                        hipMemcpyHostToDevice) != hipSuccess)
+    return false;
+  DeviceState check;
+  if (hipMemcpyFromSymbol(&check, HIP_SYMBOL(g_state), sizeof(DeviceState), 0,
+                          hipMemcpyDeviceToHost) != hipSuccess)
+    return false;
+  return __builtin_memcmp(&check, s, sizeof(DeviceState)) == 0;
 }
 struct StateRegistrar {
   StateRegistrar() { register_state_upload(&upload_state_to_this_unit); }
 };
-static StateRegistrar g_state_registrar;
+StateRegistrar g_state_registrar;
+}  // namespace
 
 __device__ __forceinline__ int launch_pe() { return blockIdx.x % g_state.num_pes; }
 __device__ __forceinline__ int launch_wg_rank() { return blockIdx.x / g_state.num_pes; }
