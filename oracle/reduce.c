@@ -95,71 +95,66 @@ static int op_defined(int dtype, int op) {
   return dtype >= ORC_SHORT && dtype <= ORC_LONGLONG;
 }
 
+/* dst[i] = dst[i] (op) src[i] over [0, n): the shape of compute_reduce
+ * (context_ib_tmpl_device.hpp:106-113), one typed loop per operator so the
+ * compiler can vectorise it. */
+#define DEF_COMBINE(NAME, T, FOLD)                                              \
+  static void NAME(int op, T *restrict dst, const T *restrict src, size_t n) {  \
+    switch (op) {                                                               \
+      case ORC_SUM: for (size_t i = 0; i < n; ++i) dst[i] = FOLD(ORC_SUM, dst[i], src[i]); break;   \
+      case ORC_PROD: for (size_t i = 0; i < n; ++i) dst[i] = FOLD(ORC_PROD, dst[i], src[i]); break; \
+      case ORC_AND: for (size_t i = 0; i < n; ++i) dst[i] = FOLD(ORC_AND, dst[i], src[i]); break;   \
+      case ORC_OR: for (size_t i = 0; i < n; ++i) dst[i] = FOLD(ORC_OR, dst[i], src[i]); break;     \
+      case ORC_XOR: for (size_t i = 0; i < n; ++i) dst[i] = FOLD(ORC_XOR, dst[i], src[i]); break;   \
+      case ORC_MAX: for (size_t i = 0; i < n; ++i) dst[i] = FOLD(ORC_MAX, dst[i], src[i]); break;   \
+      default: for (size_t i = 0; i < n; ++i) dst[i] = FOLD(ORC_MIN, dst[i], src[i]); break;        \
+    }                                                                           \
+  }
+DEF_COMBINE(combine_i16, int16_t, fold_i16)
+DEF_COMBINE(combine_i32, int32_t, fold_i32)
+DEF_COMBINE(combine_i64, int64_t, fold_i64)
+DEF_COMBINE(combine_f32, float, fold_f32)
+DEF_COMBINE(combine_f64, double, fold_f64)
+
+/* bfloat16 has no arithmetic of its own.  A sum step is done in float and
+ * rounded back to the element type, which is what an in-type
+ * `dst[i] += src[i]` amounts to; max/min keep the selected operand's bits. */
+static void combine_bf16(int op, uint16_t *restrict dst, const uint16_t *restrict src, size_t n) {
+  for (size_t i = 0; i < n; ++i) {
+    float fa = orc_bf16_to_float(dst[i]), fx = orc_bf16_to_float(src[i]);
+    if (op == ORC_SUM) dst[i] = orc_float_to_bf16(fa + fx);
+    else if (op == ORC_MAX) dst[i] = (fa >= fx || fx != fx) ? dst[i] : src[i];
+    else dst[i] = (fa <= fx || fx != fx) ? dst[i] : src[i];
+  }
+}
+
+/* Elements [e0, e1): the first member's destination starts as a copy of its
+ * source, every other member's source is folded in ascending order, and the
+ * result is copied to the remaining members' destinations.  The fold runs in
+ * a bounded scratch block so that dest == source (in place) and misaligned
+ * offsets are handled the same way. */
 static void reduce_range(int dtype, int op, char *heap, size_t stride, size_t dest_off,
                          size_t src_off, size_t e0, size_t e1, int pe_start, int log_stride,
                          int pe_size) {
+  enum { BLOCK = 4096 };
   const size_t es = orc_dtype_size(dtype);
-  for (size_t i = e0; i < e1; ++i) {
-    unsigned char result[8];
-    const char *first = heap + (size_t)member_pe(0, pe_start, log_stride) * stride + src_off + i * es;
-    switch (dtype) {
-      case ORC_SHORT: {
-        int16_t acc; memcpy(&acc, first, 2);
-        for (int k = 1; k < pe_size; ++k) {
-          int16_t x; memcpy(&x, heap + (size_t)member_pe(k, pe_start, log_stride) * stride + src_off + i * es, 2);
-          acc = fold_i16(op, acc, x);
-        }
-        memcpy(result, &acc, 2);
-      } break;
-      case ORC_INT: {
-        int32_t acc; memcpy(&acc, first, 4);
-        for (int k = 1; k < pe_size; ++k) {
-          int32_t x; memcpy(&x, heap + (size_t)member_pe(k, pe_start, log_stride) * stride + src_off + i * es, 4);
-          acc = fold_i32(op, acc, x);
-        }
-        memcpy(result, &acc, 4);
-      } break;
-      case ORC_LONG: case ORC_LONGLONG: {
-        int64_t acc; memcpy(&acc, first, 8);
-        for (int k = 1; k < pe_size; ++k) {
-          int64_t x; memcpy(&x, heap + (size_t)member_pe(k, pe_start, log_stride) * stride + src_off + i * es, 8);
-          acc = fold_i64(op, acc, x);
-        }
-        memcpy(result, &acc, 8);
-      } break;
-      case ORC_FLOAT: {
-        float acc; memcpy(&acc, first, 4);
-        for (int k = 1; k < pe_size; ++k) {
-          float x; memcpy(&x, heap + (size_t)member_pe(k, pe_start, log_stride) * stride + src_off + i * es, 4);
-          acc = fold_f32(op, acc, x);
-        }
-        memcpy(result, &acc, 4);
-      } break;
-      case ORC_DOUBLE: {
-        double acc; memcpy(&acc, first, 8);
-        for (int k = 1; k < pe_size; ++k) {
-          double x; memcpy(&x, heap + (size_t)member_pe(k, pe_start, log_stride) * stride + src_off + i * es, 8);
-          acc = fold_f64(op, acc, x);
-        }
-        memcpy(result, &acc, 8);
-      } break;
-      default: { /* ORC_BF16: the element type has no arithmetic of its own.
-                    A sum step is done in float and rounded back to the element
-                    type, which is what an in-type `dst[i] += src[i]` amounts
-                    to; max/min keep the bit pattern of the selected operand. */
-        uint16_t acc; memcpy(&acc, first, 2);
-        for (int k = 1; k < pe_size; ++k) {
-          uint16_t x; memcpy(&x, heap + (size_t)member_pe(k, pe_start, log_stride) * stride + src_off + i * es, 2);
-          float fa = orc_bf16_to_float(acc), fx = orc_bf16_to_float(x);
-          if (op == ORC_SUM) acc = orc_float_to_bf16(fa + fx);
-          else if (op == ORC_MAX) acc = (fa >= fx || fx != fx) ? acc : x;
-          else acc = (fa <= fx || fx != fx) ? acc : x;
-        }
-        memcpy(result, &acc, 2);
-      } break;
+  union { int64_t i64[BLOCK]; double f64[BLOCK]; char bytes[BLOCK * 8]; } acc, in;
+  for (size_t b = e0; b < e1; b += BLOCK) {
+    const size_t n = (e1 - b < BLOCK) ? e1 - b : BLOCK;
+    memcpy(acc.bytes, heap + (size_t)member_pe(0, pe_start, log_stride) * stride + src_off + b * es, n * es);
+    for (int k = 1; k < pe_size; ++k) {
+      memcpy(in.bytes, heap + (size_t)member_pe(k, pe_start, log_stride) * stride + src_off + b * es, n * es);
+      switch (dtype) {
+        case ORC_SHORT: combine_i16(op, (int16_t *)acc.bytes, (const int16_t *)in.bytes, n); break;
+        case ORC_INT: combine_i32(op, (int32_t *)acc.bytes, (const int32_t *)in.bytes, n); break;
+        case ORC_LONG: case ORC_LONGLONG: combine_i64(op, acc.i64, in.i64, n); break;
+        case ORC_FLOAT: combine_f32(op, (float *)acc.bytes, (const float *)in.bytes, n); break;
+        case ORC_DOUBLE: combine_f64(op, acc.f64, in.f64, n); break;
+        default: combine_bf16(op, (uint16_t *)acc.bytes, (const uint16_t *)in.bytes, n); break;
+      }
     }
     for (int m = 0; m < pe_size; ++m)
-      memcpy(heap + (size_t)member_pe(m, pe_start, log_stride) * stride + dest_off + i * es, result, es);
+      memcpy(heap + (size_t)member_pe(m, pe_start, log_stride) * stride + dest_off + b * es, acc.bytes, n * es);
   }
 }
 

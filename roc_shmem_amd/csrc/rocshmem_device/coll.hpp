@@ -58,13 +58,8 @@ __device__ __forceinline__ void wg_copy_to_members(char *dst_mine, const char *s
   size_t head = (16u - (reinterpret_cast<uintptr_t>(src) & 15u)) & 15u;
   size_t nvec = (n - head) / 16;
   size_t tail = n - head - nvec * 16;
-  if (tid < head) {
-    char b = src[tid];
-    for (int m = 0; m < as.size; ++m)
-      if (m != skip_idx) dst0[m * member_step + tid] = b;
-  }
-  if (tid < tail) {
-    size_t off = head + nvec * 16 + tid;
+  for (size_t t = tid; t < head + tail; t += nthr) {
+    size_t off = t < head ? t : nvec * 16 + t;  // head bytes, then the bytes after the vectors
     char b = src[off];
     for (int m = 0; m < as.size; ++m)
       if (m != skip_idx) dst0[m * member_step + off] = b;

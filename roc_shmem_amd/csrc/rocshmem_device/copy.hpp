@@ -109,7 +109,7 @@ __device__ __forceinline__ void group_copy(void *dst, const void *src, size_t n,
   }
   // Head: bring the destination to a 16-byte boundary.
   size_t head = (16u - (reinterpret_cast<uintptr_t>(d) & 15u)) & 15u;
-  if (tid < head) d[tid] = s[tid];
+  for (size_t i = tid; i < head; i += nthr) d[i] = s[i];
   d += head;
   s += head;
   n -= head;
@@ -131,7 +131,7 @@ __device__ __forceinline__ void group_copy(void *dst, const void *src, size_t n,
   }
   // Tail: fewer than 16 bytes.
   size_t tail = n - body;
-  if (tid < tail) d[body + tid] = s[body + tid];
+  for (size_t i = tid; i < tail; i += nthr) d[body + i] = s[body + i];
 }
 
 __device__ __forceinline__ void wg_copy(void *dst, const void *src, size_t n) {

@@ -1,0 +1,143 @@
+"""Parity of broadcast / alltoall / fcollect / barrier with the CPU oracle."""
+import numpy as np
+import pytest
+
+import oracle
+import roc_shmem_amd as rs
+from helpers import runtime
+
+pytestmark = pytest.mark.gpu
+
+GUARD = 0x3C
+
+
+def setup(n_pes, src_bytes, dst_bytes, seed):
+    src = rs.sym_array(src_bytes, np.uint8)
+    dst = rs.sym_array(dst_bytes, np.uint8)
+    heap = oracle.Heap(n_pes, src_bytes + dst_bytes + 128)
+    rng = np.random.default_rng(seed)
+    for p in range(n_pes):
+        payload = rng.integers(0, 256, size=src_bytes, dtype=np.uint8)
+        src.write(p, payload)
+        heap.view(p, 0, src_bytes, np.uint8)[:] = payload
+        dst.fill(GUARD, pe=p)
+        heap.view(p, src_bytes, dst_bytes, np.uint8)[:] = GUARD
+    return src, dst, heap
+
+
+def compare(n_pes, dst, heap, src_bytes, dst_bytes):
+    for p in range(n_pes):
+        got = dst.read(p)
+        exp = heap.view(p, src_bytes, dst_bytes, np.uint8)
+        assert np.array_equal(got, exp), "PE %d: first difference at byte %d" % (
+            p, int(np.argmax(got != exp)))
+
+
+@pytest.mark.parametrize("elem_size", [1, 2, 4, 8])
+@pytest.mark.parametrize("root", [0, 3])
+def test_broadcast_active_set_world(elem_size, root):
+    n_pes, nelem = 8, 3001
+    nbytes = nelem * elem_size
+    with runtime(n_pes):
+        src, dst, heap = setup(n_pes, nbytes, nbytes + 64, seed=elem_size * 10 + root)
+        psync = rs.sym_array(256 * 2, np.int64, fill=0)
+        rs.roc_shmem_broadcast(elem_size, dst, src, nelem, root, 0, 0, n_pes, psync, rs.Launch(2, 256))
+        rs.synchronize()
+        oracle.broadcast(heap, nbytes, 0, nbytes, root)
+        compare(n_pes, dst, heap, nbytes, nbytes + 64)
+        # root's dest untouched (clients/sos_tests/broadcast_active_set.cpp:84-96)
+        assert (dst.read(root) == GUARD).all()
+        for p in range(n_pes):
+            assert not psync.read(p).any()
+
+
+@pytest.mark.parametrize("pe_start,log_stride,pe_size,root", [(2, 0, 5, 0), (1, 1, 3, 2), (0, 2, 2, 1)])
+def test_broadcast_shrinking_and_strided_sets(pe_start, log_stride, pe_size, root):
+    # PE_root counts within the active set (clients/sos_tests/broadcast_active_set.cpp:84-96
+    # passes root 0 with PE_start = i and expects world PE i to be the root)
+    n_pes, nelem = 8, 1000
+    with runtime(n_pes):
+        src, dst, heap = setup(n_pes, nelem * 8, nelem * 8, seed=pe_start + 31)
+        psync = rs.sym_array(256, np.int64, fill=0)
+        rs.roc_shmem_broadcast(8, dst, src, nelem, root, pe_start, log_stride, pe_size, psync)
+        rs.synchronize()
+        oracle.broadcast(heap, nelem * 8, 0, nelem * 8, root, pe_start, log_stride, pe_size)
+        compare(n_pes, dst, heap, nelem * 8, nelem * 8)
+
+
+def test_broadcast_reference_pattern_and_team_form():
+    # clients/functional_tests/tester.cpp:236-271: source 1, dest 2, non-roots read 1, root keeps 2
+    n_pes, nelem = 4, 512
+    with runtime(n_pes):
+        src = rs.sym_array(nelem, np.int64)
+        dst = rs.sym_array(nelem, np.int64)
+        for p in range(n_pes):
+            src.write(p, np.full(nelem, 1, np.int64))
+            dst.write(p, np.full(nelem, 2, np.int64))
+        rs.roc_shmem_team_broadcast(8, rs.roc_shmem_team_world(), dst, src, nelem, 0)
+        rs.synchronize()
+        assert (dst.read(0) == 2).all()
+        for p in range(1, n_pes):
+            assert (dst.read(p) == 1).all()
+        # team-relative root: team {1,3}, root ordinal 1 -> world PE 3
+        rc, team = rs.roc_shmem_team_split_strided(rs.roc_shmem_team_world(), 1, 2, 2)
+        assert rc == 0
+        for p in range(n_pes):
+            src.write(p, np.full(nelem, 10 + p, np.int64))
+            dst.write(p, np.full(nelem, -1, np.int64))
+        rs.roc_shmem_team_broadcast(8, team, dst, src, nelem, 1, rs.Launch(2, 128))
+        rs.synchronize()
+        assert (dst.read(1) == 13).all()
+        for p in (0, 2, 3):
+            assert (dst.read(p) == -1).all()
+        rs.roc_shmem_team_destroy(team)
+
+
+@pytest.mark.parametrize("elem_size,nelem", [(4, 1000), (8, 257), (1, 4099), (2, 64)])
+@pytest.mark.parametrize("wgs", [1, 3])
+def test_alltoall_and_fcollect(elem_size, nelem, wgs):
+    n_pes = 8
+    block = elem_size * nelem
+    with runtime(n_pes):
+        world = rs.roc_shmem_team_world()
+        src, dst, heap = setup(n_pes, block * n_pes, block * n_pes + 32, seed=nelem)
+        rs.roc_shmem_alltoall(elem_size, world, dst, src, nelem, rs.Launch(wgs, 256))
+        rs.synchronize()
+        oracle.alltoall(heap, block * n_pes, 0, block)
+        compare(n_pes, dst, heap, block * n_pes, block * n_pes + 32)
+        src.free()
+        dst.free()
+        src, dst, heap = setup(n_pes, block, block * n_pes + 32, seed=nelem + 1)
+        rs.roc_shmem_fcollect(elem_size, world, dst, src, nelem, rs.Launch(wgs, 256))
+        rs.synchronize()
+        oracle.fcollect(heap, block, 0, block)
+        compare(n_pes, dst, heap, block, block * n_pes + 32)
+
+
+def test_alltoall_reference_pattern_on_a_sub_team():
+    # clients/functional_tests/tester.cpp:310-334: value (src_pe << 16) + dst_pe, int64
+    n_pes, nelem = 8, 100
+    with runtime(n_pes):
+        rc, team = rs.roc_shmem_team_split_strided(rs.roc_shmem_team_world(), 0, 2, 4)
+        assert rc == 0
+        members = [0, 2, 4, 6]
+        src = rs.sym_array(nelem * 4, np.int64)
+        dst = rs.sym_array(nelem * 4, np.int64, fill=0xFF)
+        for i, p in enumerate(members):
+            vals = np.repeat(np.array([(i << 16) + j for j in range(4)], np.int64), nelem)
+            src.write(p, vals)
+        rs.roc_shmem_alltoall(8, team, dst, src, nelem, rs.Launch(2, 128))
+        rs.synchronize()
+        for j, p in enumerate(members):
+            exp = np.repeat(np.array([(i << 16) + j for i in range(4)], np.int64), nelem)
+            assert np.array_equal(dst.read(p), exp)
+        for p in (1, 3, 5, 7):
+            assert (dst.read(p).view(np.uint8) == 0xFF).all()
+        rs.roc_shmem_team_destroy(team)
+
+
+def test_barrier_all_many_rounds():
+    with runtime(8, num_blocks=8):
+        rs.roc_shmem_wg_barrier_all(200, rs.Launch(4, 64))
+        rs.synchronize()
+        assert rs.take_status() == 0
