@@ -1,0 +1,285 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X-native ROC_SHMEM data path.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+One "step" is one pass of the hot path over one batch of synthetic input: a
+`roc_shmem_ctx_float_sum_wg_to_all` over 8 PE slices of 2^26 elements each
+(the configuration the HBM-roofline target is quoted on), all slices resident
+in the one GPU's HBM before the timed region starts.  The JSON line also
+carries the other workloads of the metric (bf16 / int64 reductions, wg putmem,
+small puts and AMOs, broadcast, alltoall), the roofline of the dominant kernel
+and the CPU oracle timed on the host cores of the same box.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
+
+# HBM bytes per launch of the headline kernel measured with rocprofv3 --pmc
+# (FETCH_SIZE and WRITE_SIZE, scaled by a copy kernel of known size); see
+# profiles/.  None until measured.
+MEASURED_TRAFFIC_BYTES = None
+
+# Launch shapes chosen by measurement on MI355X (256 CUs).
+TO_ALL_LAUNCH = dict(wgs_per_pe=32, wg_size=512)
+PUT_LAUNCH = dict(wgs_per_pe=64, wg_size=256)
+PUT_TILE = 4 << 20
+
+
+def event_time_ms(rs, fn, iters):
+    start, stop = rs.Event(), rs.Event()
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    ms = start.elapsed_ms(stop)
+    start.destroy()
+    stop.destroy()
+    return ms
+
+
+def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, cpu=False):
+    """Returns a dict with ms_per_step, GB/s (algorithmic 2*P*N*s bytes) and optional CPU figures."""
+    npd = rs.NP_DTYPE[dtype]
+    es = np.dtype(npd).itemsize
+    src = rs.sym_array(n, npd)
+    dst = rs.sym_array(n, npd, fill=0x5A)
+    launch = rs.Launch(**TO_ALL_LAUNCH)
+    psync = rs.sym_array(launch.wgs_per_pe * rs.ROC_SHMEM_REDUCE_SYNC_SIZE, np.int64, fill=0)
+    rng = np.random.default_rng(seed)
+    host = []
+    for p in range(n_pes):
+        if dtype in (rs.LONG, rs.LONGLONG):
+            vals = rng.integers(-(1 << 30), (1 << 30) + 1, size=n, dtype=np.int64)
+        elif dtype == rs.BF16:
+            vals = oracle.float_to_bf16(rng.standard_normal(n, dtype=np.float32))
+        else:
+            vals = rng.standard_normal(n, dtype=np.float32).astype(npd)
+        src.write(p, vals)
+        host.append(vals)
+
+    def step():
+        rs.roc_shmem_to_all(dtype, rs.SUM, dst, src, n, 0, 0, n_pes, None, psync, launch)
+
+    for _ in range(warmup):
+        step()
+    rs.synchronize()
+    ms = event_time_ms(rs, step, steps)
+    rs.synchronize()
+    status = rs.take_status()
+    if status:
+        raise RuntimeError("device status word raised: %d" % status)
+    out = {"ms_per_step": ms / steps, "GBps": 2.0 * n_pes * n * es / (ms / steps) / 1e6,
+           "bytes_per_step": 2 * n_pes * n * es}
+
+    heap = None
+    if check or cpu:
+        heap = oracle.Heap(n_pes, 2 * n * es)
+        for p in range(n_pes):
+            heap.view(p, 0, n, npd)[:] = host[p]
+    if check:
+        m = min(n, 1 << 16)
+        sample = oracle.Heap(n_pes, 2 * m * es)
+        for p in range(n_pes):
+            sample.view(p, 0, m, npd)[:] = host[p][:m]
+        got = [dst.read(p, m) for p in range(n_pes)]
+        if dtype in (rs.LONG, rs.LONGLONG):
+            oracle.to_all(sample, dtype, oracle.SUM, m * es, 0, m)
+            for p in range(n_pes):
+                assert np.array_equal(got[p], sample.view(p, m * es, m, npd)), "parity check failed"
+        else:
+            ref = oracle.to_all_f64(sample, dtype, oracle.SUM, 0, m)
+            scale = oracle.abs_sum_f64(sample, dtype, 0, m)
+            tol, eps = (1e-6, 2.0 ** -24) if dtype == rs.FLOAT else (1e-2, 2.0 ** -8)
+            for p in range(n_pes):
+                g = (oracle.bf16_to_float(got[p]) if dtype == rs.BF16 else got[p]).astype(np.float64)
+                assert (np.abs(g - ref) <= tol * np.maximum(np.abs(ref), eps * scale)).all(), \
+                    "parity check failed"
+        out["parity_checked_elements"] = m
+    if cpu:
+        cores = min(16, os.cpu_count() or 1)
+        passes = []
+        for _ in range(4):
+            t0 = time.perf_counter()
+            oracle.to_all(heap, dtype, oracle.SUM, n * es, 0, n, threads=cores)
+            passes.append(time.perf_counter() - t0)
+        best = min(passes[1:])
+        out["cpu"] = {"value": 2.0 * n_pes * n * es / best / 1e9, "unit": "GB/s", "cores": cores,
+                      "kind": "port",
+                      "sample": "same workload, full size (%d slices x 2^%d %s, sum), CPU oracle "
+                                "chunked over %d host threads, best of 3 passes after one warm-up"
+                                % (n_pes, int(np.log2(n)), np.dtype(npd).name, cores)}
+    src.free()
+    dst.free()
+    psync.free()
+    return out
+
+
+def bench_putmem(rs, steps, n_pes, msg_bytes_list):
+    """wg putmem from every PE p to PE p+1: GB/s counted as 2*m bytes per message (read+write)."""
+    total = 256 << 20
+    src = rs.sym_array(total, np.uint8, fill=7)
+    dst = rs.sym_array(total, np.uint8, fill=0)
+    res = {}
+    for m in msg_bytes_list:
+        if m >= PUT_TILE:
+            tile, n_msgs = PUT_TILE, total // PUT_TILE      # large messages tiled across workgroups
+        else:
+            tile, n_msgs = m, min(total // max(m, 256), 1 << 16)
+        stride = max(tile, 256)
+        launch = rs.Launch(**PUT_LAUNCH)
+
+        def step():
+            rs.roc_shmem_rma(rs.PUT, rs.WG, dst, src, tile, n_msgs, stride, stride, 1, launch)
+
+        step()
+        rs.synchronize()
+        ms = event_time_ms(rs, step, steps) / steps
+        moved = 2.0 * n_pes * tile * n_msgs
+        res[str(m)] = {"GBps": moved / ms / 1e6, "ms": ms, "calls_per_pe": n_msgs, "bytes_per_call": tile,
+                       "Mmsgs_per_s": n_pes * n_msgs / ms / 1e3}
+    src.free()
+    dst.free()
+    return res
+
+
+def bench_small_ops(rs, n_pes, n_ops, wgs_total, wg_size, slice_bytes, seed):
+    """10 M 8-byte puts (unique targets, lower half) and int64 fetch-adds (upper half)."""
+    rng = np.random.default_rng(seed)
+    words = slice_bytes // 8
+    mem = rs.sym_array(words, np.int64, fill=0)
+    res = {}
+    for name, kinds in (("put8", (rs.OP_P64,)), ("fetch_add", (rs.OP_FADD64,)),
+                        ("mixed", (rs.OP_P64, rs.OP_FADD64))):
+        ops = np.zeros(n_ops, rs.SMALL_OP_DTYPE)
+        is_put = np.ones(n_ops, bool) if kinds == (rs.OP_P64,) else \
+            np.zeros(n_ops, bool) if kinds == (rs.OP_FADD64,) else (np.arange(n_ops) % 2 == 0)
+        ops["kind"] = np.where(is_put, rs.OP_P64, rs.OP_FADD64)
+        ops["pe"] = rng.integers(0, n_pes, n_ops)
+        uniq = rng.permutation(n_pes * (words // 2))[:n_ops]
+        ops["pe"][is_put] = uniq[is_put] // (words // 2)
+        ops["offset"] = np.where(is_put, (uniq % (words // 2)) * 8,
+                                 (words // 2 + rng.integers(0, words // 2, n_ops)) * 8) + mem.offset
+        ops["value"] = rng.integers(-1000, 1000, n_ops)
+        dev = rs.device_array(ops)
+        launch = rs.Launch(wgs_total // n_pes, wg_size)
+
+        def step():
+            rs.roc_shmem_small_ops(dev, n_ops, None, launch)
+
+        step()
+        rs.synchronize()
+        ms = event_time_ms(rs, step, 3) / 3
+        res[name] = {"Mops_per_s": n_ops / ms / 1e3, "ms": ms}
+        dev.free()
+    status = rs.take_status()
+    if status:
+        raise RuntimeError("device status word raised: %d" % status)
+    mem.free()
+    return res
+
+
+def bench_bcast_a2a(rs, n_pes, slice_bytes):
+    world = rs.roc_shmem_team_world()
+    res = {}
+    src = rs.sym_array(slice_bytes, np.uint8, fill=3)
+    dst = rs.sym_array(slice_bytes, np.uint8, fill=0)
+    launch = rs.Launch(16, 512)
+    nelem = slice_bytes // 4
+
+    def bcast():
+        rs.roc_shmem_team_broadcast(4, world, dst, src, nelem, 0, launch)
+
+    bcast()
+    rs.synchronize()
+    ms = event_time_ms(rs, bcast, 5) / 5
+    res["broadcast"] = {"GBps": (slice_bytes + (n_pes - 1) * slice_bytes) / ms / 1e6, "ms": ms}
+    block = nelem // n_pes
+
+    def a2a():
+        rs.roc_shmem_alltoall(4, world, dst, src, block, launch)
+
+    a2a()
+    rs.synchronize()
+    ms = event_time_ms(rs, a2a, 5) / 5
+    res["alltoall"] = {"GBps": 2.0 * n_pes * slice_bytes / ms / 1e6, "ms": ms}
+    src.free()
+    dst.free()
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--quick", action="store_true", help="headline workload only")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: every PE slice lives in one GPU's HBM; this build measures one GPU only "
+              "(--gpus %d is not supported)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import oracle
+    import roc_shmem_amd as rs
+
+    # ---- headline: fp32 sum_to_all, 8 slices x 2^26 elements (4 GiB algorithmic traffic) ----
+    n_pes, n = 8, 1 << 26
+    rs.roc_shmem_init(n_pes, 1 << 30, 64, 1024)
+    head = bench_to_all(rs, oracle, args.steps, args.warmup, rs.FLOAT, n_pes, n, seed=3, cpu=True)
+    extra = {}
+    if not args.quick:
+        extra["to_all_bf16_sum_8x2^26"] = {k: v for k, v in bench_to_all(
+            rs, oracle, max(args.steps // 2, 3), 2, rs.BF16, n_pes, n, seed=3).items() if k != "cpu"}
+        extra["putmem_wg_8pe"] = bench_putmem(rs, 5, n_pes, [8, 4096, 65536, 1 << 20, 64 << 20])
+    rs.roc_shmem_finalize()
+
+    if not args.quick:
+        rs.roc_shmem_init(4, 64 << 20, 64, 1024)
+        extra["to_all_int64_sum_4x2^20"] = bench_to_all(rs, oracle, 20, 5, rs.LONG, 4, 1 << 20, seed=1)
+        rs.roc_shmem_finalize()
+
+        rs.roc_shmem_init(16, 256 << 20, 64, 1024)
+        extra["small_ops_16x64MiB_1024wg_x256"] = bench_small_ops(rs, 16, 10_000_000, 1024, 256,
+                                                                  64 << 20, seed=4)
+        extra["collectives_16x64MiB"] = bench_bcast_a2a(rs, 16, 64 << 20)
+        rs.roc_shmem_finalize()
+
+    cpu = head.pop("cpu")
+    line = {
+        "metric": "to_all reduce + putmem GB/s (% of HBM peak); small-put/AMO Mops/s",
+        "value": round(head["GBps"], 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(head["ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "float sum_to_all over 8 PE slices x 2^26 elements, N(0,1) inputs, "
+                               "all slices in one GPU's HBM (BASELINE configs[2], fp32 sum)",
+                   "pes": n_pes, "elements_per_pe": n, "algorithmic_bytes_per_step": head["bytes_per_step"],
+                   "launch": TO_ALL_LAUNCH, "parity_checked_elements": head.get("parity_checked_elements")},
+        "roofline": {"bound": "hbm", "achieved": round(head["GBps"], 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(head["GBps"] / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES},
+        "cpu_baseline": {k: (round(v, 2) if isinstance(v, float) else v) for k, v in cpu.items()},
+        "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -186,8 +186,12 @@ __device__ inline void roc_shmem_threadfence_system() { __threadfence_system(); 
 
 __device__ inline void roc_shmem_ctx_putmem(roc_shmem_ctx_t ctx, void *dest, const void *source,
                                             size_t nelems, int pe) {
+  // The copy is synchronous in the calling lane, so `source` is reusable on
+  // return (local completion, all OpenSHMEM asks of a blocking put).  Remote
+  // visibility comes with quiet/fence/barrier; the reference adds a device-wide
+  // __threadfence here (fence_.flush(), context_ib_device.cpp:164), which on a
+  // multi-XCD part means writing back a whole L2 per call.
   detail::thread_put(detail::ctx_of(ctx), dest, source, nelems, detail::world_pe(ctx, pe));
-  detail::fence_release_agent();  // reference: fence_.flush() after a blocking put
 }
 __device__ inline void roc_shmem_ctx_putmem_nbi(roc_shmem_ctx_t ctx, void *dest,
                                                 const void *source, size_t nelems, int pe) {
@@ -219,7 +223,8 @@ __device__ inline void roc_shmem_getmem_nbi(void *dest, const void *source, size
 // ---------------------------------------------------------------------------
 // Workgroup- and wavefront-level RMA (reference: roc_shmem.hpp:2029-2566;
 // GPUIBContext::putmem_wg ..., context_ib_device.cpp:189-321).  The PE is a
-// world PE.  Blocking forms order the data before the return.
+// world PE.  Blocking and non-blocking forms move the data the same way;
+// roc_shmem_ctx_quiet / fence / a barrier make it visible to other PEs.
 // ---------------------------------------------------------------------------
 
 __device__ inline void roc_shmemx_ctx_putmem_nbi_wg(roc_shmem_ctx_t ctx, void *dest,
@@ -231,9 +236,9 @@ __device__ inline void roc_shmemx_ctx_putmem_nbi_wg(roc_shmem_ctx_t ctx, void *d
 }
 __device__ inline void roc_shmemx_ctx_putmem_wg(roc_shmem_ctx_t ctx, void *dest,
                                                 const void *source, size_t nelems, int pe) {
-  if (nelems == 0) return;
+  // Same data movement as the non-blocking form: the lanes' own loads have
+  // returned before their stores issue, so the source is reusable on return.
   roc_shmemx_ctx_putmem_nbi_wg(ctx, dest, source, nelems, pe);
-  detail::fence_release_agent();
 }
 __device__ inline void roc_shmemx_ctx_getmem_nbi_wg(roc_shmem_ctx_t ctx, void *dest,
                                                     const void *source, size_t nelems, int pe) {
@@ -244,9 +249,9 @@ __device__ inline void roc_shmemx_ctx_getmem_nbi_wg(roc_shmem_ctx_t ctx, void *d
 }
 __device__ inline void roc_shmemx_ctx_getmem_wg(roc_shmem_ctx_t ctx, void *dest,
                                                 const void *source, size_t nelems, int pe) {
-  if (nelems == 0) return;
+  // Same data movement as the non-blocking form: the lanes' own loads have
+  // returned before their stores issue, so the source is reusable on return.
   roc_shmemx_ctx_getmem_nbi_wg(ctx, dest, source, nelems, pe);
-  detail::fence_release_agent();
 }
 __device__ inline void roc_shmemx_ctx_putmem_nbi_wave(roc_shmem_ctx_t ctx, void *dest,
                                                       const void *source, size_t nelems,
@@ -257,9 +262,9 @@ __device__ inline void roc_shmemx_ctx_putmem_nbi_wave(roc_shmem_ctx_t ctx, void 
 }
 __device__ inline void roc_shmemx_ctx_putmem_wave(roc_shmem_ctx_t ctx, void *dest,
                                                   const void *source, size_t nelems, int pe) {
-  if (nelems == 0) return;
+  // Same data movement as the non-blocking form: the lanes' own loads have
+  // returned before their stores issue, so the source is reusable on return.
   roc_shmemx_ctx_putmem_nbi_wave(ctx, dest, source, nelems, pe);
-  detail::fence_release_agent();
 }
 __device__ inline void roc_shmemx_ctx_getmem_nbi_wave(roc_shmem_ctx_t ctx, void *dest,
                                                       const void *source, size_t nelems,
@@ -270,9 +275,9 @@ __device__ inline void roc_shmemx_ctx_getmem_nbi_wave(roc_shmem_ctx_t ctx, void 
 }
 __device__ inline void roc_shmemx_ctx_getmem_wave(roc_shmem_ctx_t ctx, void *dest,
                                                   const void *source, size_t nelems, int pe) {
-  if (nelems == 0) return;
+  // Same data movement as the non-blocking form: the lanes' own loads have
+  // returned before their stores issue, so the source is reusable on return.
   roc_shmemx_ctx_getmem_nbi_wave(ctx, dest, source, nelems, pe);
-  detail::fence_release_agent();
 }
 
 #define ROCSHMEM_X_DEFAULT_CTX_MEM(NAME)                                                  \
