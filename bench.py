@@ -223,6 +223,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--quick", action="store_true", help="headline workload only")
+    ap.add_argument("--counter-pair", action="store_true",
+                    help="for rocprofv3 --pmc: a few launches of the headline kernel and of a "
+                         "plain wg putmem copy of known size (2 GiB read + 2 GiB written), nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: every PE slice lives in one GPU's HBM; this build measures one GPU only "
@@ -235,6 +238,13 @@ def main():
     # ---- headline: fp32 sum_to_all, 8 slices x 2^26 elements (4 GiB algorithmic traffic) ----
     n_pes, n = 8, 1 << 26
     rs.roc_shmem_init(n_pes, 1 << 30, 64, 1024)
+    if args.counter_pair:
+        out = bench_to_all(rs, oracle, 3, 1, rs.FLOAT, n_pes, n, seed=3, check=False)
+        put = bench_putmem(rs, 3, n_pes, [64 << 20])
+        rs.roc_shmem_finalize()
+        print(json.dumps({"to_all": out, "putmem_copy": put,
+                          "copy_bytes_read": n_pes * (256 << 20), "copy_bytes_written": n_pes * (256 << 20)}))
+        return
     head = bench_to_all(rs, oracle, args.steps, args.warmup, rs.FLOAT, n_pes, n, seed=3, cpu=True)
     extra = {}
     if not args.quick:

@@ -218,6 +218,17 @@ int rsm_kat_coalesce(uint64_t lane_mask, const int32_t *pe, const uint64_t *src,
                      const uint64_t *dst, const uint64_t *size, uint8_t *must_send,
                      uint64_t *out_size);
 
+/* ---- host-logic hooks (no GPU needed) ------------------------------------------------
+ * A free-standing instance of the symmetric-heap allocator that rsm_malloc uses
+ * (reference behaviour: library/src/memory/pow2_bins.hpp:90-125,264-287): offsets
+ * inside a heap of `heap_bytes`; rsm_host_alloc_alloc returns (size_t)-1 when
+ * nothing fits or the request is 0. */
+void *rsm_host_alloc_create(size_t heap_bytes);
+void rsm_host_alloc_destroy(void *allocator);
+size_t rsm_host_alloc_alloc(void *allocator, size_t request);
+int rsm_host_alloc_free(void *allocator, size_t offset);
+size_t rsm_host_alloc_in_use(void *allocator);
+
 #ifdef __cplusplus
 }
 #endif

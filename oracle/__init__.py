@@ -49,6 +49,12 @@ def _load():
     lib.orc_small_ops.argtypes = [vp, sz, vp, vp, sz, vp]
     lib.orc_wqe_build.restype = None
     lib.orc_wqe_build.argtypes = [vp, vp, u32, vp]
+    lib.orc_wqe_index.restype = C.c_uint16
+    lib.orc_wqe_index.argtypes = [vp]
+    lib.orc_wqe_opcode.restype = C.c_uint8
+    lib.orc_wqe_opcode.argtypes = [vp]
+    lib.orc_wqe_raddr.restype = u64
+    lib.orc_wqe_raddr.argtypes = [vp]
     lib.orc_doorbell.restype = None
     lib.orc_doorbell.argtypes = [vp, u32, vp]
     lib.orc_bswap16.restype = C.c_uint16
@@ -224,6 +230,18 @@ def wqe_build(slot, qp, sq_counter, opcode, size=0, raddr=0, rkey=0, laddr=0, at
     rq.request_cqe = 1 if request_cqe else 0
     _lib.orc_wqe_build(slot.ctypes.data, C.byref(qp), sq_counter & 0xFFFFFFFF, C.byref(rq))
     return slot
+
+
+def wqe_index(slot):
+    return int(_lib.orc_wqe_index(slot.ctypes.data))
+
+
+def wqe_opcode(slot):
+    return int(_lib.orc_wqe_opcode(slot.ctypes.data))
+
+
+def wqe_raddr(slot):
+    return int(_lib.orc_wqe_raddr(slot.ctypes.data))
 
 
 def doorbell(last_slot, sq_counter_after):

@@ -18,7 +18,7 @@
 
 #include "oracle.h"
 
-#define ORC_BINS 58
+#define ORC_BINS 56
 #define ORC_MIN_SHIFT 7
 
 struct orc_alloc {

@@ -65,6 +65,11 @@ SIGNATURES = {
     "rsm_sq_rkey": (i32, [i32, C.POINTER(u32)]),
     "rsm_kat_fetch_incr": (i32, [u64, i32, i32, vp, C.POINTER(u64)]),
     "rsm_kat_coalesce": (i32, [u64, vp, vp, vp, vp, vp, vp]),
+    "rsm_host_alloc_create": (vp, [sz]),
+    "rsm_host_alloc_destroy": (None, [vp]),
+    "rsm_host_alloc_alloc": (sz, [vp, sz]),
+    "rsm_host_alloc_free": (i32, [vp, sz]),
+    "rsm_host_alloc_in_use": (sz, [vp]),
 }
 
 _lib = None

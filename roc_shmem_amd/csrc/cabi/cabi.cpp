@@ -327,4 +327,22 @@ int rsm_sq_rkey(int dest_pe, uint32_t *rkey) {
   return 0;
 }
 
+// ---- host-logic hooks ------------------------------------------------------------
+
+void *rsm_host_alloc_create(size_t heap_bytes) {
+  return new rocshmem::host::Pow2Allocator(heap_bytes);
+}
+void rsm_host_alloc_destroy(void *allocator) {
+  delete static_cast<rocshmem::host::Pow2Allocator *>(allocator);
+}
+size_t rsm_host_alloc_alloc(void *allocator, size_t request) {
+  return static_cast<rocshmem::host::Pow2Allocator *>(allocator)->alloc(request);
+}
+int rsm_host_alloc_free(void *allocator, size_t offset) {
+  return static_cast<rocshmem::host::Pow2Allocator *>(allocator)->free(offset) ? 0 : -1;
+}
+size_t rsm_host_alloc_in_use(void *allocator) {
+  return static_cast<rocshmem::host::Pow2Allocator *>(allocator)->bytes_in_use();
+}
+
 }  // extern "C"
