@@ -96,6 +96,15 @@ __device__ __forceinline__ void wg_copy_to_members(char *dst_mine, const char *s
 __device__ __forceinline__ void wg_broadcast_bytes(int my_pe, void *dest, const void *source,
                                                    size_t nbytes, int root_idx, int pe_start,
                                                    int log_stride, int pe_size, long *psync) {
+  my_pe = uniform(my_pe);
+  dest = uniform(dest);
+  source = uniform(source);
+  nbytes = uniform(nbytes);
+  root_idx = uniform(root_idx);
+  pe_start = uniform(pe_start);
+  log_stride = uniform(log_stride);
+  pe_size = uniform(pe_size);
+  psync = uniform(psync);
   if (nbytes == 0) return;
   if (pe_size > kMaxPes || pe_size <= 0 || root_idx < 0 || root_idx >= pe_size) {
     status_raise(kStatusBadArgument);
@@ -125,6 +134,16 @@ __device__ __forceinline__ void wg_alltoall_bytes(int my_pe, void *dest, const v
                                                   size_t block_bytes, size_t shard_begin,
                                                   size_t shard_end, int pe_start, int log_stride,
                                                   int pe_size, long *psync) {
+  my_pe = uniform(my_pe);
+  dest = uniform(dest);
+  source = uniform(source);
+  block_bytes = uniform(block_bytes);
+  shard_begin = uniform(shard_begin);
+  shard_end = uniform(shard_end);
+  pe_start = uniform(pe_start);
+  log_stride = uniform(log_stride);
+  pe_size = uniform(pe_size);
+  psync = uniform(psync);
   if (block_bytes == 0) return;
   if (pe_size > kMaxPes || pe_size <= 0) {
     status_raise(kStatusBadArgument);
@@ -158,6 +177,16 @@ __device__ __forceinline__ void wg_fcollect_bytes(int my_pe, void *dest, const v
                                                   size_t block_bytes, size_t shard_begin,
                                                   size_t shard_end, int pe_start, int log_stride,
                                                   int pe_size, long *psync) {
+  my_pe = uniform(my_pe);
+  dest = uniform(dest);
+  source = uniform(source);
+  block_bytes = uniform(block_bytes);
+  shard_begin = uniform(shard_begin);
+  shard_end = uniform(shard_end);
+  pe_start = uniform(pe_start);
+  log_stride = uniform(log_stride);
+  pe_size = uniform(pe_size);
+  psync = uniform(psync);
   if (block_bytes == 0) return;
   if (pe_size > kMaxPes || pe_size <= 0) {
     status_raise(kStatusBadArgument);
@@ -181,6 +210,11 @@ __device__ __forceinline__ void wg_fcollect_bytes(int my_pe, void *dest, const v
 // context_ib_device_coll.cpp:67-89).
 __device__ __forceinline__ void wg_sync_members(int my_pe, int pe_start, int log_stride,
                                                 int pe_size, long *psync) {
+  my_pe = uniform(my_pe);
+  pe_start = uniform(pe_start);
+  log_stride = uniform(log_stride);
+  pe_size = uniform(pe_size);
+  psync = uniform(psync);
   if (pe_size > kMaxPes || pe_size <= 0) {
     status_raise(kStatusBadArgument);
     return;

@@ -135,12 +135,13 @@ __device__ __forceinline__ void group_copy(void *dst, const void *src, size_t n,
 }
 
 __device__ __forceinline__ void wg_copy(void *dst, const void *src, size_t n) {
-  group_copy(dst, src, n, flat_thread_id(), flat_block_size());
+  // Workgroup-collective: the arguments are the same in every lane.
+  group_copy(uniform(dst), uniform(src), uniform(n), flat_thread_id(), flat_block_size());
 }
 
 __device__ __forceinline__ void wave_copy(void *dst, const void *src, size_t n) {
   // All lanes of the calling wave take part (wave-collective call).
-  group_copy(dst, src, n, lane_id(), kWaveSize);
+  group_copy(uniform(dst), uniform(src), uniform(n), lane_id(), kWaveSize);
 }
 
 // Single-lane copy used by the thread-level put/get: the common 4- and 8-byte

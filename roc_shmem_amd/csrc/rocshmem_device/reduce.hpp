@@ -128,8 +128,8 @@ struct VecOf {
   };
 };
 
-constexpr int kReduceUnroll = 2;   // vectors per lane per pass
-constexpr int kReducePeChunk = 4;  // members whose loads are issued together
+constexpr int kReduceUnroll = 8;   // vectors per lane per pass
+constexpr int kReducePeChunk = 1;  // members whose loads are issued together
 
 struct ActiveSet {
   int pe_start;
@@ -141,40 +141,55 @@ struct ActiveSet {
 // Reduce vectors [v_begin, v_end) of the symmetric arrays `src`/`dst` (given
 // as this PE's addresses, both 16-byte aligned) over all members and write
 // the result into every member's destination.
-template <typename T, ROC_SHMEM_OP Op>
+//
+// One pass of the workgroup covers U*nthr consecutive vectors of every
+// member: access u of lane t is vector u*nthr + t of the pass, so each
+// load/store instruction of the workgroup sweeps nthr*16 consecutive bytes
+// and the U accesses of one member follow each other through U*nthr*16
+// consecutive bytes (128 KiB for 1024 lanes and U = 8).  Measured on MI355X
+// (8 slices x 256 MiB): 32 KiB per member per pass reaches 5.2 TB/s, 128 KiB
+// 5.8 TB/s; dealing the same bytes to waves as private 8 KiB chunks instead
+// (every instruction of the workgroup then touches sixteen separate 1 KiB
+// pieces) drops to 4.9 TB/s.
+//
+// Memory is addressed through raw buffer descriptors: the pass base of each
+// member is workgroup-uniform and lives in scalar registers (descriptor +
+// scalar offset), the only per-lane address part is the 32-bit `tid*16`.
+// Besides freeing some thirty vector registers of 64-bit addresses, the
+// descriptor's size field makes the last, partial pass safe without a
+// separate loop: accesses past `valid` bytes load zeros and store nothing.
+template <typename T, ROC_SHMEM_OP Op, int U = kReduceUnroll, int C = kReducePeChunk>
 __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_begin,
                                                size_t v_end, const ActiveSet &as, int my_pe,
                                                uint32_t tid, uint32_t nthr) {
   using Acc = typename AccOf<T, Op>::type;
   using V = VecOf<T>;
   constexpr int E = V::kElems;
-  constexpr int U = kReduceUnroll;
-  constexpr int C = kReducePeChunk;
+  constexpr int kRawBufferFlags = 0x00020000;  // untyped 32-bit data, no swizzle
+  constexpr int kNt = 2;                       // cache policy: non-temporal
 
   const int64_t stride = static_cast<int64_t>(g_state.slice_stride);
-  const char *src0 = reinterpret_cast<const char *>(src) +
-                     (static_cast<int64_t>(as.pe_start) - my_pe) * stride;
+  char *src0 = const_cast<char *>(reinterpret_cast<const char *>(src)) +
+               (static_cast<int64_t>(as.pe_start) - my_pe) * stride;
   char *dst0 =
       reinterpret_cast<char *>(dst) + (static_cast<int64_t>(as.pe_start) - my_pe) * stride;
   const int64_t member_step = stride << as.log_stride;
 
-  auto src_vec = [&](int k) {
-    return reinterpret_cast<const u32x4 *>(src0 + k * member_step);
-  };
-  auto dst_vec = [&](int k) { return reinterpret_cast<u32x4 *>(dst0 + k * member_step); };
+  const uint32_t lane_off = tid * 16u;
+  const uint32_t access_bytes = nthr * 16u;       // bytes one instruction of the workgroup sweeps
+  const uint32_t pass_bytes = access_bytes * U;   // at most 128 KiB
+  const size_t byte_end = v_end * 16;
 
-  size_t i = v_begin + tid;
-  const size_t step = nthr;
-
-  // Full passes: U vectors per lane.
-  for (; i + (U - 1) * step < v_end; i += U * step) {
+  for (size_t b = v_begin * 16; b < byte_end; b += pass_bytes) {
+    const size_t left = byte_end - b;
+    const int valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
     Acc acc[U][E];
     {
-      const u32x4 *s = src_vec(0);
+      __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(src0 + b, 0, valid, kRawBufferFlags);
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         typename V::Pack p;
-        p.raw = __builtin_nontemporal_load(&s[i + u * step]);
+        p.raw = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * access_bytes, kNt);
 #pragma unroll
         for (int e = 0; e < E; ++e) acc[u][e] = to_acc<T, Acc>(p.e[e]);
       }
@@ -184,9 +199,11 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
       typename V::Pack p[C][U];
 #pragma unroll
       for (int c = 0; c < C; ++c) {
-        const u32x4 *s = src_vec(k + c);
+        __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            src0 + (k + c) * member_step + b, 0, valid, kRawBufferFlags);
 #pragma unroll
-        for (int u = 0; u < U; ++u) p[c][u].raw = __builtin_nontemporal_load(&s[i + u * step]);
+        for (int u = 0; u < U; ++u)
+          p[c][u].raw = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * access_bytes, kNt);
       }
 #pragma unroll
       for (int c = 0; c < C; ++c)
@@ -197,10 +214,12 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
             acc[u][e] = fold<Op, Acc>(acc[u][e], to_acc<T, Acc>(p[c][u].e[e]));
     }
     for (; k < as.size; ++k) {
-      const u32x4 *s = src_vec(k);
+      __amdgpu_buffer_rsrc_t rs =
+          __builtin_amdgcn_make_buffer_rsrc(src0 + k * member_step + b, 0, valid, kRawBufferFlags);
       typename V::Pack p[U];
 #pragma unroll
-      for (int u = 0; u < U; ++u) p[u].raw = __builtin_nontemporal_load(&s[i + u * step]);
+      for (int u = 0; u < U; ++u)
+        p[u].raw = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * access_bytes, kNt);
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -212,30 +231,12 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
 #pragma unroll
       for (int e = 0; e < E; ++e) out[u].e[e] = from_acc<T, Acc>(acc[u][e]);
     for (int m = 0; m < as.size; ++m) {
-      u32x4 *d = dst_vec(m);
+      __amdgpu_buffer_rsrc_t rd =
+          __builtin_amdgcn_make_buffer_rsrc(dst0 + m * member_step + b, 0, valid, kRawBufferFlags);
 #pragma unroll
-      for (int u = 0; u < U; ++u) __builtin_nontemporal_store(out[u].raw, &d[i + u * step]);
+      for (int u = 0; u < U; ++u)
+        __builtin_amdgcn_raw_buffer_store_b128(out[u].raw, rd, lane_off, u * access_bytes, kNt);
     }
-  }
-  // Remainder: one vector per lane.
-  for (; i < v_end; i += step) {
-    Acc acc[E];
-    {
-      typename V::Pack p;
-      p.raw = __builtin_nontemporal_load(&src_vec(0)[i]);
-#pragma unroll
-      for (int e = 0; e < E; ++e) acc[e] = to_acc<T, Acc>(p.e[e]);
-    }
-    for (int k = 1; k < as.size; ++k) {
-      typename V::Pack p;
-      p.raw = __builtin_nontemporal_load(&src_vec(k)[i]);
-#pragma unroll
-      for (int e = 0; e < E; ++e) acc[e] = fold<Op, Acc>(acc[e], to_acc<T, Acc>(p.e[e]));
-    }
-    typename V::Pack out;
-#pragma unroll
-    for (int e = 0; e < E; ++e) out.e[e] = from_acc<T, Acc>(acc[e]);
-    for (int m = 0; m < as.size; ++m) __builtin_nontemporal_store(out.raw, &dst_vec(m)[i]);
   }
 }
 
@@ -275,6 +276,15 @@ template <typename T, ROC_SHMEM_OP Op>
 __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *source, int nreduce,
                                               int pe_start, int log_stride, int pe_size,
                                               long *psync) {
+  // Workgroup-collective: every lane holds the same arguments.
+  my_pe = uniform(my_pe);
+  dest = uniform(dest);
+  source = uniform(source);
+  nreduce = uniform(nreduce);
+  pe_start = uniform(pe_start);
+  log_stride = uniform(log_stride);
+  pe_size = uniform(pe_size);
+  psync = uniform(psync);
   if (nreduce <= 0) return;  // reference: Context::to_all early-out, context_tmpl_device.hpp:68-70
   if (pe_size > kMaxPes || pe_size <= 0) {
     status_raise(kStatusBadArgument);

@@ -102,26 +102,36 @@ __device__ __forceinline__ bool bounded_wait(const T *ptr, int cmp, T want) {
 // other set has completed in between.
 //
 // Must be called by every thread of the workgroup.
+//
+// Fences are issued by the few lanes that handle flags, not by every wave:
+// the workgroup barrier in front guarantees that all the workgroup's stores
+// have left for L2 (s_waitcnt before s_barrier), so one L2 write-back covers
+// them, and one invalidate of this CU's L1 and this XCD's L2 before the
+// closing workgroup barrier covers every wave that resumes after it.  With a
+// fence per wave, 256 workgroups of 16 waves spent 31 us in one barrier
+// (each fence walks a whole L2); the flag lanes alone need a fraction of it.
 __device__ __forceinline__ void wg_flag_barrier(long *psync, int set, int my_pe, int my_idx,
                                                 int pe_start, int log_stride, int n_pes) {
   __syncthreads();
   const uint32_t tid = flat_thread_id();
   const uint32_t nthr = flat_block_size();
-  if (tid < static_cast<uint32_t>(n_pes)) fence_release_agent();
-  for (uint32_t t = tid; t < static_cast<uint32_t>(n_pes); t += nthr) {
-    int peer = pe_start + (static_cast<int>(t) << log_stride);
-    unsigned long long *slot = reinterpret_cast<unsigned long long *>(
-        translate(psync, my_pe, peer) + set * n_pes + my_idx);
-    __hip_atomic_store(slot, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  for (uint32_t t = tid; t < static_cast<uint32_t>(n_pes); t += nthr) {
-    unsigned long long *mine =
-        reinterpret_cast<unsigned long long *>(psync + set * n_pes + static_cast<int>(t));
-    bounded_wait<unsigned long long>(mine, kWaitEq, 1ull);
-    __hip_atomic_store(mine, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (tid < static_cast<uint32_t>(n_pes)) {
+    fence_release_agent();
+    for (uint32_t t = tid; t < static_cast<uint32_t>(n_pes); t += nthr) {
+      int peer = pe_start + (static_cast<int>(t) << log_stride);
+      unsigned long long *slot = reinterpret_cast<unsigned long long *>(
+          translate(psync, my_pe, peer) + set * n_pes + my_idx);
+      __hip_atomic_store(slot, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    for (uint32_t t = tid; t < static_cast<uint32_t>(n_pes); t += nthr) {
+      unsigned long long *mine =
+          reinterpret_cast<unsigned long long *>(psync + set * n_pes + static_cast<int>(t));
+      bounded_wait<unsigned long long>(mine, kWaitEq, 1ull);
+      __hip_atomic_store(mine, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    fence_acquire_agent();
   }
   __syncthreads();
-  fence_acquire_agent();
 }
 
 }  // namespace detail

@@ -38,6 +38,27 @@ __device__ __forceinline__ uint64_t first_lane_u64(uint64_t v) {
   return (static_cast<uint64_t>(hi) << 32) | lo;
 }
 
+// Workgroup- and wave-collective calls receive the same arguments in every
+// lane.  Passing such a value through v_readfirstlane tells the compiler so:
+// address arithmetic built on it stays in scalar registers and memory
+// instructions can take a scalar base, instead of every lane carrying a
+// 64-bit address (a context handle read back from LDS, for one, is a vector
+// value to the compiler even though all lanes hold the same pointer).
+__device__ __forceinline__ uint32_t uniform(uint32_t v) { return first_lane_u32(v); }
+__device__ __forceinline__ int uniform(int v) {
+  return static_cast<int>(first_lane_u32(static_cast<uint32_t>(v)));
+}
+__device__ __forceinline__ unsigned long uniform(unsigned long v) {
+  return static_cast<unsigned long>(first_lane_u64(static_cast<uint64_t>(v)));
+}
+__device__ __forceinline__ unsigned long long uniform(unsigned long long v) {
+  return static_cast<unsigned long long>(first_lane_u64(static_cast<uint64_t>(v)));
+}
+template <typename T>
+__device__ __forceinline__ T *uniform(T *p) {
+  return reinterpret_cast<T *>(first_lane_u64(reinterpret_cast<uint64_t>(p)));
+}
+
 // Value of `v` in lane-1 through DPP wave_shr:1.  A lane whose lower
 // neighbour is inactive (or lane 0) keeps its own value.
 __device__ __forceinline__ uint32_t from_lower_lane(uint32_t v) {
