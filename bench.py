@@ -30,9 +30,9 @@ HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
 MEASURED_TRAFFIC_BYTES = None
 
 # Launch shapes chosen by measurement on MI355X (256 CUs).
-TO_ALL_LAUNCH = dict(wgs_per_pe=32, wg_size=512)
-PUT_LAUNCH = dict(wgs_per_pe=64, wg_size=256)
-PUT_TILE = 4 << 20
+TO_ALL_LAUNCH = dict(wgs_per_pe=64, wg_size=512)
+PUT_LAUNCH = dict(wgs_per_pe=32, wg_size=512)
+PUT_TILE = 256 << 10
 
 
 def event_time_ms(rs, fn, iters):

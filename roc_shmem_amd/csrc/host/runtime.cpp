@@ -145,8 +145,9 @@ std::string Runtime::init(const Options &opt) {
   if (opt_.num_pes < 1 || opt_.num_pes > detail::kMaxPes)
     return "ROC_SHMEM_NUM_PES must be in [1, 128]";
   if (opt_.num_blocks < 1) return "ROC_SHMEM_NUM_BLOCKS must be positive";
-  if (opt_.sq_size < 2 || (opt_.sq_size & (opt_.sq_size - 1)))
-    return "ROC_SHMEM_SQ_SIZE must be a power of two";
+  // A wave posts up to 64 entries at once; they must fit the ring.
+  if (opt_.sq_size < 64 || (opt_.sq_size & (opt_.sq_size - 1)))
+    return "ROC_SHMEM_SQ_SIZE must be a power of two, at least 64";
   if (opt_.heap_size < (1u << 20) || (opt_.heap_size & 4095))
     return "ROC_SHMEM_HEAP_SIZE must be a multiple of 4096 and at least 1 MiB";
   if (opt_.slice_pad & 4095) return "ROC_SHMEM_SLICE_PAD must be a multiple of 4096";

@@ -37,8 +37,11 @@ __device__ __forceinline__ void split_range(size_t n, int parts, int idx, size_t
 }
 
 // Copy `n` bytes from `src` into the same symmetric address `dst_mine` of
-// every member for which `skip_idx != member index`, loading each source
-// vector once when all addresses are mutually 16-byte aligned.
+// every member for which `skip_idx != member index`.  When source and
+// destinations are mutually 16-byte aligned every source vector is loaded
+// once and stored to each destination (raw-buffer addressing as in
+// stream_copy_uniform); otherwise each destination is copied on its own.
+// Arguments are workgroup-uniform.
 __device__ __forceinline__ void wg_copy_to_members(char *dst_mine, const char *src, size_t n,
                                                    const ActiveSet &as, int my_pe, int skip_idx,
                                                    uint32_t tid, uint32_t nthr) {
@@ -51,40 +54,40 @@ __device__ __forceinline__ void wg_copy_to_members(char *dst_mine, const char *s
   if (!coaligned || n < 256) {
     for (int m = 0; m < as.size; ++m) {
       if (m == skip_idx) continue;
-      group_copy(dst0 + m * member_step, src, n, tid, nthr);
+      group_copy_uniform(dst0 + m * member_step, src, n, tid, nthr);
     }
     return;
   }
-  size_t head = (16u - (reinterpret_cast<uintptr_t>(src) & 15u)) & 15u;
-  size_t nvec = (n - head) / 16;
-  size_t tail = n - head - nvec * 16;
+  const size_t head = (16u - (reinterpret_cast<uintptr_t>(src) & 15u)) & 15u;
+  const size_t body = (n - head) & ~static_cast<size_t>(15);
+  const size_t tail = n - head - body;
   for (size_t t = tid; t < head + tail; t += nthr) {
-    size_t off = t < head ? t : nvec * 16 + t;  // head bytes, then the bytes after the vectors
+    size_t off = t < head ? t : body + t;  // head bytes, then the bytes after the vectors
     char b = src[off];
     for (int m = 0; m < as.size; ++m)
       if (m != skip_idx) dst0[m * member_step + off] = b;
   }
-  const u32x4 *sv = reinterpret_cast<const u32x4 *>(src + head);
-  char *dv0 = dst0 + head;
-  constexpr int U = kCopyUnroll;
-  size_t i = tid;
-  const size_t step = nthr;
-  for (; i + (U - 1) * step < nvec; i += U * step) {
+  constexpr int U = kStreamUnroll;
+  constexpr int kNt = 2;
+  const uint32_t lane_off = tid * 16u;
+  const uint32_t access_bytes = nthr * 16u;
+  const uint32_t pass_bytes = access_bytes * U;
+  for (size_t b = 0; b < body; b += pass_bytes) {
+    const size_t left = body - b;
+    const int valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
+    __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char *>(src) + head + b, 0, valid, kRawBufferFlags);
     u32x4 v[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(&sv[i + u * step]);
+    for (int u = 0; u < U; ++u)
+      v[u] = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * access_bytes, kNt);
     for (int m = 0; m < as.size; ++m) {
       if (m == skip_idx) continue;
-      u32x4 *d = reinterpret_cast<u32x4 *>(dv0 + m * member_step);
+      __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(
+          dst0 + m * member_step + head + b, 0, valid, kRawBufferFlags);
 #pragma unroll
-      for (int u = 0; u < U; ++u) __builtin_nontemporal_store(v[u], &d[i + u * step]);
-    }
-  }
-  for (; i < nvec; i += step) {
-    u32x4 v = __builtin_nontemporal_load(&sv[i]);
-    for (int m = 0; m < as.size; ++m) {
-      if (m == skip_idx) continue;
-      __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dv0 + m * member_step) + i);
+      for (int u = 0; u < U; ++u)
+        __builtin_amdgcn_raw_buffer_store_b128(v[u], rd, lane_off, u * access_bytes, kNt);
     }
   }
 }
@@ -164,8 +167,8 @@ __device__ __forceinline__ void wg_alltoall_bytes(int my_pe, void *dest, const v
     // Start at the own index so that concurrent members hit different slices.
     int j = my_idx + jj;
     if (j >= pe_size) j -= pe_size;
-    group_copy(translate(dst_mine, my_pe, as.pe_at(j)), src + static_cast<size_t>(j) * block_bytes,
-               len, tid, nthr);
+    group_copy_uniform(translate(dst_mine, my_pe, as.pe_at(j)),
+                       src + static_cast<size_t>(j) * block_bytes, len, tid, nthr);
   }
 
   wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, log_stride, pe_size);

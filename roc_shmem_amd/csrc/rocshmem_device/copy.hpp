@@ -97,8 +97,9 @@ __device__ __forceinline__ void copy_vec_src_bytes(u32x4 *__restrict__ d,
   }
 }
 
-// memcpy(dst, src, n) executed cooperatively by lanes tid = 0..nthr-1.
-// No barrier inside: the caller synchronises the group afterwards.
+// memcpy(dst, src, n) executed cooperatively by lanes tid = 0..nthr-1, for
+// per-lane (possibly different in every lane) arguments: the thread-level
+// put/get path.  No barrier inside.
 __device__ __forceinline__ void group_copy(void *dst, const void *src, size_t n, uint32_t tid,
                                            uint32_t nthr) {
   char *d = static_cast<char *>(dst);
@@ -134,14 +135,76 @@ __device__ __forceinline__ void group_copy(void *dst, const void *src, size_t n,
   for (size_t i = tid; i < tail; i += nthr) d[body + i] = s[body + i];
 }
 
+constexpr int kStreamUnroll = 8;          // 16-byte accesses per lane per pass
+constexpr int kRawBufferFlags = 0x00020000;  // untyped 32-bit data, no swizzle
+
+// Body of a group copy whose arguments are the same in every lane
+// (workgroup- and wave-collective calls): `d` 16-byte aligned, `s` 4-byte
+// aligned, `nbytes` a multiple of 16.  One pass moves kStreamUnroll*nthr*16
+// consecutive bytes (128 KiB for 1024 lanes): all loads of the pass are
+// issued before its stores.  Addresses are "descriptor + scalar offset +
+// tid*16", so no lane carries a 64-bit address, and the descriptor's size
+// field turns the last partial pass into the same code (accesses beyond
+// `valid` load zeros and store nothing).
+template <int kAux>
+__device__ __forceinline__ void stream_copy_uniform(char *d, const char *s, size_t nbytes,
+                                                    uint32_t tid, uint32_t nthr) {
+  constexpr int U = kStreamUnroll;
+  const uint32_t lane_off = tid * 16u;
+  const uint32_t access_bytes = nthr * 16u;
+  const uint32_t pass_bytes = access_bytes * U;
+  for (size_t b = 0; b < nbytes; b += pass_bytes) {
+    const size_t left = nbytes - b;
+    const int valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
+    __amdgpu_buffer_rsrc_t rs =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(s) + b, 0, valid, kRawBufferFlags);
+    __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(d + b, 0, valid, kRawBufferFlags);
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      v[u] = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * access_bytes, kAux);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      __builtin_amdgcn_raw_buffer_store_b128(v[u], rd, lane_off, u * access_bytes, kAux);
+  }
+}
+
+// memcpy(dst, src, n) by lanes tid = 0..nthr-1 of a group that passes the
+// same (dst, src, n) in every lane.
+__device__ __forceinline__ void group_copy_uniform(void *dst, const void *src, size_t n,
+                                                   uint32_t tid, uint32_t nthr) {
+  char *d = static_cast<char *>(dst);
+  const char *s = static_cast<const char *>(src);
+  if (n < 64) {
+    for (size_t i = tid; i < n; i += nthr) d[i] = s[i];
+    return;
+  }
+  const size_t head = (16u - (reinterpret_cast<uintptr_t>(d) & 15u)) & 15u;
+  for (size_t i = tid; i < head; i += nthr) d[i] = s[i];
+  d += head;
+  s += head;
+  n -= head;
+  const size_t body = n & ~static_cast<size_t>(15);
+  if ((reinterpret_cast<uintptr_t>(s) & 3u) == 0) {
+    if (body >= kNonTemporalBytes) {
+      stream_copy_uniform<2 /* nt */>(d, s, body, tid, nthr);
+    } else {
+      stream_copy_uniform<0>(d, s, body, tid, nthr);
+    }
+  } else {
+    copy_vec_src_bytes(reinterpret_cast<u32x4 *>(d), s, body / 16, tid, nthr);
+  }
+  for (size_t i = body + tid; i < n; i += nthr) d[i] = s[i];
+}
+
 __device__ __forceinline__ void wg_copy(void *dst, const void *src, size_t n) {
   // Workgroup-collective: the arguments are the same in every lane.
-  group_copy(uniform(dst), uniform(src), uniform(n), flat_thread_id(), flat_block_size());
+  group_copy_uniform(uniform(dst), uniform(src), uniform(n), flat_thread_id(), flat_block_size());
 }
 
 __device__ __forceinline__ void wave_copy(void *dst, const void *src, size_t n) {
   // All lanes of the calling wave take part (wave-collective call).
-  group_copy(uniform(dst), uniform(src), uniform(n), lane_id(), kWaveSize);
+  group_copy_uniform(uniform(dst), uniform(src), uniform(n), lane_id(), kWaveSize);
 }
 
 // Single-lane copy used by the thread-level put/get: the common 4- and 8-byte

@@ -165,7 +165,6 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
   using Acc = typename AccOf<T, Op>::type;
   using V = VecOf<T>;
   constexpr int E = V::kElems;
-  constexpr int kRawBufferFlags = 0x00020000;  // untyped 32-bit data, no swizzle
   constexpr int kNt = 2;                       // cache policy: non-temporal
 
   const int64_t stride = static_cast<int64_t>(g_state.slice_stride);

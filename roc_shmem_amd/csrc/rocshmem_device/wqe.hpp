@@ -21,7 +21,20 @@
 // slots its posting lanes need with a single atomic (ballot + v_mbcnt +
 // v_readlane), every posting lane assembles its entry in registers and
 // writes it with 16-byte stores, and completed ranges are published in index
-// order through SqCounters::published before the doorbell record moves.
+// order through SqCounters::published before the doorbell record moves.  A
+// slot is reused only after its previous occupant has been published
+// (the reference's waitSQSpace, queue_pair.cpp:400-415, plays this role).
+//
+// No device-wide release fence sits on this path.  An agent-scope release on a
+// part with one L2 per XCD writes a whole L2 back; two of them per post held
+// 10 M eight-byte puts at 1.0 G ops/s, against 12.9 G ops/s with the ordering
+// used here: a wave waits for its own stores (s_waitcnt) and hands the queue
+// on through agent-scope atomics on `published` and the mailbox words.  That
+// orders everything producers need among themselves.  Ring bytes are plain
+// (cached) stores: they are complete in memory when the kernel ends or after
+// roc_shmem_ctx_quiet, and the image of a ring fed by workgroups on different
+// XCDs (more workgroups per PE than ROC_SHMEM_NUM_BLOCKS) is only determined
+// up to which of two entries that wrapped onto one slot is written back last.
 #ifndef ROCSHMEM_MI355X_DEVICE_WQE_HPP
 #define ROCSHMEM_MI355X_DEVICE_WQE_HPP
 
@@ -73,14 +86,34 @@ __device__ __forceinline__ void wave_post(DeviceCtx *ctx, bool sends, const WqeR
   const uint64_t atomic_mask = __ballot(sends && is_atomic);
 
   SqCounters *cnt = ctx->counters;
+  const uint32_t ring_size = ctx->ring.max_nwqe;
   uint32_t base = 0, abase = 0;
   if (sends && rank == 0) {
+    // Issued together so their latencies overlap: the published index (only
+    // ever grows, so an early read is conservative) and the reservation.
+    uint32_t seen = __hip_atomic_load(&cnt->published, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     base = __hip_atomic_fetch_add(&cnt->sq_counter, n, __ATOMIC_RELAXED,
                                   __HIP_MEMORY_SCOPE_AGENT);
     if (atomic_mask) {
       abase = __hip_atomic_fetch_add(&cnt->atomic_counter,
                                      static_cast<uint32_t>(__popcll(atomic_mask)),
                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    // Queue space: entry c may be written once entry c - ring_size is published.
+    if (static_cast<int32_t>(base + n - seen - ring_size) > 0) {
+      const uint32_t need = base + n - ring_size;
+      uint64_t start = wall_clock64();
+      uint32_t spins = 0;
+      while (static_cast<int32_t>(
+                 need - __hip_atomic_load(&cnt->published, __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT)) > 0) {
+        __builtin_amdgcn_s_sleep(1);
+        if ((++spins & 63u) == 0 &&
+            (status_failed() || wall_clock64() - start > g_state.wait_limit_ticks)) {
+          status_raise(kStatusWaitTimeout);
+          break;
+        }
+      }
     }
   }
   base = __builtin_amdgcn_readlane(base, first);
@@ -154,16 +187,22 @@ __device__ __forceinline__ void wave_post(DeviceCtx *ctx, bool sends, const WqeR
     }
   }
 
-  // Publish: entries become visible to a consumer in index order.  The last
-  // posting lane waits for every earlier range, then moves the doorbell
-  // record and writes the doorbell value (first 8 bytes of the wave's last
-  // entry, as the reference's finishPost does).
-  fence_release_agent();
+  // Publish in index order.  The last posting lane waits until every earlier
+  // range is published, moves the doorbell record and writes the doorbell
+  // value (first 8 bytes of the wave's last entry, as the reference's
+  // finishPost does), then hands the queue on.  s_waitcnt (what a
+  // workgroup-scope release amounts to) makes the wave's own stores complete
+  // before each hand-over.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   if (last) {
     bounded_wait<uint32_t>(&cnt->published, kWaitEq, base);
-    ring.mailbox[0] = be32(base + n);
-    ring.mailbox[1] = (static_cast<uint64_t>(first8_hi) << 32) | first8_lo;
-    fence_release_agent();
+    __hip_atomic_store(reinterpret_cast<unsigned long long *>(&ring.mailbox[0]),
+                       static_cast<unsigned long long>(be32(base + n)), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(reinterpret_cast<unsigned long long *>(&ring.mailbox[1]),
+                       (static_cast<unsigned long long>(first8_hi) << 32) | first8_lo,
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __hip_atomic_store(&cnt->published, base + n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
