@@ -24,10 +24,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
 
-# HBM bytes per launch of the headline kernel measured with rocprofv3 --pmc
-# (FETCH_SIZE and WRITE_SIZE, scaled by a copy kernel of known size); see
-# profiles/.  None until measured.
-MEASURED_TRAFFIC_BYTES = None
+# HBM bytes per launch of the headline kernel measured with rocprofv3 --pmc:
+# FETCH_SIZE 1 048 914.8 KiB and WRITE_SIZE 2 099 013.0 KiB per dispatch, each scaled by
+# what the same counter reads for a wg-putmem copy of known size (2 GiB read, 2 GiB
+# written: 1 048 669.0 and 2 097 724.2 KiB); see profiles/to_all_float_sum_8pe_2e26.md.
+MEASURED_TRAFFIC_BYTES = 4296790021
 
 # Launch shapes chosen by measurement on MI355X (256 CUs).
 TO_ALL_LAUNCH = dict(wgs_per_pe=64, wg_size=512)
@@ -136,7 +137,8 @@ def bench_putmem(rs, steps, n_pes, msg_bytes_list):
         else:
             tile, n_msgs = m, min(total // max(m, 256), 1 << 16)
         stride = max(tile, 256)
-        launch = rs.Launch(**PUT_LAUNCH)
+        # a few large workgroups stream best; short messages want many small ones
+        launch = rs.Launch(**PUT_LAUNCH) if tile >= (64 << 10) else rs.Launch(64, 256)
 
         def step():
             rs.roc_shmem_rma(rs.PUT, rs.WG, dst, src, tile, n_msgs, stride, stride, 1, launch)
