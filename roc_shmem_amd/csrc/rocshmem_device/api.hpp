@@ -232,26 +232,26 @@ __device__ inline void roc_shmemx_ctx_putmem_nbi_wg(roc_shmem_ctx_t ctx, void *d
   if (nelems == 0) return;
   const detail::DeviceCtx *c = detail::ctx_of(ctx);
   detail::wg_copy(detail::translate(dest, c->my_pe, pe), source, nelems);
-  __syncthreads();
 }
 __device__ inline void roc_shmemx_ctx_putmem_wg(roc_shmem_ctx_t ctx, void *dest,
                                                 const void *source, size_t nelems, int pe) {
-  // Same data movement as the non-blocking form: the lanes' own loads have
-  // returned before their stores issue, so the source is reusable on return.
+  // The source is reusable on return: a lane's loads have returned before its
+  // stores issue, and the lanes meet once all have issued theirs.  Nobody
+  // waits for the stores themselves.
   roc_shmemx_ctx_putmem_nbi_wg(ctx, dest, source, nelems, pe);
+  if (nelems != 0) detail::wg_rendezvous();
 }
 __device__ inline void roc_shmemx_ctx_getmem_nbi_wg(roc_shmem_ctx_t ctx, void *dest,
                                                     const void *source, size_t nelems, int pe) {
   if (nelems == 0) return;
   const detail::DeviceCtx *c = detail::ctx_of(ctx);
   detail::wg_copy(dest, detail::translate(source, c->my_pe, pe), nelems);
-  __syncthreads();
 }
 __device__ inline void roc_shmemx_ctx_getmem_wg(roc_shmem_ctx_t ctx, void *dest,
                                                 const void *source, size_t nelems, int pe) {
-  // Same data movement as the non-blocking form: the lanes' own loads have
-  // returned before their stores issue, so the source is reusable on return.
+  // Every lane of the workgroup may read any byte of `dest` on return.
   roc_shmemx_ctx_getmem_nbi_wg(ctx, dest, source, nelems, pe);
+  if (nelems != 0) __syncthreads();
 }
 __device__ inline void roc_shmemx_ctx_putmem_nbi_wave(roc_shmem_ctx_t ctx, void *dest,
                                                       const void *source, size_t nelems,
@@ -275,8 +275,8 @@ __device__ inline void roc_shmemx_ctx_getmem_nbi_wave(roc_shmem_ctx_t ctx, void 
 }
 __device__ inline void roc_shmemx_ctx_getmem_wave(roc_shmem_ctx_t ctx, void *dest,
                                                   const void *source, size_t nelems, int pe) {
-  // Same data movement as the non-blocking form: the lanes' own loads have
-  // returned before their stores issue, so the source is reusable on return.
+  // Same data movement as the non-blocking form: the wave's later loads of
+  // `dest` follow its stores through the same vector memory pipeline.
   roc_shmemx_ctx_getmem_nbi_wave(ctx, dest, source, nelems, pe);
 }
 

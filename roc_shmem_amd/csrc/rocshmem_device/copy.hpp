@@ -140,16 +140,15 @@ constexpr int kRawBufferFlags = 0x00020000;  // untyped 32-bit data, no swizzle
 
 // Body of a group copy whose arguments are the same in every lane
 // (workgroup- and wave-collective calls): `d` 16-byte aligned, `s` 4-byte
-// aligned, `nbytes` a multiple of 16.  One pass moves kStreamUnroll*nthr*16
-// consecutive bytes (128 KiB for 1024 lanes): all loads of the pass are
+// aligned, `nbytes` a multiple of 16.  One pass moves U*nthr*16
+// consecutive bytes (128 KiB for 1024 lanes and U = 8): all loads of the pass are
 // issued before its stores.  Addresses are "descriptor + scalar offset +
 // tid*16", so no lane carries a 64-bit address, and the descriptor's size
 // field turns the last partial pass into the same code (accesses beyond
 // `valid` load zeros and store nothing).
-template <int kAux>
+template <int kAux, int U>
 __device__ __forceinline__ void stream_copy_uniform(char *d, const char *s, size_t nbytes,
                                                     uint32_t tid, uint32_t nthr) {
-  constexpr int U = kStreamUnroll;
   const uint32_t lane_off = tid * 16u;
   const uint32_t access_bytes = nthr * 16u;
   const uint32_t pass_bytes = access_bytes * U;
@@ -166,6 +165,25 @@ __device__ __forceinline__ void stream_copy_uniform(char *d, const char *s, size
 #pragma unroll
     for (int u = 0; u < U; ++u)
       __builtin_amdgcn_raw_buffer_store_b128(v[u], rd, lane_off, u * access_bytes, kAux);
+  }
+}
+
+// Picks the pass depth by message size, so that a message that one or two
+// accesses of the group cover does not issue eight (six or seven of them
+// entirely out of range).
+__device__ __forceinline__ void stream_copy_sized(char *d, const char *s, size_t nbytes,
+                                                  uint32_t tid, uint32_t nthr) {
+  const size_t access_bytes = static_cast<size_t>(nthr) * 16u;
+  if (nbytes >= kNonTemporalBytes) {
+    stream_copy_uniform<2 /* nt */, kStreamUnroll>(d, s, nbytes, tid, nthr);
+  } else if (nbytes <= access_bytes) {
+    stream_copy_uniform<0, 1>(d, s, nbytes, tid, nthr);
+  } else if (nbytes <= 2 * access_bytes) {
+    stream_copy_uniform<0, 2>(d, s, nbytes, tid, nthr);
+  } else if (nbytes <= 4 * access_bytes) {
+    stream_copy_uniform<0, 4>(d, s, nbytes, tid, nthr);
+  } else {
+    stream_copy_uniform<0, kStreamUnroll>(d, s, nbytes, tid, nthr);
   }
 }
 
@@ -186,11 +204,7 @@ __device__ __forceinline__ void group_copy_uniform(void *dst, const void *src, s
   n -= head;
   const size_t body = n & ~static_cast<size_t>(15);
   if ((reinterpret_cast<uintptr_t>(s) & 3u) == 0) {
-    if (body >= kNonTemporalBytes) {
-      stream_copy_uniform<2 /* nt */>(d, s, body, tid, nthr);
-    } else {
-      stream_copy_uniform<0>(d, s, body, tid, nthr);
-    }
+    stream_copy_sized(d, s, body, tid, nthr);
   } else {
     copy_vec_src_bytes(reinterpret_cast<u32x4 *>(d), s, body / 16, tid, nthr);
   }

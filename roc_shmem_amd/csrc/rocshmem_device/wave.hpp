@@ -59,6 +59,13 @@ __device__ __forceinline__ T *uniform(T *p) {
   return reinterpret_cast<T *>(first_lane_u64(reinterpret_cast<uint64_t>(p)));
 }
 
+// Workgroup barrier without the memory fence of __syncthreads(): the lanes
+// meet, their outstanding stores keep draining.  For points where the lanes
+// only need to know that all of them got here (every lane has consumed what
+// it loaded), not that anybody's stores have landed.  Every lane of the
+// workgroup must reach it.
+__device__ __forceinline__ void wg_rendezvous() { __asm__ volatile("s_barrier" ::: "memory"); }
+
 // Value of `v` in lane-1 through DPP wave_shr:1.  A lane whose lower
 // neighbour is inactive (or lane 0) keeps its own value.
 __device__ __forceinline__ uint32_t from_lower_lane(uint32_t v) {
