@@ -48,7 +48,33 @@ def event_time_ms(rs, fn, iters):
     return ms
 
 
-def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, cpu=False):
+def per_launch_ms(rs, fn, iters):
+    """Duration of each of `iters` launches: an event between every two launches."""
+    marks = [rs.Event() for _ in range(iters + 1)]
+    marks[0].record()
+    for i in range(iters):
+        fn()
+        marks[i + 1].record()
+    out = [marks[i].elapsed_ms(marks[i + 1]) for i in range(iters)]
+    for m in marks:
+        m.destroy()
+    return out
+
+
+def device_report():
+    """Clock and power state of the GPU as rocm-smi prints it (run as a child process)."""
+    import subprocess
+    try:
+        txt = subprocess.run(["rocm-smi", "--showclocks", "--showpower", "--showperflevel"],
+                             capture_output=True, text=True, timeout=30).stdout
+    except Exception as e:  # the tool is optional
+        return {"rocm_smi": "unavailable: %s" % e}
+    keep = [ln.strip() for ln in txt.splitlines() if ln.startswith("GPU[0]")]
+    return {"rocm_smi": keep[:16]}
+
+
+def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, cpu=False,
+                 spread=False):
     """Returns a dict with ms_per_step, GB/s (algorithmic 2*P*N*s bytes) and optional CPU figures."""
     npd = rs.NP_DTYPE[dtype]
     es = np.dtype(npd).itemsize
@@ -81,6 +107,12 @@ def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, c
         raise RuntimeError("device status word raised: %d" % status)
     out = {"ms_per_step": ms / steps, "GBps": 2.0 * n_pes * n * es / (ms / steps) / 1e6,
            "bytes_per_step": 2 * n_pes * n * es}
+    if spread:
+        each = sorted(per_launch_ms(rs, step, steps))
+        rs.synchronize()
+        out["ms_median"] = each[len(each) // 2]
+        out["ms_min"] = each[0]
+        out["ms_max"] = each[-1]
 
     heap = None
     if check or cpu:
@@ -108,17 +140,25 @@ def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, c
         out["parity_checked_elements"] = m
     if cpu:
         cores = min(16, os.cpu_count() or 1)
-        passes = []
-        for _ in range(4):
-            t0 = time.perf_counter()
-            oracle.to_all(heap, dtype, oracle.SUM, n * es, 0, n, threads=cores)
-            passes.append(time.perf_counter() - t0)
-        best = min(passes[1:])
-        out["cpu"] = {"value": 2.0 * n_pes * n * es / best / 1e9, "unit": "GB/s", "cores": cores,
+
+        def cpu_rate(threads, passes):
+            best = None
+            for i in range(passes + 1):          # the first pass warms the pages
+                t0 = time.perf_counter()
+                oracle.to_all(heap, dtype, oracle.SUM, n * es, 0, n, threads=threads)
+                dt = time.perf_counter() - t0
+                if i and (best is None or dt < best):
+                    best = dt
+            return 2.0 * n_pes * n * es / best / 1e9
+
+        out["cpu"] = {"value": cpu_rate(cores, 3), "unit": "GB/s", "cores": cores,
                       "kind": "port",
                       "sample": "same workload, full size (%d slices x 2^%d %s, sum), CPU oracle "
                                 "chunked over %d host threads, best of 3 passes after one warm-up"
-                                % (n_pes, int(np.log2(n)), np.dtype(npd).name, cores)}
+                                % (n_pes, int(np.log2(n)), np.dtype(npd).name, cores),
+                      "one_thread_per_pe": {"value": round(cpu_rate(min(n_pes, cores), 2), 2),
+                                            "cores": min(n_pes, cores)},
+                      "single_thread": {"value": round(cpu_rate(1, 1), 2), "cores": 1}}
     src.free()
     dst.free()
     psync.free()
@@ -223,7 +263,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--quick", action="store_true", help="headline workload only")
     ap.add_argument("--counter-pair", action="store_true",
                     help="for rocprofv3 --pmc: a few launches of the headline kernel and of a "
@@ -237,6 +277,7 @@ def main():
     import oracle
     import roc_shmem_amd as rs
 
+    device = device_report() if not args.counter_pair else {}
     # ---- headline: fp32 sum_to_all, 8 slices x 2^26 elements (4 GiB algorithmic traffic) ----
     n_pes, n = 8, 1 << 26
     rs.roc_shmem_init(n_pes, 1 << 30, 64, 1024)
@@ -247,7 +288,8 @@ def main():
         print(json.dumps({"to_all": out, "putmem_copy": put,
                           "copy_bytes_read": n_pes * (256 << 20), "copy_bytes_written": n_pes * (256 << 20)}))
         return
-    head = bench_to_all(rs, oracle, args.steps, args.warmup, rs.FLOAT, n_pes, n, seed=3, cpu=True)
+    head = bench_to_all(rs, oracle, args.steps, args.warmup, rs.FLOAT, n_pes, n, seed=3, cpu=True,
+                        spread=True)
     extra = {}
     if not args.quick:
         extra["to_all_bf16_sum_8x2^26"] = {k: v for k, v in bench_to_all(
@@ -288,6 +330,9 @@ def main():
                      "unit": "GB/s", "frac": round(head["GBps"] / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES},
         "cpu_baseline": {k: (round(v, 2) if isinstance(v, float) else v) for k, v in cpu.items()},
+        "per_launch_ms": {"median": round(head["ms_median"], 4), "min": round(head["ms_min"], 4),
+                          "max": round(head["ms_max"], 4)},
+        "device": device,
         "extra": extra,
     }
     print(json.dumps(line))

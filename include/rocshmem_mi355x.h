@@ -204,6 +204,42 @@ int rsm_sq_constants(int pe, int block, uint32_t *ctrl_qp_sq, uint64_t *ctrl_sig
                      uint32_t *atomic_lkey, uint64_t *atomic_ret_base, uint32_t *max_nwqe);
 int rsm_sq_rkey(int dest_pe, uint32_t *rkey);
 
+/* ---- consumer pass, completion queues, queue mode -----------------------------------
+ * What a NIC does with the rings in the reference: take published entries off
+ * a ring in order, complete them (reference reader: QueuePair::quiet_internal,
+ * gpu_ib/queue_pair.cpp:118-191) and free their slots (waitSQSpace,
+ * queue_pair.cpp:400-415).  Here a kernel does it, between producer kernels. */
+typedef struct rsm_consume_totals {
+  uint64_t retired;        /* entries taken off the rings                          */
+  uint64_t writes;         /* RDMA WRITE entries, inline or not                    */
+  uint64_t reads;          /* RDMA READ entries                                    */
+  uint64_t atomics;        /* fetch-add and compare-and-swap entries               */
+  uint64_t bytes;          /* payload bytes the entries describe                   */
+  uint64_t completions;    /* completion entries written                           */
+  uint64_t lost;           /* entries overwritten before the pass saw them         */
+  uint64_t rejected;       /* malformed entries: retired, never executed           */
+  uint64_t local_skipped;  /* local buffer outside the symmetric heap: not executed */
+} rsm_consume_totals_t;
+/* Retire what the rings of PE `pe`, block `block` (-1: all) have published.
+ * `target_arena` NULL: check every entry and write completions only.  Otherwise
+ * a device buffer laid out like the arena (rsm_arena): every well-formed entry
+ * is also executed against it, ring by ring in index order - replaying the
+ * rings onto a copy of the arena taken before the producers ran reproduces
+ * what they did (swap / set, recorded as compare-and-swap with compare operand
+ * 0, only where the target held 0).  Payloads of non-inline writes are read
+ * where the producer left them.  Synchronous. */
+int rsm_sq_consume(int pe, int block, void *target_arena, rsm_consume_totals_t *totals);
+/* 0 (default, or ROC_SHMEM_SQ_MODE unset): rings are logs, a slot is reused once
+ * its previous entry is published.  1 (ROC_SHMEM_SQ_MODE=queue): rings are queues,
+ * a slot is reused only after rsm_sq_consume retired it; a producer that finds
+ * its ring full waits (bounded) and raises the status word. */
+int rsm_sq_set_mode(int queue_mode);
+int rsm_sq_consumer_state(int pe, int block, uint32_t *consumed, uint32_t *cq_producer);
+int rsm_cq_image(int pe, int block, void *host_out, size_t bytes);        /* sq_size x 64 B */
+int rsm_atomic_ret_image(int pe, int block, void *host_out, size_t bytes); /* 4096 x 8 B     */
+/* The arena holding every PE slice: PE p's heap starts at base + p*slice_stride. */
+int rsm_arena(void **base, size_t *bytes, size_t *slice_stride);
+
 /* ---- wave-level known-answer drivers ----------------------------------------------
  * Block::fetch_incr contract (containers/share_strategy.hpp:70-83): lanes named
  * by `lane_mask` of every wave of an n_wgs x wg_size grid call the

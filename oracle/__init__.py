@@ -49,6 +49,8 @@ def _load():
     lib.orc_small_ops.argtypes = [vp, sz, vp, vp, sz, vp]
     lib.orc_wqe_build.restype = None
     lib.orc_wqe_build.argtypes = [vp, vp, u32, vp]
+    lib.orc_sq_consume.restype = None
+    lib.orc_sq_consume.argtypes = [vp, vp, u32, u32, vp, vp, vp, vp, vp, u32, vp, vp]
     lib.orc_wqe_index.restype = C.c_uint16
     lib.orc_wqe_index.argtypes = [vp]
     lib.orc_wqe_opcode.restype = C.c_uint8
@@ -86,6 +88,9 @@ NP_DTYPE = {SHORT: np.int16, INT: np.int32, LONG: np.int64, LONGLONG: np.int64,
 
 SMALL_OP_DTYPE = np.dtype([("kind", "<u4"), ("pe", "<u4"), ("offset", "<u8"),
                            ("value", "<i8"), ("aux", "<i8")])
+# Kinds of the small-operation stream (the codes of enum rsm_small_kind).
+(OP_P64, OP_FADD64, OP_ADD64, OP_FINC64, OP_INC64, OP_CSWAP64, OP_FETCH64, OP_SET64, OP_SWAP64,
+ OP_P32, OP_FADD32, OP_PUTMEM, OP_GETMEM, OP_FAND64, OP_FOR64, OP_FXOR64) = range(16)
 
 
 def dtype_size(dtype):
@@ -230,6 +235,39 @@ def wqe_build(slot, qp, sq_counter, opcode, size=0, raddr=0, rkey=0, laddr=0, at
     rq.request_cqe = 1 if request_cqe else 0
     _lib.orc_wqe_build(slot.ctypes.data, C.byref(qp), sq_counter & 0xFFFFFFFF, C.byref(rq))
     return slot
+
+
+class Arena(C.Structure):
+    _fields_ = [("heap_base0", C.c_uint64), ("slice_stride", C.c_uint64), ("heap_size", C.c_uint64),
+                ("num_pes", C.c_int), ("rkeys", C.c_void_p)]
+
+
+class ConsumeTotals(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in ("retired", "writes", "reads", "atomics", "bytes",
+                                          "completions", "lost", "rejected", "local_skipped")]
+
+    def as_dict(self):
+        return {n: int(getattr(self, n)) for n, _ in self._fields_}
+
+
+def sq_consume(qp, ring, consumed, published, heap_base0, slice_stride, heap_size, rkeys, target,
+               sources, atomic_ret, cq, cq_producer=0, totals=None):
+    """Retire entries [consumed, published) of one ring image (uint8, max_nwqe*64) in order.
+
+    ``target`` / ``sources``: uint8 images laid out like the arena (``target`` may be None).
+    ``atomic_ret``: uint64[4096]; ``cq``: uint8 image of the completion queue.  Returns
+    (new cq_producer, ConsumeTotals)."""
+    rk = np.ascontiguousarray(rkeys, dtype=np.uint32)
+    arena = Arena(heap_base0, slice_stride, heap_size, len(rk), rk.ctypes.data)
+    totals = totals if totals is not None else ConsumeTotals()
+    prod = C.c_uint32(cq_producer)
+    assert ring.dtype == np.uint8 and ring.flags["C_CONTIGUOUS"] and ring.size == qp.max_nwqe * 64
+    assert cq.dtype == np.uint8 and cq.size % 64 == 0 and atomic_ret.dtype == np.uint64
+    _lib.orc_sq_consume(C.byref(qp), ring.ctypes.data, consumed & 0xFFFFFFFF, published & 0xFFFFFFFF,
+                        C.byref(arena), None if target is None else target.ctypes.data,
+                        None if sources is None else sources.ctypes.data, atomic_ret.ctypes.data,
+                        cq.ctypes.data, cq.size // 64, C.byref(prod), C.byref(totals))
+    return prod.value, totals
 
 
 def wqe_index(slot):

@@ -101,6 +101,30 @@ typedef struct orc_wqe_req {
 /* Overwrites, inside the 64-byte slot, exactly the bytes the reference writes. */
 void orc_wqe_build(uint8_t slot[64], const orc_qp_t *qp, uint32_t sq_counter,
                    const orc_wqe_req_t *rq);
+/* ---- ring consumer (consume.c) ------------------------------------------------- */
+
+typedef struct orc_arena {
+  uint64_t heap_base0;   /* address of PE 0's heap as the entries name it */
+  uint64_t slice_stride;
+  uint64_t heap_size;
+  int num_pes;
+  const uint32_t *rkeys; /* per destination PE, as stored in the entries */
+} orc_arena_t;
+
+typedef struct orc_consume_totals {
+  uint64_t retired, writes, reads, atomics, bytes, completions, lost, rejected, local_skipped;
+} orc_consume_totals_t;
+
+/* Retires entries [consumed, published) of one ring in order.  `target` (may be
+ * NULL: check and complete only) and `sources` are host images laid out like
+ * the arena: operations are executed on `target`, payloads of non-inline writes
+ * are read from `sources`.  `atomic_ret` is the ring's 4096-word return window,
+ * `cq` its completion queue of `cq_size` 64-byte entries. */
+void orc_sq_consume(const orc_qp_t *qp, const uint8_t *ring, uint32_t consumed, uint32_t published,
+                    const orc_arena_t *arena, uint8_t *target, const uint8_t *sources,
+                    uint64_t *atomic_ret, uint8_t *cq, uint32_t cq_size, uint32_t *cq_producer,
+                    orc_consume_totals_t *totals);
+
 /* Parse helpers used by the ring checker. */
 uint16_t orc_wqe_index(const uint8_t slot[64]);
 uint8_t orc_wqe_opcode(const uint8_t slot[64]);

@@ -63,6 +63,12 @@ SIGNATURES = {
     "rsm_sq_constants": (i32, [i32, i32, C.POINTER(u32), C.POINTER(u64), C.POINTER(u32),
                                C.POINTER(u32), C.POINTER(u64), C.POINTER(u32)]),
     "rsm_sq_rkey": (i32, [i32, C.POINTER(u32)]),
+    "rsm_sq_consume": (i32, [i32, i32, vp, vp]),
+    "rsm_sq_set_mode": (i32, [i32]),
+    "rsm_sq_consumer_state": (i32, [i32, i32, C.POINTER(u32), C.POINTER(u32)]),
+    "rsm_cq_image": (i32, [i32, i32, vp, sz]),
+    "rsm_atomic_ret_image": (i32, [i32, i32, vp, sz]),
+    "rsm_arena": (i32, [C.POINTER(vp), C.POINTER(sz), C.POINTER(sz)]),
     "rsm_kat_fetch_incr": (i32, [u64, i32, i32, vp, C.POINTER(u64)]),
     "rsm_kat_coalesce": (i32, [u64, vp, vp, vp, vp, vp, vp]),
     "rsm_host_alloc_create": (vp, [sz]),

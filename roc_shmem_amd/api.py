@@ -20,6 +20,8 @@ __all__ = [
     "roc_shmem_broadcast", "roc_shmem_team_broadcast", "roc_shmem_alltoall",
     "roc_shmem_fcollect", "roc_shmem_wg_barrier_all", "roc_shmem_small_ops",
     "sq_reset", "sq_read", "sq_image", "sq_state", "sq_constants", "sq_rkey",
+    "sq_consume", "sq_set_mode", "sq_consumer_state", "cq_image", "atomic_ret_image", "arena",
+    "read_device", "write_device",
     "kat_fetch_incr", "kat_coalesce", "take_status", "synchronize", "heap_bytes_in_use",
     "sym_array", "Event", "device_array", "heap_base",
     "SHORT", "INT", "LONG", "LONGLONG", "FLOAT", "DOUBLE", "BF16",
@@ -341,6 +343,66 @@ def sq_rkey(dest_pe):
     k = C.c_uint32(0)
     _check(L.load().rsm_sq_rkey(dest_pe, C.byref(k)))
     return k.value
+
+
+class ConsumeTotals(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in ("retired", "writes", "reads", "atomics", "bytes",
+                                          "completions", "lost", "rejected", "local_skipped")]
+
+    def as_dict(self):
+        return {n: int(getattr(self, n)) for n, _ in self._fields_}
+
+
+def sq_consume(pe=-1, block=-1, target_arena=None):
+    """Consumer pass over the rings of (pe, block), -1 = all (rsm_sq_consume): retire what
+    they published, write completion entries and, when ``target_arena`` (a DeviceArray laid
+    out like the arena) is given, execute every entry against it.  Returns the totals."""
+    t = ConsumeTotals()
+    _check(L.load().rsm_sq_consume(pe, block, _addr(target_arena) if target_arena is not None else None,
+                                   C.byref(t)))
+    return t.as_dict()
+
+
+def sq_set_mode(queue):
+    """False: rings are logs that wrap freely; True: slots are freed by sq_consume only."""
+    _check(L.load().rsm_sq_set_mode(1 if queue else 0))
+
+
+def sq_consumer_state(pe, block):
+    a, b = C.c_uint32(0), C.c_uint32(0)
+    _check(L.load().rsm_sq_consumer_state(pe, block, C.byref(a), C.byref(b)))
+    return {"consumed": a.value, "cq_producer": b.value}
+
+
+def cq_image(pe, block, entries):
+    out = np.zeros(entries * 64, dtype=np.uint8)
+    _check(L.load().rsm_cq_image(pe, block, out.ctypes.data, out.nbytes))
+    return out.reshape(entries, 64)
+
+
+def atomic_ret_image(pe, block, words=4096):
+    out = np.zeros(words, dtype=np.uint64)
+    _check(L.load().rsm_atomic_ret_image(pe, block, out.ctypes.data, out.nbytes))
+    return out
+
+
+def arena():
+    """(base address, bytes, slice stride) of the arena that holds every PE slice."""
+    base, nbytes, stride = C.c_void_p(0), C.c_size_t(0), C.c_size_t(0)
+    _check(L.load().rsm_arena(C.byref(base), C.byref(nbytes), C.byref(stride)))
+    return base.value, nbytes.value, stride.value
+
+
+def read_device(addr, nbytes):
+    """Bytes [addr, addr+nbytes) of device memory as a uint8 array."""
+    out = np.empty(nbytes, dtype=np.uint8)
+    _check(L.load().rsm_copy_to_host(out.ctypes.data, _addr(addr), nbytes))
+    return out
+
+
+def write_device(addr, values):
+    a = np.ascontiguousarray(values)
+    _check(L.load().rsm_copy_to_device(_addr(addr), a.ctypes.data, a.nbytes))
 
 
 def kat_fetch_incr(lane_mask, n_wgs, wg_size):

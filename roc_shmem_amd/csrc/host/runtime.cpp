@@ -99,6 +99,7 @@ Options Options::from_env() {
     double d = atof(s);
     if (d > 0) o.wait_limit_s = d;
   }
+  if (const char *s = getenv("ROC_SHMEM_SQ_MODE")) o.sq_queue_mode = strcmp(s, "queue") == 0;
   return o;
 }
 
@@ -174,6 +175,11 @@ std::string Runtime::init(const Options &opt) {
   RT_HIP(hipMemset(queue_mem_, 0, queue_mem_bytes_));
   RT_HIP(hipMalloc(reinterpret_cast<void **>(&counters_dev_), sizeof(detail::SqCounters) * rings));
   RT_HIP(hipMemset(counters_dev_, 0, sizeof(detail::SqCounters) * rings));
+  // Completion queues: as many entries as the send queue has slots
+  // (reference: cqe = max_send_wr, connection.cpp:200-206).
+  const size_t cq_bytes = static_cast<size_t>(opt_.sq_size) * 64;
+  cq_mem_bytes_ = cq_bytes * rings;
+  RT_HIP(hipMalloc(reinterpret_cast<void **>(&cq_mem_), cq_mem_bytes_));
 
   // Synthetic queue-pair constants standing in for what the reference
   // harvests from a NIC-built template WQE (connection.cpp:379-391).
@@ -204,6 +210,9 @@ std::string Runtime::init(const Options &opt) {
       c.ring.lkey = bswap32(0x2000u);
       c.ring.atomic_lkey = bswap32(0x3000u);
       c.ring.max_nwqe = opt_.sq_size;
+      c.ring.cq = reinterpret_cast<uint64_t *>(cq_mem_ + cq_bytes * r);
+      c.ring.cq_size = opt_.sq_size;
+      c.ring.cq_log_size = static_cast<uint32_t>(__builtin_ctz(opt_.sq_size));
       c.counters = counters_dev_ + r;
     }
   }
@@ -232,6 +241,9 @@ std::string Runtime::init(const Options &opt) {
   state_.team_world = world_->device;
   state_.status = status_dev_;
   state_.wait_limit_ticks = static_cast<uint64_t>(opt_.wait_limit_s * 100e6);  // 100 MHz clock
+  state_.sq_queue_mode = opt_.sq_queue_mode ? 1u : 0u;
+  state_.pad_ = 0;
+  reset_queues(nullptr);
   if (!upload_state_everywhere(state_))
     return "could not upload the device state into every translation unit";
   RT_HIP(hipDeviceSynchronize());
@@ -246,6 +258,7 @@ void Runtime::teardown() {
   if (rkeys_dev_) (void)hipFree(rkeys_dev_);
   if (counters_dev_) (void)hipFree(counters_dev_);
   if (queue_mem_) (void)hipFree(queue_mem_);
+  if (cq_mem_) (void)hipFree(cq_mem_);
   if (base_heap_dev_) (void)hipFree(base_heap_dev_);
   if (arena_) (void)hipFree(arena_);
   teams_dev_ = nullptr;
@@ -254,6 +267,7 @@ void Runtime::teardown() {
   rkeys_dev_ = nullptr;
   counters_dev_ = nullptr;
   queue_mem_ = nullptr;
+  cq_mem_ = nullptr;
   base_heap_dev_ = nullptr;
   arena_ = nullptr;
   teams_.clear();
@@ -359,8 +373,18 @@ const TeamRecord *Runtime::team_record(const detail::Team *team) const {
   return it == teams_.end() ? nullptr : &it->second;
 }
 
+bool Runtime::set_sq_queue_mode(bool queue) {
+  (void)hipDeviceSynchronize();
+  state_.sq_queue_mode = queue ? 1u : 0u;
+  return upload_state_everywhere(state_);
+}
+
 void Runtime::reset_queues(hipStream_t stream) {
   (void)hipMemsetAsync(queue_mem_, 0, queue_mem_bytes_, stream);
+  (void)hipMemsetAsync(cq_mem_, 0, cq_mem_bytes_, stream);
+  // op_own (last byte of every completion entry) = invalid opcode, owner 0:
+  // what a reader finds before the first completion lands in an entry.
+  (void)hipMemset2DAsync(cq_mem_ + 63, 64, 0xF0, 1, cq_mem_bytes_ / 64, stream);
   (void)hipMemsetAsync(counters_dev_, 0,
                        sizeof(detail::SqCounters) * static_cast<size_t>(opt_.num_pes) *
                            opt_.num_blocks,

@@ -51,6 +51,7 @@ struct Options {
   uint32_t sq_size = 1024;         // ROC_SHMEM_SQ_SIZE (reference: connection.hpp:225)
   size_t slice_pad = 0;            // ROC_SHMEM_SLICE_PAD, extra bytes between slices
   double wait_limit_s = 2.0;       // ROC_SHMEM_WAIT_LIMIT_S, bound of a device flag wait
+  bool sq_queue_mode = false;      // ROC_SHMEM_SQ_MODE=queue: slots are freed by the consumer pass
   static Options from_env();
 };
 
@@ -95,8 +96,17 @@ class Runtime {
   const detail::DeviceCtx &ctx_image(int pe, int block) const {
     return ctx_images_[static_cast<size_t>(pe) * opt_.num_blocks + block];
   }
-  // Zero every ring, mailbox and producer index.
+  // Zero every ring, mailbox, producer and consumer index; completion entries
+  // go back to "owned by hardware, invalid".
   void reset_queues(hipStream_t stream);
+  // false: rings are logs that wrap freely; true: rings are queues whose
+  // slots are freed only by the consumer pass.  Returns false when the state
+  // could not be re-uploaded.
+  bool set_sq_queue_mode(bool queue);
+  bool sq_queue_mode() const { return state_.sq_queue_mode != 0; }
+  const detail::DeviceState &device_state() const { return state_; }
+  char *arena() const { return arena_; }
+  size_t arena_bytes() const { return stride_ * static_cast<size_t>(opt_.num_pes); }
 
   // Reads and clears the sticky device status word.
   uint32_t take_status();
@@ -121,6 +131,8 @@ class Runtime {
   std::vector<detail::DeviceCtx> ctx_images_;
   char *queue_mem_ = nullptr;   // rings + mailboxes + atomic-return windows
   size_t queue_mem_bytes_ = 0;
+  char *cq_mem_ = nullptr;      // completion queues, sq_size 64-byte entries per ring
+  size_t cq_mem_bytes_ = 0;
   detail::SqCounters *counters_dev_ = nullptr;
   uint32_t *rkeys_dev_ = nullptr;
   uint32_t *status_dev_ = nullptr;

@@ -60,6 +60,11 @@ struct SqRing {
   uint32_t lkey;
   uint32_t atomic_lkey;
   uint32_t max_nwqe;
+  // Completion queue filled by the consumer pass (reference: current_cq_q,
+  // cq_size, cq_log_size, queue_pair.hpp:340-396): cq_size 64-byte entries.
+  uint64_t *cq;
+  uint32_t cq_size;
+  uint32_t cq_log_size;
 };
 
 // Mutable producer indices of a ring, on their own cache line.
@@ -67,7 +72,9 @@ struct alignas(64) SqCounters {
   uint32_t sq_counter;      // free-running WQE index (reference: queue_pair.hpp:378)
   uint32_t published;       // every WQE below this index is complete in memory
   uint32_t atomic_counter;  // free-running AMO return-slot index
-  uint32_t pad_[13];
+  uint32_t consumed;        // every WQE below this index has been retired by the consumer pass
+  uint32_t cq_producer;     // free-running count of completion entries written
+  uint32_t pad_[11];
 };
 
 // One context = one (PE, block) pair (reference: GPUIBContext members,
@@ -92,6 +99,11 @@ struct DeviceState {
   Team *team_world;
   uint32_t *status;
   uint64_t wait_limit_ticks;   // wall_clock64() ticks a flag wait may take
+  // 0: a ring is a log, a slot may be rewritten once its previous entry is
+  // published.  1: a ring is a queue, a slot may be rewritten only after the
+  // consumer pass has retired its previous entry.
+  uint32_t sq_queue_mode;
+  uint32_t pad_;
 };
 
 }  // namespace detail

@@ -89,9 +89,12 @@ __device__ __forceinline__ void wave_post(DeviceCtx *ctx, bool sends, const WqeR
   const uint32_t ring_size = ctx->ring.max_nwqe;
   uint32_t base = 0, abase = 0;
   if (sends && rank == 0) {
-    // Issued together so their latencies overlap: the published index (only
-    // ever grows, so an early read is conservative) and the reservation.
-    uint32_t seen = __hip_atomic_load(&cnt->published, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // Issued together so their latencies overlap: the index that frees slots
+    // (only ever grows, so an early read is conservative) and the reservation.
+    // Slots are freed by publication when the ring is a log and by the
+    // consumer pass when it is a queue.
+    uint32_t *freed = g_state.sq_queue_mode ? &cnt->consumed : &cnt->published;
+    uint32_t seen = __hip_atomic_load(freed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     base = __hip_atomic_fetch_add(&cnt->sq_counter, n, __ATOMIC_RELAXED,
                                   __HIP_MEMORY_SCOPE_AGENT);
     if (atomic_mask) {
@@ -99,14 +102,14 @@ __device__ __forceinline__ void wave_post(DeviceCtx *ctx, bool sends, const WqeR
                                      static_cast<uint32_t>(__popcll(atomic_mask)),
                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    // Queue space: entry c may be written once entry c - ring_size is published.
+    // Queue space: entry c may be written once entry c - ring_size is freed.
     if (static_cast<int32_t>(base + n - seen - ring_size) > 0) {
       const uint32_t need = base + n - ring_size;
       uint64_t start = wall_clock64();
       uint32_t spins = 0;
       while (static_cast<int32_t>(
-                 need - __hip_atomic_load(&cnt->published, __ATOMIC_RELAXED,
-                                          __HIP_MEMORY_SCOPE_AGENT)) > 0) {
+                 need - __hip_atomic_load(freed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >
+             0) {
         __builtin_amdgcn_s_sleep(1);
         if ((++spins & 63u) == 0 &&
             (status_failed() || wall_clock64() - start > g_state.wait_limit_ticks)) {

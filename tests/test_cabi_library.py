@@ -30,8 +30,13 @@ def test_every_declared_symbol_is_exported_and_bound():
 def test_each_kernel_unit_keeps_its_own_device_state():
     # One upload hook per translation unit that contains device code; a single shared hook
     # would leave the other units' kernels with a zeroed state.
+    import glob
     from roc_shmem_amd import _lib
-    assert _lib.load().rsm_state_units() == 6
+    csrc = os.path.join(ROOT, "roc_shmem_amd", "csrc")
+    drivers = glob.glob(os.path.join(csrc, "cabi", "drv_*.hip"))
+    # every driver unit, plus cabi.cpp and host/api_host.cpp, which include the device header too
+    assert len(drivers) >= 5
+    assert _lib.load().rsm_state_units() == len(drivers) + 2
 
 
 @pytest.mark.skipif(gpu_present(), reason="checks the no-GPU error path")
