@@ -183,7 +183,9 @@ void broadcast_team(size_t elem_size, roc_shmem_team_t team, void *dest, const v
 namespace detail {
 // Registration of one translation unit's copy of the device state.
 typedef bool (*StateUploadFn)(const DeviceState *);
-void register_state_upload(StateUploadFn fn);
+// `layout` is the unit's detail::kStateLayout; roc_shmem_init fails when it is
+// not the library's own.
+void register_state_upload(StateUploadFn fn, uint32_t layout);
 }  // namespace detail
 
 }  // namespace rocshmem

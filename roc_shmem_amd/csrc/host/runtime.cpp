@@ -244,6 +244,9 @@ std::string Runtime::init(const Options &opt) {
   state_.sq_queue_mode = opt_.sq_queue_mode ? 1u : 0u;
   state_.pad_ = 0;
   reset_queues(nullptr);
+  if (!state_layouts_agree())
+    return "a translation unit of this program was compiled against other device headers than "
+           "this library (rebuild it against include/ and roc_shmem_amd/csrc of this library)";
   if (!upload_state_everywhere(state_))
     return "could not upload the device state into every translation unit";
   RT_HIP(hipDeviceSynchronize());
@@ -404,28 +407,43 @@ uint32_t Runtime::take_status() {
 // ---------------------------------------------------------------------------
 
 typedef bool (*UploadFn)(const detail::DeviceState *);
-static std::vector<UploadFn> &registry() {
-  static std::vector<UploadFn> fns;
-  return fns;
+struct Unit {
+  UploadFn fn;
+  uint32_t layout;
+  bool operator<(const Unit &o) const { return fn < o.fn; }
+  bool operator==(const Unit &o) const { return fn == o.fn; }
+};
+static std::vector<Unit> &registry() {
+  static std::vector<Unit> units;
+  return units;
+}
+
+bool state_layouts_agree() {
+  for (const Unit &u : registry())
+    if (u.layout != detail::kStateLayout) return false;
+  return true;
 }
 
 bool upload_state_everywhere(const detail::DeviceState &state) {
+  if (!state_layouts_agree()) return false;
   bool ok = true;
-  for (UploadFn fn : registry()) ok = fn(&state) && ok;
+  for (const Unit &u : registry()) ok = u.fn(&state) && ok;
   return ok;
 }
 
 int registered_state_units() {
-  std::vector<UploadFn> fns = registry();
-  std::sort(fns.begin(), fns.end());
-  return static_cast<int>(std::unique(fns.begin(), fns.end()) - fns.begin());
+  std::vector<Unit> units = registry();
+  std::sort(units.begin(), units.end());
+  return static_cast<int>(std::unique(units.begin(), units.end()) - units.begin());
 }
 
 }  // namespace host
 
 namespace detail {
 typedef bool (*StateUploadFn)(const DeviceState *);
-void register_state_upload(StateUploadFn fn) { host::registry().push_back(fn); }
+void register_state_upload(StateUploadFn fn, uint32_t layout) {
+  host::registry().push_back(host::Unit{fn, layout});
+}
 }  // namespace detail
 
 }  // namespace rocshmem

@@ -147,6 +147,8 @@ class Runtime {
 // copies the device state into its own __constant__ instance.
 // Returns false when any unit could not be updated and verified.
 bool upload_state_everywhere(const detail::DeviceState &state);
+// False when a registered unit was compiled against different state structures.
+bool state_layouts_agree();
 // Number of distinct translation units registered for state uploads.
 int registered_state_units();
 

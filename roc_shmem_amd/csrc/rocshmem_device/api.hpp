@@ -42,7 +42,7 @@ bool upload_state_to_this_unit(const DeviceState *s) {
   return __builtin_memcmp(&check, s, sizeof(DeviceState)) == 0;
 }
 struct StateRegistrar {
-  StateRegistrar() { register_state_upload(&upload_state_to_this_unit); }
+  StateRegistrar() { register_state_upload(&upload_state_to_this_unit, kStateLayout); }
 };
 StateRegistrar g_state_registrar;
 }  // namespace

@@ -106,6 +106,18 @@ struct DeviceState {
   uint32_t pad_;
 };
 
+// Fingerprint of the structures device code and the host library share.  Device
+// code is compiled into every user program (the interface is header-only); a
+// program built against other headers than the library it loads would index
+// ctx_table with the wrong stride and follow wild pointers, so every unit hands
+// its fingerprint to the library, which refuses to initialise on a mismatch.
+// Bump kStateRevision when a layout changes without changing a size.
+constexpr uint32_t kStateRevision = 2;
+constexpr uint32_t kStateLayout =
+    (kStateRevision * 0x01000193u) ^
+    static_cast<uint32_t>(sizeof(DeviceState) | (sizeof(DeviceCtx) << 8) | (sizeof(Team) << 16) |
+                          (sizeof(SqCounters) << 24));
+
 }  // namespace detail
 }  // namespace rocshmem
 

@@ -10,14 +10,34 @@ import subprocess
 
 import pytest
 
+import glob
+
 HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
 BINARY = os.path.join(HERE, "cxx", "host_api_check")
+
+
+def newest_header():
+    pats = [os.path.join(ROOT, "include", "*.h*"),
+            os.path.join(ROOT, "roc_shmem_amd", "csrc", "rocshmem_device", "*.hpp")]
+    return max(os.path.getmtime(f) for p in pats for f in glob.glob(p))
+
+
+def test_check_program_is_not_older_than_the_headers_it_inlines():
+    # The device interface is header-only: a program built before a header changed carries
+    # device code for the old state layout.  (The library refuses to initialise for such a
+    # program; this catches it before anything runs.)
+    if not os.path.exists(BINARY):
+        pytest.skip("tests/cxx/host_api_check is not built yet")
+    assert os.path.getmtime(BINARY) >= newest_header(), \
+        "tests/cxx/host_api_check is stale: run __graft_entry__.build()"
 
 
 @pytest.mark.gpu
 def test_host_api_program():
     if not os.path.exists(BINARY):
         pytest.fail("tests/cxx/host_api_check is not built: run __graft_entry__.build()")
+    assert os.path.getmtime(BINARY) >= newest_header(), "stale check program: run __graft_entry__.build()"
     print("running", BINARY, flush=True)
     out = subprocess.run([BINARY], capture_output=True, text=True, timeout=100)
     tail = (out.stdout + out.stderr)[-3000:]
