@@ -223,6 +223,16 @@ def bench_small_ops(rs, n_pes, n_ops, wgs_total, wg_size, slice_bytes, seed):
         ms = event_time_ms(rs, step, 3) / 3
         res[name] = {"Mops_per_s": n_ops / ms / 1e3, "ms": ms}
         dev.free()
+    # Consumer pass over what the last stream left in the rings (each ring keeps its newest
+    # sq_size entries): check + complete only, host-timed around the synchronous call.
+    t0 = time.perf_counter()
+    totals = rs.sq_consume()
+    dt = time.perf_counter() - t0
+    if totals["rejected"]:
+        raise RuntimeError("the consumer pass rejected %d ring entries" % totals["rejected"])
+    res["consume_check_only"] = {"entries": totals["retired"], "rejected": totals["rejected"],
+                                 "lost_to_wraparound": totals["lost"], "ms": dt * 1e3,
+                                 "Mentries_per_s": totals["retired"] / dt / 1e6}
     status = rs.take_status()
     if status:
         raise RuntimeError("device status word raised: %d" % status)
