@@ -212,6 +212,29 @@ def test_owner_bit_flips_on_every_lap_of_the_completion_queue():
         assert counters == [(64 * lap + i) & 0xFFFF for i in range(64)]
 
 
+def test_hand_assembled_completion_entries():
+    # tests/golden/wqe_hand_assembled.json: completion entries written out by hand.
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                           "wqe_hand_assembled.json")) as f:
+        g = json.load(f)
+    assert len(g["completions"]) >= 2
+    for e in g["completions"]:
+        qp = make_qp(max_nwqe=1024)
+        qp.ctrl_qp_sq = int.from_bytes(bytes.fromhex(e["qpn_bytes"]), "little")
+        ring = Ring(qp)
+        ring.count = e["wqe_index"]                       # the entry sits at this stream position
+        ring.post(oracle.OP_WRITE, 0, 0, size=4, inline=b"abcd", cqe=True)
+        cq = np.zeros(e["cq_size"] * 64, np.uint8)
+        cq[63::64] = 0xF0
+        prod, totals, view, _ = consume(ring, None, None, consumed=e["wqe_index"], cq=cq,
+                                        cq_producer=e["cq_producer"])
+        assert prod == e["cq_producer"] + 1 and totals["rejected"] == 0
+        want = bytes.fromhex("".join(e["bytes"]).replace(" ", ""))
+        assert bytes(view[e["cq_producer"] % e["cq_size"]]) == want, e["name"]
+
+
 def test_replay_agrees_with_the_small_operation_model():
     # The same random stream through (a) the small-op model and (b) builder -> ring -> consumer.
     rng = np.random.default_rng(11)

@@ -4,6 +4,8 @@ The reference holds no test or fixture for WQE bytes (parity unpinned); the chec
 here are what the entry format itself fixes, plus three entries assembled by hand from the
 field table of the format."""
 import itertools
+import json
+import os
 
 import numpy as np
 
@@ -18,38 +20,33 @@ def qp(ctrl_qp_sq=0x030201, ctrl_sig=0, lkey=0x00200000, atomic_lkey=0x00300000,
     return q
 
 
+def golden():
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                           "wqe_hand_assembled.json")) as f:
+        return json.load(f)
+
+
+def num(v):
+    return int(v, 0) if isinstance(v, str) else int(v)
+
+
 def test_hand_assembled_entries():
-    # 8-byte inline RDMA write, counter 0x1234, qpn bytes 01 02 03, raddr 0x0000_7FAB_CDEF_0128,
-    # rkey bytes 00 00 10 05 in memory, payload 88 77 66 55 44 33 22 11
-    slot = np.full(64, 0xEE, np.uint8)
-    oracle.wqe_build(slot, qp(), 0x1234, oracle.OP_WRITE, size=8, raddr=0x00007FABCDEF0128,
-                     rkey=0x05100000, inline=bytes([0x88, 0x77, 0x66, 0x55, 0x44, 0x33, 0x22, 0x11]))
-    want = bytes.fromhex(
-        "00" "1234" "08" "010203" "03" "00" "EEEE" "00" "00000000"
-        "00007FABCDEF0128" "00001005" "EEEEEEEE"
-        "80000008" "8877665544332211" "EEEEEEEE"
-        "EEEEEEEEEEEEEEEEEEEEEEEEEEEEEEEE")
-    assert bytes(slot) == want
-    # 4 KiB RDMA read with a data pointer segment, completion requested
-    slot = np.zeros(64, np.uint8)
-    oracle.wqe_build(slot, qp(), 0x10001, oracle.OP_READ, size=4096, raddr=0x7F1122334455,
-                     rkey=0x01000000, laddr=0x7FFF00000040, request_cqe=True)
-    want = bytes.fromhex(
-        "00" "0001" "10" "010203" "03" "00" "0000" "08" "00000000"
-        "00007F1122334455" "00000001" "00000000"
-        "00001000" "00002000" "00007FFF00000040"
-        "00000000000000000000000000000000")
-    assert bytes(slot) == want
-    # fetch-add of -2, return slot 5
-    slot = np.zeros(64, np.uint8)
-    oracle.wqe_build(slot, qp(), 7, oracle.OP_ATOMIC_FA, size=8, raddr=0x1000, rkey=0xAABBCCDD,
-                     atomic_data=-2, atomic_cmp=0, atomic_pos=5, request_cqe=True)
-    want = bytes.fromhex(
-        "00" "0007" "12" "010203" "04" "00" "0000" "08" "00000000"
-        "0000000000001000" "DDCCBBAA" "00000000"
-        "FFFFFFFFFFFFFFFE" "0000000000000000"
-        "00000008" "00003000" "00007F0000001028")
-    assert bytes(slot) == want
+    # Entries written out by hand from the entry format (tests/golden/wqe_hand_assembled.json).
+    g = golden()
+    q = g["queue"]
+    queue = qp(num(q["ctrl_qp_sq"]), num(q["ctrl_sig"]), num(q["lkey"]), num(q["atomic_lkey"]),
+               num(q["atomic_ret_base"]), num(q["max_nwqe"]))
+    assert len(g["entries"]) >= 4
+    for e in g["entries"]:
+        slot = np.full(64, int(e["background"], 16), np.uint8)
+        oracle.wqe_build(slot, queue, num(e["counter"]), num(e["opcode"]), size=e["size"],
+                         raddr=num(e["raddr"]), rkey=num(e["rkey"]), laddr=num(e.get("laddr", 0)),
+                         atomic_data=num(e.get("atomic_data", 0)), atomic_cmp=num(e.get("atomic_cmp", 0)),
+                         inline=bytes.fromhex(e.get("inline", "")), atomic_pos=e.get("atomic_pos", 0),
+                         request_cqe=e["cqe"])
+        want = bytes.fromhex("".join(e["bytes"]).replace(" ", ""))
+        assert len(want) == 64
+        assert bytes(slot) == want, e["name"]
 
 
 def test_format_invariants():
