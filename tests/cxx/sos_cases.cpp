@@ -1,0 +1,602 @@
+// The reference's host-program tests (clients/sos_tests/*.cpp), restated for a
+// process that hosts every PE.  Each case keeps the reference's inputs and its
+// closed-form expectation and cites the file it follows.  Where the
+// reference's SPMD code says "every PE does X", the case loops over the PEs
+// with roc_shmemx_set_pe; where it dereferences symmetric memory on the host
+// (the reference's heap is host-visible), the case goes through
+// roc_shmem_<T>_put / _get on the calling PE, because the arena here is
+// ordinary device memory.  A collective is called once for all members.
+// Exit code 0 and a final line "SOS_CASES_OK" mean every case passed.
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "roc_shmem.hpp"
+
+using namespace rocshmem;
+
+static int failures = 0;
+static const char *current_case = "";
+#define EXPECT(cond, ...)                                        \
+  do {                                                           \
+    if (!(cond)) {                                               \
+      if (++failures <= 20) {                                    \
+        printf("FAIL [%s] %s:%d: ", current_case, __FILE__, __LINE__); \
+        printf(__VA_ARGS__);                                     \
+        printf("\n");                                            \
+      }                                                          \
+    }                                                            \
+  } while (0)
+
+// A symmetric array of n elements of T with host-side access per PE.
+template <typename T>
+struct Sym {
+  T *ptr;
+  int n;
+  explicit Sym(int count) : ptr(static_cast<T *>(roc_shmem_malloc(count * sizeof(T)))), n(count) {
+    if (!ptr) {
+      printf("roc_shmem_malloc failed\n");
+      exit(2);
+    }
+  }
+  ~Sym() { roc_shmem_free(ptr); }
+  void store(int pe, const std::vector<T> &v) const {
+    roc_shmem_putmem(ptr, v.data(), static_cast<size_t>(n) * sizeof(T), pe);
+  }
+  void fill(int pe, T value) const { store(pe, std::vector<T>(n, value)); }
+  std::vector<T> load(int pe) const {
+    std::vector<T> v(n);
+    roc_shmem_getmem(v.data(), ptr, static_cast<size_t>(n) * sizeof(T), pe);
+    return v;
+  }
+};
+
+static int npes;
+
+// ---- reductions ---------------------------------------------------------------------
+
+#define FOR_REDUCE_TYPES(X) X(short, short) X(int, int) X(long, long) X(float, float) X(double, double) X(long long, longlong)
+#define FOR_BITWISE_TYPES(X) X(short, short) X(int, int) X(long, long) X(long long, longlong)
+
+// clients/sos_tests/to_all.cpp:118-760, N = 128: max/min of me+i, sum of me, and of me,
+// prod of me+1, or of (me+1)%4, xor of me%2, checked on every PE.
+template <typename T, typename Call, typename Src, typename Want>
+static void reduce_case(const char *name, Call call, Src src_of, Want want_of) {
+  current_case = name;
+  const int N = 128;
+  Sym<T> src(N), dst(N);
+  for (int me = 0; me < npes; ++me) {
+    std::vector<T> v(N);
+    for (int i = 0; i < N; ++i) v[i] = static_cast<T>(src_of(me, i));
+    src.store(me, v);
+    dst.fill(me, static_cast<T>(-9));
+  }
+  roc_shmem_barrier_all();
+  call(dst.ptr, src.ptr, N);
+  for (int me = 0; me < npes; ++me) {
+    std::vector<T> got = dst.load(me);
+    for (int i = 0; i < N; ++i)
+      EXPECT(got[i] == static_cast<T>(want_of(i)), "PE %d element %d: %g, expected %g", me, i,
+             static_cast<double>(got[i]), static_cast<double>(want_of(i)));
+  }
+}
+
+static void to_all_cases() {
+  long factorial = 1;
+  for (int i = 1; i <= npes; ++i) factorial *= i;
+#define MAXMIN_SUM_PROD(T, TNAME)                                                                  \
+  reduce_case<T>("to_all.cpp max " #TNAME,                                                         \
+                 [](T *d, const T *s, int n) {                                                     \
+                   roc_shmem_ctx_##TNAME##_max_to_all(ROC_SHMEM_CTX_DEFAULT, d, s, n, 0, 0, npes,  \
+                                                      nullptr, nullptr);                           \
+                 },                                                                                \
+                 [](int me, int i) { return me + i; }, [](int i) { return npes - 1 + i; });        \
+  reduce_case<T>("to_all.cpp min " #TNAME,                                                         \
+                 [](T *d, const T *s, int n) {                                                     \
+                   roc_shmem_ctx_##TNAME##_min_to_all(ROC_SHMEM_CTX_DEFAULT, d, s, n, 0, 0, npes,  \
+                                                      nullptr, nullptr);                           \
+                 },                                                                                \
+                 [](int me, int i) { return me + i; }, [](int i) { return i; });                   \
+  reduce_case<T>("to_all.cpp sum " #TNAME,                                                         \
+                 [](T *d, const T *s, int n) {                                                     \
+                   roc_shmem_ctx_##TNAME##_sum_to_all(ROC_SHMEM_CTX_DEFAULT, d, s, n, 0, 0, npes,  \
+                                                      nullptr, nullptr);                           \
+                 },                                                                                \
+                 [](int me, int) { return me; }, [](int) { return npes * (npes - 1) / 2; });       \
+  reduce_case<T>("to_all.cpp prod " #TNAME,                                                        \
+                 [](T *d, const T *s, int n) {                                                     \
+                   roc_shmem_ctx_##TNAME##_prod_to_all(ROC_SHMEM_CTX_DEFAULT, d, s, n, 0, 0, npes, \
+                                                       nullptr, nullptr);                          \
+                 },                                                                                \
+                 [](int me, int) { return me + 1; }, [factorial](int) { return factorial; });
+  FOR_REDUCE_TYPES(MAXMIN_SUM_PROD)
+#undef MAXMIN_SUM_PROD
+#define BITWISE(T, TNAME)                                                                          \
+  reduce_case<T>("to_all.cpp and " #TNAME,                                                         \
+                 [](T *d, const T *s, int n) {                                                     \
+                   roc_shmem_ctx_##TNAME##_and_to_all(ROC_SHMEM_CTX_DEFAULT, d, s, n, 0, 0, npes,  \
+                                                      nullptr, nullptr);                           \
+                 },                                                                                \
+                 [](int me, int) { return me; }, [](int) { return 0; });                           \
+  reduce_case<T>("to_all.cpp or " #TNAME,                                                          \
+                 [](T *d, const T *s, int n) {                                                     \
+                   roc_shmem_ctx_##TNAME##_or_to_all(ROC_SHMEM_CTX_DEFAULT, d, s, n, 0, 0, npes,   \
+                                                     nullptr, nullptr);                            \
+                 },                                                                                \
+                 [](int me, int) { return (me + 1) % 4; }, [](int) { return npes == 1 ? 1 : 3; }); \
+  reduce_case<T>("to_all.cpp xor " #TNAME,                                                         \
+                 [](T *d, const T *s, int n) {                                                     \
+                   roc_shmem_ctx_##TNAME##_xor_to_all(ROC_SHMEM_CTX_DEFAULT, d, s, n, 0, 0, npes,  \
+                                                      nullptr, nullptr);                           \
+                 },                                                                                \
+                 [](int me, int) { return me % 2; }, [](int) { return (npes / 2) % 2; });
+  FOR_BITWISE_TYPES(BITWISE)
+#undef BITWISE
+}
+
+// clients/sos_tests/max_reduction.cpp:65-99: N = 3, src = me + i, long max -> npes - 1 + i.
+static void max_reduction() {
+  current_case = "max_reduction.cpp";
+  const int N = 3;
+  Sym<long> src(N), dst(N);
+  for (int me = 0; me < npes; ++me) src.store(me, {me + 0L, me + 1L, me + 2L});
+  roc_shmem_barrier_all();
+  roc_shmem_ctx_long_max_to_all(ROC_SHMEM_CTX_DEFAULT, dst.ptr, src.ptr, N, 0, 0, npes, nullptr, nullptr);
+  for (int me = 0; me < npes; ++me) {
+    std::vector<long> got = dst.load(me);
+    for (int i = 0; i < N; ++i) EXPECT(got[i] == npes - 1 + i, "PE %d dst[%d] = %ld", me, i, got[i]);
+  }
+}
+
+// clients/sos_tests/big_reduction.cpp:76-107 (long max over N elements of me + i) and
+// reduce_in_place.cpp:58-69 (dest == source).
+static void big_and_in_place_reduction() {
+  current_case = "big_reduction.cpp / reduce_in_place.cpp";
+  const int N = 1 << 20;
+  Sym<long> buf(N);
+  std::vector<long> v(N);
+  for (int me = 0; me < npes; ++me) {
+    for (int i = 0; i < N; ++i) v[i] = me + i;
+    buf.store(me, v);
+  }
+  roc_shmem_barrier_all();
+  roc_shmem_ctx_long_max_to_all(ROC_SHMEM_CTX_DEFAULT, buf.ptr, buf.ptr, N, 0, 0, npes, nullptr, nullptr);
+  for (int me = 0; me < npes; ++me) {
+    std::vector<long> got = buf.load(me);
+    for (int i = 0; i < N; ++i) EXPECT(got[i] == npes - 1 + i, "PE %d [%d] = %ld", me, i, got[i]);
+  }
+}
+
+// clients/sos_tests/reduce_active_set.cpp:78-113: for i = 0..npes-1 the PEs i..npes-1 sum
+// src = me (long long); members get sum_{p>=i} p, the others keep -1.
+static void reduce_active_set() {
+  current_case = "reduce_active_set.cpp";
+  const int N = 4;
+  Sym<long long> src(N), dst(N);
+  for (int start = 0; start < npes; ++start) {
+    for (int me = 0; me < npes; ++me) {
+      src.fill(me, me);
+      dst.fill(me, -1);
+    }
+    roc_shmem_barrier_all();
+    roc_shmem_ctx_longlong_sum_to_all(ROC_SHMEM_CTX_DEFAULT, dst.ptr, src.ptr, N, start, 0, npes - start,
+                                      nullptr, nullptr);
+    long long want = 0;
+    for (int p = start; p < npes; ++p) want += p;
+    for (int me = 0; me < npes; ++me) {
+      std::vector<long long> got = dst.load(me);
+      for (int i = 0; i < N; ++i)
+        EXPECT(got[i] == (me >= start ? want : -1), "start %d PE %d [%d] = %lld", start, me, i, got[i]);
+    }
+  }
+}
+
+// clients/sos_tests/shmem_team_reduce.cpp:88-101 on the world team: src = 1 -> and/or/max/min/prod
+// give 1, sum gives npes, xor gives npes % 2.
+static void team_reduce() {
+  current_case = "shmem_team_reduce.cpp";
+  const int N = 10;
+  Sym<int> src(N), dst(N);
+  for (int me = 0; me < npes; ++me) src.fill(me, 1);
+  struct {
+    void (*call)(roc_shmem_ctx_t, roc_shmem_team_t, int *, const int *, int);
+    int want;
+    const char *name;
+  } ops[] = {
+      {roc_shmem_ctx_int_and_to_all, 1, "and"},   {roc_shmem_ctx_int_or_to_all, 1, "or"},
+      {roc_shmem_ctx_int_max_to_all, 1, "max"},   {roc_shmem_ctx_int_min_to_all, 1, "min"},
+      {roc_shmem_ctx_int_prod_to_all, 1, "prod"}, {roc_shmem_ctx_int_sum_to_all, npes, "sum"},
+      {roc_shmem_ctx_int_xor_to_all, npes % 2, "xor"},
+  };
+  for (auto &op : ops) {
+    for (int me = 0; me < npes; ++me) dst.fill(me, -7);
+    op.call(ROC_SHMEM_CTX_DEFAULT, ROC_SHMEM_TEAM_WORLD, dst.ptr, src.ptr, N);
+    for (int me = 0; me < npes; ++me) {
+      std::vector<int> got = dst.load(me);
+      for (int i = 0; i < N; ++i) EXPECT(got[i] == op.want, "%s PE %d [%d] = %d", op.name, me, i, got[i]);
+    }
+  }
+}
+
+// ---- put / get -------------------------------------------------------------------------
+
+// clients/sos_tests/put1.cpp:38-68: PE 0 puts ten longs 1..10 into PE 1.
+static void put1() {
+  current_case = "put1.cpp";
+  long source[10] = {1, 2, 3, 4, 5, 6, 7, 8, 9, 10};
+  Sym<long> target(10);
+  for (int me = 0; me < npes; ++me) target.fill(me, 0);
+  roc_shmemx_set_pe(0);
+  roc_shmem_long_put(target.ptr, source, 10, 1);
+  roc_shmem_barrier_all();
+  std::vector<long> got = target.load(1);
+  EXPECT(memcmp(got.data(), source, sizeof(source)) == 0, "target on PE 1 differs from the source");
+  for (int me = 0; me < npes; ++me)
+    if (me != 1) {
+      std::vector<long> other = target.load(me);
+      for (long x : other) EXPECT(x == 0, "PE %d was written", me);
+    }
+}
+
+// clients/sos_tests/get_nbi.cpp:47-76 (PE 0 gets source = i + 1 from every PE, quiet, compare) and
+// put_nbi.cpp (the mirror image with put_nbi + quiet).
+static void get_nbi_put_nbi() {
+  current_case = "get_nbi.cpp / put_nbi.cpp";
+  Sym<long> source(10), target(10);
+  std::vector<long> pattern(10);
+  for (int i = 0; i < 10; ++i) pattern[i] = i + 1;
+  for (int me = 0; me < npes; ++me) {
+    source.store(me, pattern);
+    target.fill(me, 0);
+  }
+  roc_shmem_barrier_all();
+  roc_shmemx_set_pe(0);
+  for (int j = 0; j < npes; ++j) {
+    long local[10] = {0};
+    roc_shmem_long_get_nbi(local, source.ptr, 10, j);
+    roc_shmem_quiet();
+    for (int i = 0; i < 10; ++i) EXPECT(local[i] == i + 1, "get_nbi from PE %d [%d] = %ld", j, i, local[i]);
+  }
+  for (int j = 0; j < npes; ++j) roc_shmem_long_put_nbi(target.ptr, pattern.data(), 10, j);
+  roc_shmem_quiet();
+  for (int j = 0; j < npes; ++j) {
+    std::vector<long> got = target.load(j);
+    for (int i = 0; i < 10; ++i) EXPECT(got[i] == i + 1, "put_nbi to PE %d [%d] = %ld", j, i, got[i]);
+  }
+}
+
+// clients/sos_tests/bigput.cpp:202-263 and bigget.cpp: a large block of Source[i] = i + 1 moved
+// to / from the next PE arrives unchanged.
+static void bigput_bigget() {
+  current_case = "bigput.cpp / bigget.cpp";
+  const int N = 1 << 20;
+  Sym<int> source(N), target(N);
+  std::vector<int> pattern(N), back(N);
+  for (int i = 0; i < N; ++i) pattern[i] = i + 1;
+  for (int me = 0; me < npes; ++me) {
+    source.store(me, pattern);
+    target.fill(me, -90);
+  }
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    // the host-side put takes any host or device pointer as its local buffer
+    roc_shmem_int_put(target.ptr, pattern.data(), N, (me + 1) % npes);
+  }
+  roc_shmem_barrier_all();
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    roc_shmem_int_get(back.data(), target.ptr, N, (me + 1) % npes);
+    EXPECT(back == pattern, "block fetched by PE %d differs", me);
+  }
+}
+
+// clients/sos_tests/cxx_test_shmem_p.cpp:42-62 and cxx_test_shmem_g.cpp:42-64, all standard types,
+// with and without a context: p of (TYPE)me to the right-hand neighbour; g from it.
+template <typename T, typename P, typename G>
+static void p_g_case(const char *name, P p, G g) {
+  current_case = name;
+  Sym<T> remote(1);
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    p(remote.ptr, static_cast<T>(me), (me + 1) % npes);
+  }
+  roc_shmem_barrier_all();
+  for (int me = 0; me < npes; ++me)
+    EXPECT(remote.load(me)[0] == static_cast<T>((me + npes - 1) % npes), "p: PE %d", me);
+  for (int me = 0; me < npes; ++me) remote.fill(me, static_cast<T>(me));
+  roc_shmem_barrier_all();
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    EXPECT(g(remote.ptr, (me + 1) % npes) == static_cast<T>((me + 1) % npes), "g: PE %d", me);
+  }
+}
+
+static void p_and_g() {
+#define PG(T, TNAME)                                                                              \
+  p_g_case<T>("cxx_test_shmem_p/g " #TNAME,                                                       \
+              [](T *d, T v, int pe) { roc_shmem_##TNAME##_p(d, v, pe); },                         \
+              [](const T *s, int pe) { return roc_shmem_##TNAME##_g(s, pe); });                   \
+  p_g_case<T>("cxx_test_shmem_p/g ctx " #TNAME,                                                   \
+              [](T *d, T v, int pe) { roc_shmem_ctx_##TNAME##_p(ROC_SHMEM_CTX_DEFAULT, d, v, pe); }, \
+              [](const T *s, int pe) { return roc_shmem_ctx_##TNAME##_g(ROC_SHMEM_CTX_DEFAULT, s, pe); });
+  PG(float, float) PG(double, double) PG(char, char) PG(signed char, schar) PG(short, short) PG(int, int)
+  PG(long, long) PG(long long, longlong) PG(unsigned char, uchar) PG(unsigned short, ushort)
+  PG(unsigned int, uint) PG(unsigned long, ulong) PG(unsigned long long, ulonglong)
+#undef PG
+}
+
+// ---- atomics ------------------------------------------------------------------------------
+
+#define FOR_AMO_TYPES(X)                                                                            \
+  X(int, int) X(long, long) X(long long, longlong) X(unsigned int, uint) X(unsigned long, ulong)    \
+  X(unsigned long long, ulonglong) X(int32_t, int32) X(int64_t, int64) X(uint32_t, uint32)          \
+  X(uint64_t, uint64) X(size_t, size) X(ptrdiff_t, ptrdiff)
+
+template <typename T, typename Add, typename FetchAdd>
+static void atomic_add_case(const char *name, Add add, FetchAdd fetch_add) {
+  // cxx_test_shmem_atomic_add.cpp:85-144: every PE adds me + 1 to every PE -> npes(npes+1)/2;
+  // the fetching form additionally returns something no larger than the final value.
+  current_case = name;
+  Sym<T> remote(1);
+  for (int me = 0; me < npes; ++me) remote.fill(me, 0);
+  roc_shmem_barrier_all();
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    for (int i = 0; i < npes; ++i) add(remote.ptr, static_cast<T>(me + 1), i);
+  }
+  roc_shmem_barrier_all();
+  const T total = static_cast<T>(npes * (npes + 1) / 2);
+  for (int me = 0; me < npes; ++me) EXPECT(remote.load(me)[0] == total, "add: PE %d", me);
+  for (int me = 0; me < npes; ++me) remote.fill(me, 0);
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    for (int i = 0; i < npes; ++i) {
+      T old = fetch_add(remote.ptr, static_cast<T>(me + 1), i);
+      EXPECT(old <= total, "fetch_add: PE %d old too large", me);
+    }
+  }
+  for (int me = 0; me < npes; ++me) EXPECT(remote.load(me)[0] == total, "fetch_add: PE %d", me);
+}
+
+template <typename T, typename Fetch, typename Inc, typename FetchInc, typename Cswap>
+static void atomic_fetch_inc_cswap_case(const char *name, Fetch fetch, Inc inc, FetchInc fetch_inc,
+                                        Cswap cswap) {
+  current_case = name;
+  Sym<T> remote(1);
+  // cxx_test_shmem_atomic_fetch.cpp:66-107: *remote = me; fetch from the neighbour gives its rank.
+  for (int me = 0; me < npes; ++me) remote.fill(me, static_cast<T>(me));
+  roc_shmem_barrier_all();
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    EXPECT(fetch(remote.ptr, (me + 1) % npes) == static_cast<T>((me + 1) % npes), "fetch: PE %d", me);
+  }
+  // cxx_test_shmem_atomic_inc.cpp:85-147: every PE increments every PE once -> npes; a fetched
+  // old value is never larger than npes.
+  for (int me = 0; me < npes; ++me) remote.fill(me, 0);
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    for (int i = 0; i < npes; ++i) inc(remote.ptr, i);
+  }
+  for (int me = 0; me < npes; ++me) EXPECT(remote.load(me)[0] == static_cast<T>(npes), "inc: PE %d", me);
+  for (int me = 0; me < npes; ++me) remote.fill(me, 0);
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    for (int i = 0; i < npes; ++i) EXPECT(fetch_inc(remote.ptr, i) <= static_cast<T>(npes), "fetch_inc old");
+  }
+  for (int me = 0; me < npes; ++me)
+    EXPECT(remote.load(me)[0] == static_cast<T>(npes), "fetch_inc: PE %d", me);
+  // cxx_test_shmem_atomic_cswap.cpp:73-111: *remote = npes; cswap(cond npes, value me) on the
+  // neighbour returns npes and leaves the left-hand neighbour's rank.
+  for (int me = 0; me < npes; ++me) remote.fill(me, static_cast<T>(npes));
+  roc_shmem_barrier_all();
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    T old = cswap(remote.ptr, static_cast<T>(npes), static_cast<T>(me), (me + 1) % npes);
+    EXPECT(old == static_cast<T>(npes), "cswap old: PE %d", me);
+  }
+  for (int me = 0; me < npes; ++me)
+    EXPECT(remote.load(me)[0] == static_cast<T>((me + npes - 1) % npes), "cswap: PE %d", me);
+}
+
+static void atomics() {
+#define AMO(T, TNAME)                                                                               \
+  atomic_add_case<T>("cxx_test_shmem_atomic_add " #TNAME,                                           \
+                     [](T *d, T v, int pe) { roc_shmem_##TNAME##_atomic_add(d, v, pe); },           \
+                     [](T *d, T v, int pe) { return roc_shmem_##TNAME##_atomic_fetch_add(d, v, pe); }); \
+  atomic_add_case<T>(                                                                               \
+      "cxx_test_shmem_atomic_add ctx " #TNAME,                                                      \
+      [](T *d, T v, int pe) { roc_shmem_ctx_##TNAME##_atomic_add(ROC_SHMEM_CTX_DEFAULT, d, v, pe); }, \
+      [](T *d, T v, int pe) {                                                                       \
+        return roc_shmem_ctx_##TNAME##_atomic_fetch_add(ROC_SHMEM_CTX_DEFAULT, d, v, pe);           \
+      });                                                                                           \
+  atomic_fetch_inc_cswap_case<T>(                                                                   \
+      "cxx_test_shmem_atomic_fetch/inc/cswap " #TNAME,                                              \
+      [](T *d, int pe) { return roc_shmem_##TNAME##_atomic_fetch(d, pe); },                         \
+      [](T *d, int pe) { roc_shmem_##TNAME##_atomic_inc(d, pe); },                                  \
+      [](T *d, int pe) { return roc_shmem_##TNAME##_atomic_fetch_inc(d, pe); },                     \
+      [](T *d, T c, T v, int pe) { return roc_shmem_##TNAME##_atomic_compare_swap(d, c, v, pe); }); \
+  atomic_fetch_inc_cswap_case<T>(                                                                   \
+      "cxx_test_shmem_atomic_fetch/inc/cswap ctx " #TNAME,                                          \
+      [](T *d, int pe) { return roc_shmem_ctx_##TNAME##_atomic_fetch(ROC_SHMEM_CTX_DEFAULT, d, pe); }, \
+      [](T *d, int pe) { roc_shmem_ctx_##TNAME##_atomic_inc(ROC_SHMEM_CTX_DEFAULT, d, pe); },       \
+      [](T *d, int pe) { return roc_shmem_ctx_##TNAME##_atomic_fetch_inc(ROC_SHMEM_CTX_DEFAULT, d, pe); }, \
+      [](T *d, T c, T v, int pe) {                                                                  \
+        return roc_shmem_ctx_##TNAME##_atomic_compare_swap(ROC_SHMEM_CTX_DEFAULT, d, c, v, pe);     \
+      });
+  FOR_AMO_TYPES(AMO)
+#undef AMO
+}
+
+// clients/sos_tests/atomic_inc.cpp / lfinc.cpp:90-111: `loops` rounds in which every PE
+// fetch-increments one counter on PE 0; the values handed out are 0 .. npes*loops-1, each once.
+static void lfinc() {
+  current_case = "lfinc.cpp / atomic_inc.cpp";
+  const int loops = 10;
+  Sym<long> counter(1);
+  for (int me = 0; me < npes; ++me) counter.fill(me, 0);
+  std::vector<int> seen(npes * loops, 0);
+  for (int round = 0; round < loops; ++round)
+    for (int me = 0; me < npes; ++me) {
+      roc_shmemx_set_pe(me);
+      long v = roc_shmem_long_atomic_fetch_inc(counter.ptr, 0);
+      EXPECT(v >= 0 && v < npes * loops && seen[v]++ == 0, "value %ld handed out twice or out of range", v);
+    }
+  EXPECT(counter.load(0)[0] == npes * loops, "final count %ld", counter.load(0)[0]);
+}
+
+// clients/sos_tests/mt_a2a.cpp:50-118, one thread's view: every PE adds its rank to dest[tid] on
+// every PE (sum (npes-1)npes/2), increments flag[tid] everywhere (npes), then puts -1 to its
+// neighbour and reads -1 back from every PE.
+static void mt_a2a() {
+  current_case = "mt_a2a.cpp";
+  const int T = 8;
+  Sym<long> dest(T), flag(T);
+  for (int me = 0; me < npes; ++me) {
+    dest.fill(me, 0);
+    flag.fill(me, 0);
+  }
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    for (int tid = 0; tid < T; ++tid)
+      for (int i = 1; i <= npes; ++i) roc_shmem_int64_atomic_add(reinterpret_cast<int64_t *>(&dest.ptr[tid]), me, (me + i) % npes);
+  }
+  roc_shmem_fence();
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    for (int tid = 0; tid < T; ++tid)
+      for (int i = 1; i <= npes; ++i) roc_shmem_int64_atomic_inc(reinterpret_cast<int64_t *>(&flag.ptr[tid]), (me + i) % npes);
+  }
+  for (int me = 0; me < npes; ++me) {
+    std::vector<long> d = dest.load(me), f = flag.load(me);
+    for (int tid = 0; tid < T; ++tid)
+      EXPECT(d[tid] == (npes - 1) * npes / 2 && f[tid] == npes, "PE %d tid %d: dest %ld flag %ld", me, tid,
+             d[tid], f[tid]);
+  }
+  roc_shmem_barrier_all();
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    long val = -1;
+    for (int tid = 0; tid < T; ++tid) roc_shmem_long_put(&dest.ptr[tid], &val, 1, (me + 1) % npes);
+  }
+  roc_shmem_barrier_all();
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    for (int tid = 0; tid < T; ++tid)
+      for (int i = 1; i <= npes; ++i) {
+        long val = 0;
+        roc_shmem_long_get(&val, &dest.ptr[tid], 1, (me + i) % npes);
+        EXPECT(val == -1, "PE %d tid %d from PE %d: %ld", me, tid, (me + i) % npes, val);
+      }
+  }
+}
+
+// ---- broadcast ---------------------------------------------------------------------------------
+
+// clients/sos_tests/bcast.cpp:99-133: ten rounds, 16 bytes growing by 1 KiB each; root 1 of the
+// world; src[i] = i + 1 (src[0] stays 0); every PE but the root receives, the root's dst stays 0.
+static void bcast() {
+  current_case = "bcast.cpp";
+  int n_bytes = 16;
+  for (int loop = 1; loop <= 10; ++loop) {
+    const int n = n_bytes / static_cast<int>(sizeof(long));
+    Sym<long> buf(2 * n);
+    long *dst = buf.ptr, *src = buf.ptr + n;
+    std::vector<long> init(2 * n, 0);
+    for (int i = 1; i < n; ++i) init[n + i] = i + 1;
+    for (int me = 0; me < npes; ++me) buf.store(me, init);
+    roc_shmem_barrier_all();
+    roc_shmem_ctx_long_broadcast(ROC_SHMEM_CTX_DEFAULT, dst, src, n, 1, 0, 0, npes, nullptr);
+    for (int me = 0; me < npes; ++me) {
+      std::vector<long> got = buf.load(me);
+      for (int i = 0; i < n; ++i)
+        EXPECT(got[i] == (me == 1 ? 0 : init[n + i]), "round %d PE %d dst[%d] = %ld", loop, me, i, got[i]);
+    }
+    n_bytes += 1024;
+  }
+}
+
+// clients/sos_tests/bcast_flood.cpp:145-170: back-to-back int broadcasts from root 0 of
+// source[i] = i + 1 over target = -90.
+static void bcast_flood() {
+  current_case = "bcast_flood.cpp";
+  const int elements = 4096, loops = 20;
+  Sym<int> source(elements), target(elements);
+  std::vector<int> pattern(elements);
+  for (int i = 0; i < elements; ++i) pattern[i] = i + 1;
+  for (int me = 0; me < npes; ++me) {
+    source.store(me, pattern);
+    target.fill(me, -90);
+  }
+  roc_shmem_barrier_all();
+  for (int i = 0; i < loops; ++i)
+    roc_shmem_ctx_int_broadcast(ROC_SHMEM_CTX_DEFAULT, target.ptr, source.ptr, elements, 0, 0, 0, npes, nullptr);
+  roc_shmem_barrier_all();
+  for (int me = 0; me < npes; ++me) {
+    std::vector<int> got = target.load(me);
+    for (int i = 0; i < elements; ++i)
+      EXPECT(got[i] == (me == 0 ? -90 : i + 1), "PE %d target[%d] = %d", me, i, got[i]);
+  }
+}
+
+// clients/sos_tests/broadcast_active_set.cpp:84-128: the active set shrinks from the front
+// (PE_start = i, size = npes - i) and the root is its first member; members other than the root
+// receive the root's value, everybody else keeps what it had.
+static void broadcast_active_set() {
+  current_case = "broadcast_active_set.cpp";
+  const int N = 8;
+  Sym<long> src(N), dst(N);
+  for (int start = 0; start < npes; ++start) {
+    for (int me = 0; me < npes; ++me) {
+      src.fill(me, me + 100);
+      dst.fill(me, -1);
+    }
+    roc_shmem_barrier_all();
+    roc_shmem_ctx_long_broadcast(ROC_SHMEM_CTX_DEFAULT, dst.ptr, src.ptr, N, 0, start, 0, npes - start, nullptr);
+    for (int me = 0; me < npes; ++me) {
+      std::vector<long> got = dst.load(me);
+      const long want = me > start ? start + 100 : -1;
+      for (int i = 0; i < N; ++i) EXPECT(got[i] == want, "start %d PE %d [%d] = %ld", start, me, i, got[i]);
+    }
+  }
+}
+
+int main() {
+  if (!getenv("ROC_SHMEM_NUM_PES")) setenv("ROC_SHMEM_NUM_PES", "6", 1);
+  setenv("ROC_SHMEM_HEAP_SIZE", "134217728", 0);
+  roc_shmem_init();
+  npes = roc_shmem_n_pes();
+  struct {
+    const char *name;
+    void (*run)();
+  } cases[] = {{"to_all", to_all_cases},
+               {"max_reduction", max_reduction},
+               {"big_reduction", big_and_in_place_reduction},
+               {"reduce_active_set", reduce_active_set},
+               {"team_reduce", team_reduce},
+               {"put1", put1},
+               {"get_nbi", get_nbi_put_nbi},
+               {"bigput", bigput_bigget},
+               {"p_g", p_and_g},
+               {"atomics", atomics},
+               {"lfinc", lfinc},
+               {"mt_a2a", mt_a2a},
+               {"bcast", bcast},
+               {"bcast_flood", bcast_flood},
+               {"broadcast_active_set", broadcast_active_set}};
+  for (auto &c : cases) {
+    const int before = failures;
+    c.run();
+    roc_shmemx_set_pe(0);
+    EXPECT(roc_shmemx_take_status() == 0, "device status word raised");
+    printf("%-22s %s\n", c.name, failures == before ? "ok" : "FAILED");
+    fflush(stdout);
+  }
+  roc_shmem_finalize();
+  if (failures) {
+    printf("SOS_CASES_FAILED %d\n", failures);
+    return 1;
+  }
+  printf("SOS_CASES_OK\n");
+  return 0;
+}

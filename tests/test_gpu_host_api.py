@@ -15,6 +15,7 @@ import glob
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 BINARY = os.path.join(HERE, "cxx", "host_api_check")
+SOS_BINARY = os.path.join(HERE, "cxx", "sos_cases")
 
 
 def newest_header():
@@ -27,10 +28,11 @@ def test_check_program_is_not_older_than_the_headers_it_inlines():
     # The device interface is header-only: a program built before a header changed carries
     # device code for the old state layout.  (The library refuses to initialise for such a
     # program; this catches it before anything runs.)
-    if not os.path.exists(BINARY):
-        pytest.skip("tests/cxx/host_api_check is not built yet")
-    assert os.path.getmtime(BINARY) >= newest_header(), \
-        "tests/cxx/host_api_check is stale: run __graft_entry__.build()"
+    for binary in (BINARY, SOS_BINARY):
+        if not os.path.exists(binary):
+            pytest.skip("%s is not built yet" % binary)
+        assert os.path.getmtime(binary) >= newest_header(), \
+            "%s is stale: run __graft_entry__.build()" % binary
 
 
 @pytest.mark.gpu
@@ -43,3 +45,18 @@ def test_host_api_program():
     tail = (out.stdout + out.stderr)[-3000:]
     assert out.returncode == 0, tail
     assert "HOST_API_OK" in out.stdout, tail
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("num_pes", [2, 6])
+def test_reference_host_programs_restated(num_pes):
+    # tests/cxx/sos_cases.cpp: the reference's clients/sos_tests programs, one function each.
+    if not os.path.exists(SOS_BINARY):
+        pytest.fail("tests/cxx/sos_cases is not built: run __graft_entry__.build()")
+    assert os.path.getmtime(SOS_BINARY) >= newest_header(), "stale check program: run __graft_entry__.build()"
+    print("running", SOS_BINARY, "with", num_pes, "PEs", flush=True)
+    env = dict(os.environ, ROC_SHMEM_NUM_PES=str(num_pes))
+    out = subprocess.run([SOS_BINARY], capture_output=True, text=True, timeout=110, env=env)
+    tail = (out.stdout + out.stderr)[-3000:]
+    assert out.returncode == 0, tail
+    assert "SOS_CASES_OK" in out.stdout, tail
