@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <functional>
 #include <sstream>
 
 namespace rocshmem {
@@ -352,7 +353,9 @@ int Runtime::team_split(detail::Team *parent, int start, int stride, int size,
   if (stride_world & (stride_world - 1)) return -1;  // collectives address members by log2 stride
   int log_stride = 0;
   while ((1 << log_stride) < stride_world) ++log_stride;
-  if (static_cast<int>(teams_.size()) >= kMaxTeams - 1) {
+  // teams_ holds the world team too; the reference counts user teams only
+  // (num_user_teams >= max_num_teams - 1 aborts, roc_shmem.cpp:224-228).
+  if (static_cast<int>(teams_.size()) - 1 >= kMaxTeams - 1) {
     fprintf(stderr, "rocshmem: too many teams (limit %d)\n", kMaxTeams);
     abort();  // reference: roc_shmem.cpp:224-228
   }
@@ -410,7 +413,7 @@ typedef bool (*UploadFn)(const detail::DeviceState *);
 struct Unit {
   UploadFn fn;
   uint32_t layout;
-  bool operator<(const Unit &o) const { return fn < o.fn; }
+  bool operator<(const Unit &o) const { return std::less<UploadFn>()(fn, o.fn); }
   bool operator==(const Unit &o) const { return fn == o.fn; }
 };
 static std::vector<Unit> &registry() {

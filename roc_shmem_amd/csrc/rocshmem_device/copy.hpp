@@ -221,14 +221,30 @@ __device__ __forceinline__ void wave_copy(void *dst, const void *src, size_t n) 
   group_copy_uniform(uniform(dst), uniform(src), uniform(n), lane_id(), kWaveSize);
 }
 
+// One naturally aligned element moved with device-coherent accesses (agent-scope
+// relaxed atomics: the store is written through this XCD's L2, the load does
+// not trust a line another XCD may have changed).  Single-element puts and
+// gets are what programs signal and poll with - p on one PE, wait_until or a
+// g loop on another, no quiet in between (reference: ping_pong_tester.cpp:
+// 48-57) - so they must not sit in a write-back cache or be served from a
+// stale line until the kernel ends.
+template <typename W>
+__device__ __forceinline__ void coherent_store(void *dst, W bits) {
+  __hip_atomic_store(static_cast<W *>(dst), bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename W>
+__device__ __forceinline__ W coherent_load(const void *src) {
+  return __hip_atomic_load(static_cast<const W *>(src), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // Single-lane copy used by the thread-level put/get: the common 4- and 8-byte
-// naturally aligned messages are a single store.
+// naturally aligned messages are one coherent load and one coherent store.
 __device__ __forceinline__ void lane_copy(void *dst, const void *src, size_t n) {
   uintptr_t both = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src);
   if (n == 8 && (both & 7u) == 0) {
-    *static_cast<uint64_t *>(dst) = *static_cast<const uint64_t *>(src);
+    coherent_store<uint64_t>(dst, coherent_load<uint64_t>(src));
   } else if (n == 4 && (both & 3u) == 0) {
-    *static_cast<uint32_t *>(dst) = *static_cast<const uint32_t *>(src);
+    coherent_store<uint32_t>(dst, coherent_load<uint32_t>(src));
   } else {
     group_copy(dst, src, n, 0u, 1u);
   }

@@ -32,6 +32,9 @@ __device__ __forceinline__ void thread_put(DeviceCtx *ctx, void *dest, const voi
                                            size_t nbytes, int pe) {
   if (nbytes == 0) return;  // reference: Context::putmem early-out, context_device.cpp:80-82
   char *remote = translate(static_cast<char *>(dest), ctx->my_pe, pe);
+  // The operation itself goes first: its latency is what a waiting PE sees,
+  // and it overlaps with the chain of queue atomics behind the post.
+  lane_copy(remote, source, nbytes);
   CoalesceResult c = wave_coalesce(pe, reinterpret_cast<uint64_t>(source),
                                    reinterpret_cast<uint64_t>(dest), nbytes);
   WqeRequest rq;
@@ -47,13 +50,13 @@ __device__ __forceinline__ void thread_put(DeviceCtx *ctx, void *dest, const voi
     rq.inline_data = gather_inline(source, static_cast<uint32_t>(c.size));
   }
   wave_post(ctx, c.must_send, rq);
-  lane_copy(remote, source, nbytes);
 }
 
 __device__ __forceinline__ void thread_get(DeviceCtx *ctx, void *dest, const void *source,
                                            size_t nbytes, int pe) {
   if (nbytes == 0) return;
   const char *remote = translate(static_cast<const char *>(source), ctx->my_pe, pe);
+  lane_copy(dest, remote, nbytes);
   CoalesceResult c = wave_coalesce(pe, reinterpret_cast<uint64_t>(source),
                                    reinterpret_cast<uint64_t>(dest), nbytes);
   WqeRequest rq;
@@ -66,7 +69,6 @@ __device__ __forceinline__ void thread_get(DeviceCtx *ctx, void *dest, const voi
   rq.inline_data = 0;
   rq.pe = pe;
   wave_post(ctx, c.must_send, rq);
-  lane_copy(dest, remote, nbytes);
 }
 
 // Single-element put of a register value (reference: GPUIBContext::p,
@@ -74,9 +76,36 @@ __device__ __forceinline__ void thread_get(DeviceCtx *ctx, void *dest, const voi
 // stack copy, which never satisfies the coalescer's contiguity test, so every
 // lane posts its own inline entry; the same holds here without touching
 // scratch memory.
+// One element of a standard type through device-coherent accesses (see
+// coherent_store in copy.hpp).
+template <typename T>
+__device__ __forceinline__ void element_store(T *p, T value) {
+  static_assert(sizeof(T) == 1 || sizeof(T) == 2 || sizeof(T) == 4 || sizeof(T) == 8, "element size");
+  using W = typename std::conditional<
+      sizeof(T) == 8, uint64_t,
+      typename std::conditional<sizeof(T) == 4, uint32_t,
+                                typename std::conditional<sizeof(T) == 2, uint16_t, uint8_t>::type>::type>::type;
+  W bits;
+  __builtin_memcpy(&bits, &value, sizeof(T));
+  coherent_store<W>(p, bits);
+}
+template <typename T>
+__device__ __forceinline__ T element_load(const T *p) {
+  static_assert(sizeof(T) == 1 || sizeof(T) == 2 || sizeof(T) == 4 || sizeof(T) == 8, "element size");
+  using W = typename std::conditional<
+      sizeof(T) == 8, uint64_t,
+      typename std::conditional<sizeof(T) == 4, uint32_t,
+                                typename std::conditional<sizeof(T) == 2, uint16_t, uint8_t>::type>::type>::type;
+  W bits = coherent_load<W>(p);
+  T value;
+  __builtin_memcpy(&value, &bits, sizeof(T));
+  return value;
+}
+
 template <typename T>
 __device__ __forceinline__ void thread_p(DeviceCtx *ctx, T *dest, T value, int pe) {
   T *remote = translate(dest, ctx->my_pe, pe);
+  element_store(remote, value);
   uint64_t bits = 0;
   __builtin_memcpy(&bits, &value, sizeof(T));
   WqeRequest rq;
@@ -89,12 +118,12 @@ __device__ __forceinline__ void thread_p(DeviceCtx *ctx, T *dest, T value, int p
   rq.inline_data = bits;
   rq.pe = pe;
   wave_post(ctx, true, rq);
-  *remote = value;
 }
 
 template <typename T>
 __device__ __forceinline__ T thread_g(DeviceCtx *ctx, const T *source, int pe) {
   const T *remote = translate(source, ctx->my_pe, pe);
+  const T value = element_load(remote);
   WqeRequest rq;
   rq.opcode = kOpcodeRdmaRead;
   rq.size = sizeof(T);
@@ -105,7 +134,7 @@ __device__ __forceinline__ T thread_g(DeviceCtx *ctx, const T *source, int pe) {
   rq.inline_data = 0;
   rq.pe = pe;
   wave_post(ctx, true, rq);
-  return *remote;
+  return value;
 }
 
 // ---- atomics ---------------------------------------------------------------
@@ -151,22 +180,22 @@ __device__ __forceinline__ void amo_record(DeviceCtx *ctx, uint8_t opcode, T *re
 template <typename T>
 __device__ __forceinline__ T amo_fetch_add(DeviceCtx *ctx, T *dest, T value, int pe) {
   T *remote = translate(dest, ctx->my_pe, pe);
+  const T old = __hip_atomic_fetch_add(remote, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   amo_record<T>(ctx, kOpcodeAtomicFa, remote, value, T(0), pe);
-  return __hip_atomic_fetch_add(remote, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return old;
 }
 
 template <typename T>
 __device__ __forceinline__ void amo_add(DeviceCtx *ctx, T *dest, T value, int pe) {
   T *remote = translate(dest, ctx->my_pe, pe);
-  amo_record<T>(ctx, kOpcodeAtomicFa, remote, value, T(0), pe);
   (void)__hip_atomic_fetch_add(remote, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  amo_record<T>(ctx, kOpcodeAtomicFa, remote, value, T(0), pe);
 }
 
 // compare_swap(dest, cond, value): store `value` iff *dest == cond; returns the old value.
 template <typename T>
 __device__ __forceinline__ T amo_fetch_cas(DeviceCtx *ctx, T *dest, T value, T cond, int pe) {
   T *remote = translate(dest, ctx->my_pe, pe);
-  amo_record<T>(ctx, kOpcodeAtomicCs, remote, value, cond, pe);
   using W = typename AtomicWord<T>::type;
   W expected, desired;
   __builtin_memcpy(&expected, &cond, sizeof(T));
@@ -174,6 +203,7 @@ __device__ __forceinline__ T amo_fetch_cas(DeviceCtx *ctx, T *dest, T value, T c
   __hip_atomic_compare_exchange_strong(reinterpret_cast<W *>(remote), &expected, desired,
                                        __ATOMIC_RELAXED, __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
+  amo_record<T>(ctx, kOpcodeAtomicCs, remote, value, cond, pe);
   T old;
   __builtin_memcpy(&old, &expected, sizeof(T));
   return old;
@@ -187,12 +217,12 @@ __device__ __forceinline__ T amo_fetch_cas(DeviceCtx *ctx, T *dest, T value, T c
 template <typename T>
 __device__ __forceinline__ T amo_swap(DeviceCtx *ctx, T *dest, T value, int pe) {
   T *remote = translate(dest, ctx->my_pe, pe);
-  amo_record<T>(ctx, kOpcodeAtomicCs, remote, value, T(0), pe);
   using W = typename AtomicWord<T>::type;
   W desired;
   __builtin_memcpy(&desired, &value, sizeof(T));
   W prev = __hip_atomic_exchange(reinterpret_cast<W *>(remote), desired, __ATOMIC_RELAXED,
                                  __HIP_MEMORY_SCOPE_AGENT);
+  amo_record<T>(ctx, kOpcodeAtomicCs, remote, value, T(0), pe);
   T old;
   __builtin_memcpy(&old, &prev, sizeof(T));
   return old;
@@ -202,10 +232,10 @@ template <typename T>
 __device__ __forceinline__ T amo_fetch(DeviceCtx *ctx, T *dest, int pe) {
   // reference: fetch == fetch_add(0), roc_shmem_gpu.cpp:589-598
   T *remote = translate(dest, ctx->my_pe, pe);
-  amo_record<T>(ctx, kOpcodeAtomicFa, remote, T(0), T(0), pe);
   using W = typename AtomicWord<T>::type;
   W raw = __hip_atomic_load(reinterpret_cast<W *>(remote), __ATOMIC_RELAXED,
                             __HIP_MEMORY_SCOPE_AGENT);
+  amo_record<T>(ctx, kOpcodeAtomicFa, remote, T(0), T(0), pe);
   T old;
   __builtin_memcpy(&old, &raw, sizeof(T));
   return old;

@@ -1,0 +1,469 @@
+// User kernels written the way the reference's functional testers are
+// (clients/functional_tests/*_tester.cpp), compiled against the public header
+// only, each citing the tester it follows.  Differences forced by "one process
+// hosts every PE": the grid carries the workgroups of all PEs
+// (blockIdx.x % n_pes is the PE, blockIdx.x / n_pes the workgroup's index within
+// it, where the reference uses blockIdx.x), kernel arguments that name
+// symmetric objects pass through roc_shmemx_my_addr, and "only rank 0
+// launches" becomes "only PE 0's workgroups act".
+// Exit code 0 and a final line "DEVICE_API_OK" mean every case passed.
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "roc_shmem.hpp"
+
+using namespace rocshmem;
+
+static int failures = 0;
+static const char *current_case = "";
+#define EXPECT(cond, ...)                                               \
+  do {                                                                  \
+    if (!(cond)) {                                                      \
+      if (++failures <= 20) {                                           \
+        printf("FAIL [%s] %s:%d: ", current_case, __FILE__, __LINE__);  \
+        printf(__VA_ARGS__);                                            \
+        printf("\n");                                                   \
+      }                                                                 \
+    }                                                                   \
+  } while (0)
+
+static int npes;
+
+static void finish_kernel(const char *what) {
+  roc_shmem_barrier_all();
+  hipError_t e = hipGetLastError();
+  EXPECT(e == hipSuccess, "%s: %s", what, hipGetErrorString(e));
+  EXPECT(roc_shmemx_take_status() == 0, "%s: device status word raised", what);
+}
+
+template <typename T>
+static std::vector<T> load(const T *sym, int n, int pe) {
+  std::vector<T> v(n);
+  roc_shmem_getmem(v.data(), sym, n * sizeof(T), pe);
+  return v;
+}
+template <typename T>
+static void fill(T *sym, int n, T value, int pe) {
+  std::vector<T> v(n, value);
+  roc_shmem_putmem(sym, v.data(), n * sizeof(T), pe);
+}
+
+__device__ inline int wg_index() { return blockIdx.x / roc_shmem_n_pes(); }
+
+// ---- ping_pong_tester.cpp:32-62 ----------------------------------------------------------
+__global__ void PingPongTest(int loop, int skip, uint64_t *timer, int *r_buf) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  int pe = roc_shmem_ctx_my_pe(ctx);
+  r_buf = roc_shmemx_my_addr(r_buf);
+  const int w = wg_index();
+  if (threadIdx.x == 0 && pe < 2) {
+    uint64_t start = 0;
+    for (int i = 0; i < loop + skip; i++) {
+      if (i == skip) start = roc_shmem_timer();
+      if (pe == 0) {
+        roc_shmem_ctx_int_p(ctx, &r_buf[w], i + 1, 1);
+        roc_shmem_int_wait_until(&r_buf[w], ROC_SHMEM_CMP_EQ, i + 1);
+      } else {
+        roc_shmem_int_wait_until(&r_buf[w], ROC_SHMEM_CMP_EQ, i + 1);
+        roc_shmem_ctx_int_p(ctx, &r_buf[w], i + 1, 0);
+      }
+    }
+    timer[blockIdx.x] = roc_shmem_timer() - start;
+  }
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+static void ping_pong() {
+  current_case = "ping_pong_tester.cpp";
+  const int wgs = 4, loop = 200, skip = 20;
+  int *r_buf = static_cast<int *>(roc_shmem_malloc(sizeof(int) * wgs));
+  uint64_t *timer = nullptr;
+  (void)hipMalloc(reinterpret_cast<void **>(&timer), sizeof(uint64_t) * wgs * npes);
+  (void)hipMemset(timer, 0, sizeof(uint64_t) * wgs * npes);
+  for (int pe = 0; pe < npes; ++pe) fill(r_buf, wgs, 0, pe);
+  PingPongTest<<<wgs * npes, 64>>>(loop, skip, timer, r_buf);
+  finish_kernel("PingPongTest");
+  for (int pe = 0; pe < 2; ++pe)
+    for (int v : load(r_buf, wgs, pe)) EXPECT(v == loop + skip, "PE %d r_buf = %d", pe, v);
+  std::vector<uint64_t> t(wgs * npes);
+  (void)hipMemcpy(t.data(), timer, sizeof(uint64_t) * t.size(), hipMemcpyDeviceToHost);
+  // ticks of the 100 MHz constant clock; one iteration is a full round trip
+  printf("  ping-pong round trip: %.2f us (p + wait_until, 4 pairs at once)\n",
+         t[0] / 100.0 / loop);
+  (void)hipFree(timer);
+  roc_shmem_free(r_buf);
+}
+
+// ---- roc_shmem_<T>_wait_until / _test, all six comparisons (context_tmpl_device.hpp:199-246) ----
+__global__ void CompareTest(long *word, float *fword, int *results) {
+  roc_shmem_wg_init();
+  word = roc_shmemx_my_addr(word);
+  fword = roc_shmemx_my_addr(fword);
+  if (threadIdx.x == 0 && roc_shmem_my_pe() == 0) {
+    int k = 0;
+    // *word == 5
+    results[k++] = roc_shmem_long_test(word, ROC_SHMEM_CMP_EQ, 5);
+    results[k++] = roc_shmem_long_test(word, ROC_SHMEM_CMP_EQ, 6);
+    results[k++] = roc_shmem_long_test(word, ROC_SHMEM_CMP_NE, 6);
+    results[k++] = roc_shmem_long_test(word, ROC_SHMEM_CMP_NE, 5);
+    results[k++] = roc_shmem_long_test(word, ROC_SHMEM_CMP_GT, 4);
+    results[k++] = roc_shmem_long_test(word, ROC_SHMEM_CMP_GT, 5);
+    results[k++] = roc_shmem_long_test(word, ROC_SHMEM_CMP_GE, 5);
+    results[k++] = roc_shmem_long_test(word, ROC_SHMEM_CMP_GE, 6);
+    results[k++] = roc_shmem_long_test(word, ROC_SHMEM_CMP_LT, 6);
+    results[k++] = roc_shmem_long_test(word, ROC_SHMEM_CMP_LT, 5);
+    results[k++] = roc_shmem_long_test(word, ROC_SHMEM_CMP_LE, 5);
+    results[k++] = roc_shmem_long_test(word, ROC_SHMEM_CMP_LE, 4);
+    // satisfied waits return at once
+    roc_shmem_long_wait_until(word, ROC_SHMEM_CMP_EQ, 5);
+    roc_shmem_long_wait_until(word, ROC_SHMEM_CMP_NE, 0);
+    roc_shmem_long_wait_until(word, ROC_SHMEM_CMP_GT, -1);
+    roc_shmem_long_wait_until(word, ROC_SHMEM_CMP_GE, 5);
+    roc_shmem_long_wait_until(word, ROC_SHMEM_CMP_LT, 100);
+    roc_shmem_long_wait_until(word, ROC_SHMEM_CMP_LE, 5);
+    // *fword == -1.5f
+    results[k++] = roc_shmem_float_test(fword, ROC_SHMEM_CMP_LT, -1.0f);
+    results[k++] = roc_shmem_float_test(fword, ROC_SHMEM_CMP_GT, -1.0f);
+    roc_shmem_float_wait_until(fword, ROC_SHMEM_CMP_EQ, -1.5f);
+    results[k++] = 77;
+  }
+  roc_shmem_wg_finalize();
+}
+
+static void compare_ops() {
+  current_case = "wait_until / test comparisons";
+  long *word = static_cast<long *>(roc_shmem_malloc(sizeof(long)));
+  float *fword = static_cast<float *>(roc_shmem_malloc(sizeof(float)));
+  int *results = nullptr;
+  (void)hipMalloc(reinterpret_cast<void **>(&results), 32 * sizeof(int));
+  (void)hipMemset(results, 0xff, 32 * sizeof(int));
+  roc_shmem_long_p(word, 5, 0);
+  roc_shmem_float_p(fword, -1.5f, 0);
+  CompareTest<<<npes, 64>>>(word, fword, results);
+  finish_kernel("CompareTest");
+  int got[15];
+  (void)hipMemcpy(got, results, sizeof(got), hipMemcpyDeviceToHost);
+  const int want[15] = {1, 0, 1, 0, 1, 0, 1, 0, 1, 0, 1, 0, 1, 0, 77};
+  for (int i = 0; i < 15; ++i) EXPECT(got[i] == want[i], "result %d = %d, expected %d", i, got[i], want[i]);
+  (void)hipFree(results);
+  roc_shmem_free(fword);
+  roc_shmem_free(word);
+}
+
+// ---- shmem_ptr_tester.cpp:31-44 ------------------------------------------------------------------
+__global__ void ShmemPtrTest(char *r_buf, int *available) {
+  roc_shmem_wg_init();
+  if (threadIdx.x == 0 && roc_shmem_my_pe() == 0) {
+    char *local_addr = roc_shmemx_my_addr(r_buf) + 4;
+    void *remote_addr = roc_shmem_ptr(local_addr, 1);
+    if (remote_addr != NULL) {
+      *available = 1;
+      static_cast<char *>(remote_addr)[0] = '1';
+    }
+  }
+  roc_shmem_wg_finalize();
+}
+
+static void shmem_ptr() {
+  current_case = "shmem_ptr_tester.cpp";
+  char *r_buf = static_cast<char *>(roc_shmem_malloc(64));
+  int *available = nullptr;
+  (void)hipMalloc(reinterpret_cast<void **>(&available), sizeof(int));
+  (void)hipMemset(available, 0, sizeof(int));
+  for (int pe = 0; pe < npes; ++pe) fill(r_buf, 64, '0', pe);
+  ShmemPtrTest<<<npes, 64>>>(r_buf, available);
+  finish_kernel("ShmemPtrTest");
+  int avail = 0;
+  (void)hipMemcpy(&avail, available, sizeof(int), hipMemcpyDeviceToHost);
+  EXPECT(avail == 1, "every slice is directly addressable here");
+  for (int pe = 0; pe < npes; ++pe) {
+    std::vector<char> got = load(r_buf, 64, pe);
+    for (int i = 0; i < 64; ++i)
+      EXPECT(got[i] == ((pe == 1 && i == 4) ? '1' : '0'), "PE %d byte %d = %c", pe, i, got[i]);
+  }
+  (void)hipFree(available);
+  roc_shmem_free(r_buf);
+}
+
+// ---- team_ctx_infra_tester.cpp:41-90 ---------------------------------------------------------------
+#define NUM_TEAMS 39  // ROC_SHMEM_MAX_NUM_TEAMS - 1
+__global__ void TeamCtxInfraTest(roc_shmem_team_t *team, int *errors) {
+  __shared__ roc_shmem_ctx_t ctx1, ctx2, ctx3;
+  __shared__ roc_shmem_ctx_t ctx[NUM_TEAMS];
+  roc_shmem_wg_init();
+  roc_shmem_wg_team_create_ctx(team[0], ROC_SHMEM_CTX_WG_PRIVATE, &ctx1);
+  roc_shmem_wg_team_create_ctx(team[0], ROC_SHMEM_CTX_WG_PRIVATE, &ctx2);
+  roc_shmem_wg_ctx_destroy(ctx1);
+  roc_shmem_wg_team_create_ctx(team[0], ROC_SHMEM_CTX_WG_PRIVATE, &ctx3);
+  __syncthreads();
+  if (ctx3.team_opaque != ctx2.team_opaque) atomicAdd(errors, 1);
+  roc_shmem_wg_ctx_destroy(ctx2);
+  roc_shmem_wg_ctx_destroy(ctx3);
+  __syncthreads();
+  for (int team_i = 0; team_i < NUM_TEAMS; team_i++)
+    roc_shmem_wg_team_create_ctx(team[team_i], ROC_SHMEM_CTX_WG_PRIVATE, &ctx[team_i]);
+  if (ctx[0].team_opaque == ctx[NUM_TEAMS - 1].team_opaque) atomicAdd(errors, 1);
+  for (int a = 0; a < NUM_TEAMS; a++)
+    for (int b = a + 1; b < NUM_TEAMS; b++)
+      if (threadIdx.x == 0 && ctx[a].team_opaque == ctx[b].team_opaque) atomicAdd(errors, 1);
+  __syncthreads();
+  for (int team_i = 0; team_i < NUM_TEAMS; team_i++) roc_shmem_wg_ctx_destroy(ctx[team_i]);
+  // an invalid team is refused (roc_shmem_gpu.cpp:269-274)
+  if (roc_shmem_wg_team_create_ctx(ROC_SHMEM_TEAM_INVALID, ROC_SHMEM_CTX_WG_PRIVATE, &ctx1) != -1)
+    atomicAdd(errors, 1);
+  roc_shmem_wg_finalize();
+}
+
+static void team_ctx_infra() {
+  current_case = "team_ctx_infra_tester.cpp";
+  roc_shmem_team_t dup[NUM_TEAMS];
+  for (int i = 0; i < NUM_TEAMS; ++i) {
+    dup[i] = ROC_SHMEM_TEAM_INVALID;
+    roc_shmem_team_split_strided(ROC_SHMEM_TEAM_WORLD, 0, 1, npes, nullptr, 0, &dup[i]);
+    EXPECT(dup[i] != ROC_SHMEM_TEAM_INVALID, "team %d is invalid", i);
+  }
+  roc_shmem_team_t *dev_teams = nullptr;
+  int *errors = nullptr;
+  (void)hipMalloc(reinterpret_cast<void **>(&dev_teams), sizeof(dup));
+  (void)hipMemcpy(dev_teams, dup, sizeof(dup), hipMemcpyHostToDevice);
+  (void)hipMalloc(reinterpret_cast<void **>(&errors), sizeof(int));
+  (void)hipMemset(errors, 0, sizeof(int));
+  TeamCtxInfraTest<<<npes * 2, 64>>>(dev_teams, errors);
+  finish_kernel("TeamCtxInfraTest");
+  int n = -1;
+  (void)hipMemcpy(&n, errors, sizeof(int), hipMemcpyDeviceToHost);
+  EXPECT(n == 0, "%d context/team identity errors", n);
+  for (int i = 0; i < NUM_TEAMS; ++i) roc_shmem_team_destroy(dup[i]);
+  (void)hipFree(errors);
+  (void)hipFree(dev_teams);
+}
+
+// ---- team_ctx_primitive_tester.cpp:33-68: put / get through a team context; PE numbers are the
+// team's.  The team here is {1, 3} of the world, so team PE 1 is world PE 3.
+__global__ void TeamCtxPrimitiveTest(char *s_buf, char *r_buf, int size, int type,
+                                     roc_shmem_team_t team) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_team_create_ctx(team, ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  s_buf = roc_shmemx_my_addr(s_buf);
+  r_buf = roc_shmemx_my_addr(r_buf);
+  if (threadIdx.x == 0 && roc_shmem_my_pe() == 1) {   // team PE 0
+    switch (type) {
+      case 0: roc_shmem_ctx_getmem(ctx, r_buf, s_buf, size, 1); break;
+      case 1: roc_shmem_ctx_getmem_nbi(ctx, r_buf, s_buf, size, 1); break;
+      case 2: roc_shmem_ctx_putmem(ctx, r_buf, s_buf, size, 1); break;
+      default: roc_shmem_ctx_putmem_nbi(ctx, r_buf, s_buf, size, 1); break;
+    }
+    roc_shmem_ctx_quiet(ctx);
+  }
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+static void team_ctx_primitive() {
+  current_case = "team_ctx_primitive_tester.cpp";
+  if (npes < 4) return;
+  const int size = 1000;
+  char *s_buf = static_cast<char *>(roc_shmem_malloc(size));
+  char *r_buf = static_cast<char *>(roc_shmem_malloc(size));
+  roc_shmem_team_t team = ROC_SHMEM_TEAM_INVALID;
+  roc_shmem_team_split_strided(ROC_SHMEM_TEAM_WORLD, 1, 2, 2, nullptr, 0, &team);
+  EXPECT(team != ROC_SHMEM_TEAM_INVALID, "split {1, 3}");
+  for (int type = 0; type < 4; ++type) {
+    for (int pe = 0; pe < npes; ++pe) {
+      fill(s_buf, size, static_cast<char>('a' + pe), pe);
+      fill(r_buf, size, '1', pe);
+    }
+    TeamCtxPrimitiveTest<<<npes, 64>>>(s_buf, r_buf, size, type, team);
+    finish_kernel("TeamCtxPrimitiveTest");
+    const bool is_get = type < 2;
+    for (int pe = 0; pe < npes; ++pe) {
+      // get: world PE 1 receives PE 3's source; put: world PE 3 receives PE 1's source
+      char want = '1';
+      if (is_get && pe == 1) want = 'a' + 3;
+      if (!is_get && pe == 3) want = 'a' + 1;
+      std::vector<char> got = load(r_buf, size, pe);
+      for (int i = 0; i < size; ++i) EXPECT(got[i] == want, "type %d PE %d byte %d = %c", type, pe, i, got[i]);
+    }
+  }
+  roc_shmem_team_destroy(team);
+  roc_shmem_free(r_buf);
+  roc_shmem_free(s_buf);
+}
+
+// ---- sync_tester.cpp:33-63 and barrier_all_tester.cpp: loops of sync_all / team_sync / barrier_all,
+// here with a hand-off in every round so that a barrier that lets a PE through early is seen.
+__global__ void SyncTest(int loop, int type, long *slot, roc_shmem_team_t team, int *errors) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  slot = roc_shmemx_my_addr(slot) + wg_index();
+  const int me = roc_shmem_ctx_my_pe(ctx);
+  const int n = roc_shmem_ctx_n_pes(ctx);
+  for (int i = 1; i <= loop; i++) {
+    if (threadIdx.x == 0) {
+      roc_shmem_ctx_long_p(ctx, slot, 1000L * me + i, (me + 1) % n);
+      roc_shmem_ctx_quiet(ctx);
+    }
+    switch (type) {
+      case 0: roc_shmem_ctx_wg_sync_all(ctx); break;
+      case 1: roc_shmem_ctx_wg_team_sync(ctx, team); break;
+      default: roc_shmem_ctx_wg_barrier_all(ctx); break;
+    }
+    if (threadIdx.x == 0 && roc_shmem_ctx_long_g(ctx, slot, me) != 1000L * ((me + n - 1) % n) + i)
+      atomicAdd(errors, 1);
+    // nobody overwrites a slot before its owner has looked at it
+    switch (type) {
+      case 0: roc_shmem_ctx_wg_sync_all(ctx); break;
+      case 1: roc_shmem_ctx_wg_team_sync(ctx, team); break;
+      default: roc_shmem_ctx_wg_barrier_all(ctx); break;
+    }
+  }
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+static void sync_and_barrier() {
+  current_case = "sync_tester.cpp / barrier_all_tester.cpp";
+  const int wgs = 3, loop = 50;
+  long *slot = static_cast<long *>(roc_shmem_malloc(sizeof(long) * wgs));
+  int *errors = nullptr;
+  (void)hipMalloc(reinterpret_cast<void **>(&errors), sizeof(int));
+  roc_shmem_team_t dup = ROC_SHMEM_TEAM_INVALID;
+  roc_shmem_team_split_strided(ROC_SHMEM_TEAM_WORLD, 0, 1, npes, nullptr, 0, &dup);
+  for (int type = 0; type < 3; ++type) {
+    (void)hipMemset(errors, 0, sizeof(int));
+    for (int pe = 0; pe < npes; ++pe) fill(slot, wgs, -1L, pe);
+    SyncTest<<<npes * wgs, 128>>>(loop, type, slot, dup, errors);
+    finish_kernel("SyncTest");
+    int n = -1;
+    (void)hipMemcpy(&n, errors, sizeof(int), hipMemcpyDeviceToHost);
+    EXPECT(n == 0, "type %d: %d hand-offs seen too early or too late", type, n);
+  }
+  roc_shmem_team_destroy(dup);
+  (void)hipFree(errors);
+  roc_shmem_free(slot);
+}
+
+// ---- swarm_tester.cpp:31-58: every thread of PE 0's workgroup gets its own chunk from PE 1 -------
+__global__ void GetSwarmTest(int loop, char *s_buf, char *r_buf, int size) {
+  __shared__ roc_shmem_ctx_t ctx;
+  int provided;
+  roc_shmem_wg_init_thread(ROC_SHMEM_THREAD_MULTIPLE, &provided);
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  __syncthreads();
+  s_buf = roc_shmemx_my_addr(s_buf);
+  r_buf = roc_shmemx_my_addr(r_buf);
+  int index = threadIdx.x * size;
+  if (roc_shmem_ctx_my_pe(ctx) == 0 && provided == ROC_SHMEM_THREAD_MULTIPLE) {
+    for (int i = 0; i < loop; i++) {
+      roc_shmem_ctx_getmem(ctx, &r_buf[index], &s_buf[index], size, 1);
+      __syncthreads();
+    }
+  }
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+static void swarm() {
+  current_case = "swarm_tester.cpp";
+  const int wg_size = 256;
+  for (int size : {1, 4, 8, 24, 100}) {
+    char *s_buf = static_cast<char *>(roc_shmem_malloc(size * wg_size));
+    char *r_buf = static_cast<char *>(roc_shmem_malloc(size * wg_size));
+    for (int pe = 0; pe < npes; ++pe) {
+      fill(s_buf, size * wg_size, pe == 1 ? '0' : 'x', pe);
+      fill(r_buf, size * wg_size, '1', pe);
+    }
+    GetSwarmTest<<<npes, wg_size>>>(3, s_buf, r_buf, size);
+    finish_kernel("GetSwarmTest");
+    for (char c : load(r_buf, size * wg_size, 0)) EXPECT(c == '0', "size %d: got %c", size, c);
+    for (char c : load(r_buf, size * wg_size, 1)) EXPECT(c == '1', "size %d: PE 1 was written", size);
+    roc_shmem_free(r_buf);
+    roc_shmem_free(s_buf);
+  }
+}
+
+// ---- the context-less forms (ROC_SHMEM_CTX_DEFAULT; roc_shmem.hpp:907-1147) ------------------------
+__global__ void DefaultCtxTest(long *data, long *counter, int n) {
+  roc_shmem_wg_init();
+  data = roc_shmemx_my_addr(data);
+  counter = roc_shmemx_my_addr(counter);
+  const int me = roc_shmem_my_pe();
+  const int np = roc_shmem_n_pes();
+  if (threadIdx.x == 0) {
+    roc_shmem_long_p(&data[0], 10 + me, (me + 1) % np);
+    roc_shmem_putmem(&data[1], &data[n], sizeof(long) * 2, (me + 1) % np);  // data[n..n+1] -> neighbour's data[1..2]
+    roc_shmem_long_atomic_add(counter, me + 1, 0);
+    (void)roc_shmem_long_atomic_fetch_inc(counter + 1, 0);
+    roc_shmem_fence();
+    roc_shmem_quiet();
+  }
+  roc_shmem_wg_barrier_all();
+  if (threadIdx.x == 0) {
+    data[3] = roc_shmem_long_g(&data[0], (me + 1) % np);   // what the neighbour received from me
+    roc_shmem_getmem(&data[4], &data[1], sizeof(long) * 2, (me + 1) % np);
+  }
+  roc_shmem_wg_sync_all();
+  roc_shmem_wg_finalize();
+}
+
+static void default_ctx() {
+  current_case = "context-less device API";
+  const int n = 8;
+  long *data = static_cast<long *>(roc_shmem_malloc(sizeof(long) * (n + 2)));
+  long *counter = static_cast<long *>(roc_shmem_malloc(sizeof(long) * 2));
+  for (int pe = 0; pe < npes; ++pe) {
+    std::vector<long> v(n + 2, -1);
+    v[n] = 100 + pe;
+    v[n + 1] = 200 + pe;
+    roc_shmem_putmem(data, v.data(), sizeof(long) * (n + 2), pe);
+    fill(counter, 2, 0L, pe);
+  }
+  DefaultCtxTest<<<npes, 64>>>(data, counter, n);
+  finish_kernel("DefaultCtxTest");
+  for (int pe = 0; pe < npes; ++pe) {
+    const int left = (pe + npes - 1) % npes;
+    std::vector<long> got = load(data, n + 2, pe);
+    EXPECT(got[0] == 10 + left && got[1] == 100 + left && got[2] == 200 + left, "PE %d received %ld %ld %ld",
+           pe, got[0], got[1], got[2]);
+    EXPECT(got[3] == 10 + pe && got[4] == 100 + pe && got[5] == 200 + pe, "PE %d read back %ld %ld %ld", pe,
+           got[3], got[4], got[5]);
+  }
+  std::vector<long> c = load(counter, 2, 0);
+  EXPECT(c[0] == npes * (npes + 1) / 2 && c[1] == npes, "counters %ld %ld", c[0], c[1]);
+  roc_shmem_free(counter);
+  roc_shmem_free(data);
+}
+
+int main() {
+  if (!getenv("ROC_SHMEM_NUM_PES")) setenv("ROC_SHMEM_NUM_PES", "4", 1);
+  setenv("ROC_SHMEM_HEAP_SIZE", "67108864", 0);
+  roc_shmem_init();
+  npes = roc_shmem_n_pes();
+  struct {
+    const char *name;
+    void (*run)();
+  } cases[] = {{"ping_pong", ping_pong},       {"compare_ops", compare_ops},
+               {"shmem_ptr", shmem_ptr},       {"team_ctx_infra", team_ctx_infra},
+               {"team_ctx_primitive", team_ctx_primitive}, {"sync_and_barrier", sync_and_barrier},
+               {"swarm", swarm},               {"default_ctx", default_ctx}};
+  for (auto &c : cases) {
+    const int before = failures;
+    c.run();
+    printf("%-20s %s\n", c.name, failures == before ? "ok" : "FAILED");
+    fflush(stdout);
+  }
+  roc_shmem_finalize();
+  if (failures) {
+    printf("DEVICE_API_FAILED %d\n", failures);
+    return 1;
+  }
+  printf("DEVICE_API_OK\n");
+  return 0;
+}

@@ -16,6 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 BINARY = os.path.join(HERE, "cxx", "host_api_check")
 SOS_BINARY = os.path.join(HERE, "cxx", "sos_cases")
+DEVICE_BINARY = os.path.join(HERE, "cxx", "device_api_cases")
 
 
 def newest_header():
@@ -28,7 +29,7 @@ def test_check_program_is_not_older_than_the_headers_it_inlines():
     # The device interface is header-only: a program built before a header changed carries
     # device code for the old state layout.  (The library refuses to initialise for such a
     # program; this catches it before anything runs.)
-    for binary in (BINARY, SOS_BINARY):
+    for binary in (BINARY, SOS_BINARY, DEVICE_BINARY):
         if not os.path.exists(binary):
             pytest.skip("%s is not built yet" % binary)
         assert os.path.getmtime(binary) >= newest_header(), \
@@ -60,3 +61,17 @@ def test_reference_host_programs_restated(num_pes):
     tail = (out.stdout + out.stderr)[-3000:]
     assert out.returncode == 0, tail
     assert "SOS_CASES_OK" in out.stdout, tail
+
+
+@pytest.mark.gpu
+def test_reference_functional_testers_restated():
+    # tests/cxx/device_api_cases.cpp: user kernels in the style of clients/functional_tests.
+    if not os.path.exists(DEVICE_BINARY):
+        pytest.fail("tests/cxx/device_api_cases is not built: run __graft_entry__.build()")
+    assert os.path.getmtime(DEVICE_BINARY) >= newest_header(), "stale check program: run __graft_entry__.build()"
+    print("running", DEVICE_BINARY, flush=True)
+    out = subprocess.run([DEVICE_BINARY], capture_output=True, text=True, timeout=110)
+    tail = (out.stdout + out.stderr)[-3000:]
+    print(out.stdout[-1500:], flush=True)
+    assert out.returncode == 0, tail
+    assert "DEVICE_API_OK" in out.stdout, tail
