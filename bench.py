@@ -74,13 +74,13 @@ def device_report():
 
 
 def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, cpu=False,
-                 spread=False):
+                 spread=False, launch_shape=None):
     """Returns a dict with ms_per_step, GB/s (algorithmic 2*P*N*s bytes) and optional CPU figures."""
     npd = rs.NP_DTYPE[dtype]
     es = np.dtype(npd).itemsize
     src = rs.sym_array(n, npd)
     dst = rs.sym_array(n, npd, fill=0x5A)
-    launch = rs.Launch(**TO_ALL_LAUNCH)
+    launch = rs.Launch(**(launch_shape or TO_ALL_LAUNCH))
     psync = rs.sym_array(launch.wgs_per_pe * rs.ROC_SHMEM_REDUCE_SYNC_SIZE, np.int64, fill=0)
     rng = np.random.default_rng(seed)
     host = []
@@ -309,7 +309,17 @@ def main():
 
     if not args.quick:
         rs.roc_shmem_init(4, 64 << 20, 64, 1024)
-        extra["to_all_int64_sum_4x2^20"] = bench_to_all(rs, oracle, 20, 5, rs.LONG, 4, 1 << 20, seed=1)
+        # 64 MiB of traffic: launch, two flag barriers and 12 us of streaming; fewer workgroups win
+        extra["to_all_int64_sum_4x2^20"] = bench_to_all(rs, oracle, 50, 10, rs.LONG, 4, 1 << 20, seed=1,
+                                                        launch_shape=dict(wgs_per_pe=32, wg_size=512))
+        barrier_launch, rounds = rs.Launch(1, 256), 500
+
+        def barriers():
+            rs.roc_shmem_wg_barrier_all(rounds, barrier_launch)
+
+        barriers()
+        rs.synchronize()
+        extra["wg_barrier_all_4pe_us"] = event_time_ms(rs, barriers, 3) / 3 / rounds * 1e3
         rs.roc_shmem_finalize()
 
         rs.roc_shmem_init(16, 256 << 20, 64, 1024)
