@@ -31,7 +31,7 @@ HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
 MEASURED_TRAFFIC_BYTES = 4296790021
 
 # Launch shapes chosen by measurement on MI355X (256 CUs).
-TO_ALL_LAUNCH = dict(wgs_per_pe=64, wg_size=512)
+TO_ALL_LAUNCH = dict(wgs_per_pe=32, wg_size=1024)
 PUT_LAUNCH = dict(wgs_per_pe=32, wg_size=512)
 PUT_TILE = 256 << 10
 

@@ -87,7 +87,7 @@ typedef struct rsm_small_op {
 typedef struct rsm_launch {
   int wgs_per_pe;   /* workgroups acting for each PE (>= 1)                        */
   int wg_size;      /* threads per workgroup, multiple of 64, <= 1024              */
-  size_t tile;      /* elements (or bytes) per device call; 0 = split evenly       */
+  size_t tile;      /* elements (or bytes) per device call; 0 = chosen by the entry point */
   void *stream;     /* hipStream_t, NULL = the default stream                      */
 } rsm_launch_t;
 
@@ -138,11 +138,14 @@ int rsm_event_elapsed_ms(void *start, void *stop, float *ms);   /* synchronises 
 
 /* ---- reductions ------------------------------------------------------------
  * roc_shmem_ctx_<T>_<op>_wg_to_all, active-set form (roc_shmem.hpp:837-851;
- * GPUIBContext::to_all, gpu_ib/context_ib_tmpl_device.hpp:262-307).  Workgroup w
- * of every member PE reduces tiles w, w+wgs_per_pe, ... of `launch->tile`
- * elements with its own pSync slice pSync + w*256.  `pSync` therefore holds
- * wgs_per_pe*256 longs, all ROC_SHMEM_SYNC_VALUE on entry and on return;
- * `pWrk` may be NULL (it is not used). */
+ * GPUIBContext::to_all, gpu_ib/context_ib_tmpl_device.hpp:262-307).  With
+ * `launch->tile` > 0, workgroup w of every member PE makes one standard call
+ * per tile w, w+wgs_per_pe, ... of `launch->tile` elements.  With tile == 0 the
+ * PE's workgroups share a single reduction through the sharded extension
+ * (roc_shmemx_ctx_<T>_<op>_wg_to_all_shard: passes of the whole range dealt
+ * round-robin to members and workgroups).  Either way workgroup w uses its own
+ * pSync slice pSync + w*256: `pSync` holds wgs_per_pe*256 longs, all
+ * ROC_SHMEM_SYNC_VALUE on entry and on return; `pWrk` may be NULL (unused). */
 int rsm_to_all(int dtype, int op, void *dest, const void *source, size_t nreduce, int pe_start,
                int log_pe_stride, int pe_size, void *pWrk, long *pSync,
                const rsm_launch_t *launch);

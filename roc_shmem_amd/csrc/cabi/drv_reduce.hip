@@ -25,6 +25,20 @@ struct ToAll;
                                                 T *dest, const T *source, int n) {            \
       roc_shmem_ctx_##TNAME##_##OPNAME##_wg_to_all(ctx, team, dest, source, n);               \
     }                                                                                         \
+    static __device__ __forceinline__ void active_set_shard(                                  \
+        roc_shmem_ctx_t ctx, T *dest, const T *source, size_t n, int pe_start, int log_stride, \
+        int pe_size, T *pWrk, long *pSync, int shard, int nshards) {                          \
+      roc_shmemx_ctx_##TNAME##_##OPNAME##_wg_to_all_shard(ctx, dest, source, n, pe_start,     \
+                                                          log_stride, pe_size, pWrk, pSync,   \
+                                                          shard, nshards);                    \
+    }                                                                                         \
+    static __device__ __forceinline__ void team_shard(roc_shmem_ctx_t ctx,                    \
+                                                      roc_shmem_team_t team, T *dest,         \
+                                                      const T *source, size_t n, int shard,   \
+                                                      int nshards) {                          \
+      roc_shmemx_ctx_##TNAME##_##OPNAME##_wg_to_all_shard(ctx, team, dest, source, n, shard,  \
+                                                          nshards);                           \
+    }                                                                                         \
   };
 #define RSM_TO_ALL_ARITH(T, TNAME)            \
   RSM_TO_ALL(T, TNAME, sum, ROC_SHMEM_SUM)    \
@@ -68,10 +82,17 @@ __global__ void __launch_bounds__(1024)
     const T *source = roc_shmemx_my_addr(source0);
     T *pWrk = roc_shmemx_my_addr(pWrk0);
     long *pSync = roc_shmemx_my_addr(pSync0) + w * ROC_SHMEM_REDUCE_SYNC_SIZE;
-    for (size_t off = w * tile; off < n; off += nw * tile) {
-      size_t cnt = n - off < tile ? n - off : tile;
-      ToAll<T, Op>::active_set(ctx, dest + off, source + off, static_cast<int>(cnt), pe_start,
-                               log_stride, pe_size, pWrk, pSync);
+    if (tile == 0) {
+      // one reduction shared by the PE's workgroups (sharded extension)
+      ToAll<T, Op>::active_set_shard(ctx, dest, source, n, pe_start, log_stride, pe_size, pWrk,
+                                     pSync, static_cast<int>(w), static_cast<int>(nw));
+    } else {
+      // one standard call per tile, tiles dealt round-robin to the PE's workgroups
+      for (size_t off = w * tile; off < n; off += nw * tile) {
+        size_t cnt = n - off < tile ? n - off : tile;
+        ToAll<T, Op>::active_set(ctx, dest + off, source + off, static_cast<int>(cnt), pe_start,
+                                 log_stride, pe_size, pWrk, pSync);
+      }
     }
   }
   roc_shmem_wg_ctx_destroy(ctx);
@@ -94,9 +115,14 @@ __global__ void __launch_bounds__(1024)
   if (member) {
     T *dest = roc_shmemx_my_addr(dest0);
     const T *source = roc_shmemx_my_addr(source0);
-    for (size_t off = w * tile; off < n; off += nw * tile) {
-      size_t cnt = n - off < tile ? n - off : tile;
-      ToAll<T, Op>::team(ctx, team, dest + off, source + off, static_cast<int>(cnt));
+    if (tile == 0) {
+      ToAll<T, Op>::team_shard(ctx, team, dest, source, n, static_cast<int>(w),
+                               static_cast<int>(nw));
+    } else {
+      for (size_t off = w * tile; off < n; off += nw * tile) {
+        size_t cnt = n - off < tile ? n - off : tile;
+        ToAll<T, Op>::team(ctx, team, dest + off, source + off, static_cast<int>(cnt));
+      }
     }
   }
   roc_shmem_wg_ctx_destroy(ctx);
@@ -171,10 +197,8 @@ int run(int dtype, int op, const rsm::Launch &l, ReduceArgs a) {
   const size_t es = dtype_size(dtype);
   if (!es) return rsm::fail("to_all: unknown dtype");
   if (a.n == 0) return 0;  // zero-element reductions are no-ops (context_tmpl_device.hpp:68-70)
-  if (a.tile == 0) {
-    size_t t = (a.n + l.wgs_per_pe - 1) / l.wgs_per_pe;
-    a.tile = (t + 1023) / 1024 * 1024;
-  }
+  // tile == 0: the PE's workgroups share one reduction through the sharded
+  // extension; otherwise each standard call covers `tile` elements.
   if (a.tile > 0x7fffffffull) return rsm::fail("to_all: tile does not fit the API's int nreduce");
   bool ok = false;
   switch (dtype) {

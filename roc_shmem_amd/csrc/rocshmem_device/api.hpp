@@ -395,34 +395,57 @@ ROCSHMEM_STANDARD_TYPES(ROCSHMEM_TYPED_RMA_GRAN_ALL)
 namespace detail {
 template <typename T, ROC_SHMEM_OP Op>
 __device__ __forceinline__ void to_all_active_set(roc_shmem_ctx_t ctx, T *dest, const T *source,
-                                                  int nreduce, int pe_start, int log_stride,
-                                                  int pe_size, long *psync) {
+                                                  size_t nreduce, int pe_start, int log_stride,
+                                                  int pe_size, long *psync, int shard = 0,
+                                                  int nshards = 1) {
   wg_all_reduce<T, Op>(ctx_of(ctx)->my_pe, dest, source, nreduce, pe_start, log_stride, pe_size,
-                       psync);
+                       psync, shard, nshards);
 }
 // reference: GPUIBContext::to_all(team, ...), context_ib_tmpl_device.hpp:238-260
 template <typename T, ROC_SHMEM_OP Op>
 __device__ __forceinline__ void to_all_team(roc_shmem_ctx_t ctx, roc_shmem_team_t team, T *dest,
-                                            const T *source, int nreduce) {
+                                            const T *source, size_t nreduce, int shard = 0,
+                                            int nshards = 1) {
   const DeviceCtx *c = ctx_of(ctx);
   const Team *t = team_of(team);
   wg_all_reduce<T, Op>(c->my_pe, dest, source, nreduce, t->wrt_world.pe_start,
                        t->wrt_world.log_stride, t->wrt_world.size,
-                       team_psync(c, t->reduce_psync_off));
+                       team_psync(c, t->reduce_psync_off), shard, nshards);
 }
 }  // namespace detail
 
+// The _shard forms are an extension: `nshards` workgroups of every member PE
+// share one reduction.  All of them pass the same dest / source / nreduce
+// (a size_t here) and their own shard number; shard s uses its own pSync
+// (active-set form) or the pSync slice of its context's block (team form).
+// Every source must be complete before any workgroup of that PE calls, and a
+// destination is complete only when all shards have returned (at the latest
+// when the kernel ends).
 #define ROCSHMEM_REDUCTION(T, TNAME, OPNAME, OP)                                              \
   __device__ inline void roc_shmem_ctx_##TNAME##_##OPNAME##_wg_to_all(                         \
       roc_shmem_ctx_t ctx, T *dest, const T *source, int nreduce, int PE_start,                \
       int logPE_stride, int PE_size, T *pWrk, long *pSync) {                                   \
     (void)pWrk;                                                                                \
-    detail::to_all_active_set<T, OP>(ctx, dest, source, nreduce, PE_start, logPE_stride,       \
-                                     PE_size, pSync);                                          \
+    if (nreduce <= 0) return;                                                                  \
+    detail::to_all_active_set<T, OP>(ctx, dest, source, static_cast<size_t>(nreduce),          \
+                                     PE_start, logPE_stride, PE_size, pSync);                  \
   }                                                                                            \
   __device__ inline void roc_shmem_ctx_##TNAME##_##OPNAME##_wg_to_all(                         \
       roc_shmem_ctx_t ctx, roc_shmem_team_t team, T *dest, const T *source, int nreduce) {     \
-    detail::to_all_team<T, OP>(ctx, team, dest, source, nreduce);                              \
+    if (nreduce <= 0) return;                                                                  \
+    detail::to_all_team<T, OP>(ctx, team, dest, source, static_cast<size_t>(nreduce));         \
+  }                                                                                            \
+  __device__ inline void roc_shmemx_ctx_##TNAME##_##OPNAME##_wg_to_all_shard(                  \
+      roc_shmem_ctx_t ctx, T *dest, const T *source, size_t nreduce, int PE_start,             \
+      int logPE_stride, int PE_size, T *pWrk, long *pSync, int shard, int nshards) {           \
+    (void)pWrk;                                                                                \
+    detail::to_all_active_set<T, OP>(ctx, dest, source, nreduce, PE_start, logPE_stride,       \
+                                     PE_size, pSync, shard, nshards);                          \
+  }                                                                                            \
+  __device__ inline void roc_shmemx_ctx_##TNAME##_##OPNAME##_wg_to_all_shard(                  \
+      roc_shmem_ctx_t ctx, roc_shmem_team_t team, T *dest, const T *source, size_t nreduce,    \
+      int shard, int nshards) {                                                                \
+    detail::to_all_team<T, OP>(ctx, team, dest, source, nreduce, shard, nshards);              \
   }
 #define ROCSHMEM_ARITH_REDUCTIONS(T, TNAME)            \
   ROCSHMEM_REDUCTION(T, TNAME, sum, ROC_SHMEM_SUM)     \

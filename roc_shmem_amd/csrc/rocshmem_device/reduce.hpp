@@ -161,7 +161,8 @@ struct ActiveSet {
 template <typename T, ROC_SHMEM_OP Op, int U = kReduceUnroll, int C = kReducePeChunk>
 __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_begin,
                                                size_t v_end, const ActiveSet &as, int my_pe,
-                                               uint32_t tid, uint32_t nthr) {
+                                               uint32_t tid, uint32_t nthr, size_t first_pass = 0,
+                                               size_t pass_step = 1) {
   using Acc = typename AccOf<T, Op>::type;
   using V = VecOf<T>;
   constexpr int E = V::kElems;
@@ -179,7 +180,9 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
   const uint32_t pass_bytes = access_bytes * U;   // at most 128 KiB
   const size_t byte_end = v_end * 16;
 
-  for (size_t b = v_begin * 16; b < byte_end; b += pass_bytes) {
+  // This workgroup takes passes first_pass, first_pass + pass_step, ... of the range.
+  const size_t step_bytes = pass_step * pass_bytes;
+  for (size_t b = v_begin * 16 + first_pass * pass_bytes; b < byte_end; b += step_bytes) {
     const size_t left = byte_end - b;
     const int valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
     Acc acc[U][E];
@@ -272,9 +275,9 @@ __device__ __forceinline__ void reduce_elements(T *dst, const T *src, size_t e_b
 // needed.  dest == source (in place) is allowed: a share is read and then
 // overwritten by the same lanes.
 template <typename T, ROC_SHMEM_OP Op>
-__device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *source, int nreduce,
+__device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *source, size_t nreduce,
                                               int pe_start, int log_stride, int pe_size,
-                                              long *psync) {
+                                              long *psync, int shard = 0, int nshards = 1) {
   // Workgroup-collective: every lane holds the same arguments.
   my_pe = uniform(my_pe);
   dest = uniform(dest);
@@ -284,8 +287,10 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
   log_stride = uniform(log_stride);
   pe_size = uniform(pe_size);
   psync = uniform(psync);
-  if (nreduce <= 0) return;  // reference: Context::to_all early-out, context_tmpl_device.hpp:68-70
-  if (pe_size > kMaxPes || pe_size <= 0) {
+  shard = uniform(shard);
+  nshards = uniform(nshards);
+  if (nreduce == 0) return;  // reference: Context::to_all early-out, context_tmpl_device.hpp:68-70
+  if (pe_size > kMaxPes || pe_size <= 0 || nshards <= 0 || shard < 0 || shard >= nshards) {
     status_raise(kStatusBadArgument);
     return;
   }
@@ -293,7 +298,11 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
   const int my_idx = (my_pe - pe_start) >> log_stride;
   const uint32_t tid = flat_thread_id();
   const uint32_t nthr = flat_block_size();
-  const size_t n = static_cast<size_t>(nreduce);
+  const size_t n = nreduce;
+  // The range is dealt to pe_size * nshards workgroups: member k's workgroup
+  // of shard s is part s * pe_size + k.
+  const size_t parts = static_cast<size_t>(pe_size) * nshards;
+  const size_t part = static_cast<size_t>(shard) * pe_size + my_idx;
 
   wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, log_stride, pe_size);
 
@@ -302,18 +311,30 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
       ((reinterpret_cast<uintptr_t>(dest) | reinterpret_cast<uintptr_t>(source)) & 15u) == 0;
   if (aligned) {
     const size_t nvec = n / E;
-    const size_t share = (nvec + pe_size - 1) / pe_size;
-    size_t v0 = share * my_idx;
-    size_t v1 = v0 + share;
-    if (v0 > nvec) v0 = nvec;
-    if (v1 > nvec) v1 = nvec;
-    reduce_vectors<T, Op>(dest, source, v0, v1, as, my_pe, tid, nthr);
-    if (my_idx == pe_size - 1 && nvec * E < n) {
+    if (nshards == 1) {
+      // One workgroup per member: member k takes the k-th contiguous share.
+      const size_t share = (nvec + pe_size - 1) / pe_size;
+      size_t v0 = share * my_idx;
+      size_t v1 = v0 + share;
+      if (v0 > nvec) v0 = nvec;
+      if (v1 > nvec) v1 = nvec;
+      reduce_vectors<T, Op>(dest, source, v0, v1, as, my_pe, tid, nthr);
+    } else {
+      // Several workgroups per member: passes are dealt round-robin over all
+      // of them, so that the workgroups running at one moment sweep one
+      // compact window of every array.  Measured on MI355X (8 -> 8 fp32
+      // reduction, no barriers): 6.06 TB/s against 5.86 TB/s when every
+      // workgroup walks a region of its own; giving each member a contiguous
+      // share and striding only within it was no better and less even across
+      // launch shapes.
+      reduce_vectors<T, Op>(dest, source, 0, nvec, as, my_pe, tid, nthr, part, parts);
+    }
+    if (part == parts - 1 && nvec * E < n) {
       reduce_elements<T, Op>(dest, source, nvec * E, n, as, my_pe, tid, nthr);
     }
   } else {
-    const size_t share = (n + pe_size - 1) / pe_size;
-    size_t e0 = share * my_idx;
+    const size_t share = (n + parts - 1) / parts;
+    size_t e0 = share * part;
     size_t e1 = e0 + share;
     if (e0 > n) e0 = n;
     if (e1 > n) e1 = n;
