@@ -246,10 +246,11 @@ def bench_bcast_a2a(rs, n_pes, slice_bytes):
     src = rs.sym_array(slice_bytes, np.uint8, fill=3)
     dst = rs.sym_array(slice_bytes, np.uint8, fill=0)
     launch = rs.Launch(16, 512)
+    bcast_launch = rs.Launch(8, 1024)
     nelem = slice_bytes // 4
 
     def bcast():
-        rs.roc_shmem_team_broadcast(4, world, dst, src, nelem, 0, launch)
+        rs.roc_shmem_team_broadcast(4, world, dst, src, nelem, 0, bcast_launch)
 
     bcast()
     rs.synchronize()

@@ -26,6 +26,23 @@ __device__ __forceinline__ void bcast_team_call(roc_shmem_ctx_t c, roc_shmem_tea
 __device__ __forceinline__ void bcast_team_call(roc_shmem_ctx_t c, roc_shmem_team_t t, int *d, const int *s, int n, int root) { roc_shmem_ctx_int_wg_broadcast(c, t, d, s, n, root); }
 __device__ __forceinline__ void bcast_team_call(roc_shmem_ctx_t c, roc_shmem_team_t t, long *d, const long *s, int n, int root) { roc_shmem_ctx_long_wg_broadcast(c, t, d, s, n, root); }
 
+#define RSM_BCAST_SHARD(T, TNAME)                                                               \
+  __device__ __forceinline__ void bcast_shard_call(roc_shmem_ctx_t c, T *d, const T *s, size_t n, \
+                                                   int root, int ps, int ls, int sz, long *p,   \
+                                                   int sh, int nsh) {                           \
+    roc_shmemx_ctx_##TNAME##_wg_broadcast_shard(c, d, s, n, root, ps, ls, sz, p, sh, nsh);      \
+  }                                                                                             \
+  __device__ __forceinline__ void bcast_team_shard_call(roc_shmem_ctx_t c, roc_shmem_team_t t,  \
+                                                        T *d, const T *s, size_t n, int root,   \
+                                                        int sh, int nsh) {                      \
+    roc_shmemx_ctx_##TNAME##_wg_broadcast_shard(c, t, d, s, n, root, sh, nsh);                  \
+  }
+RSM_BCAST_SHARD(char, char)
+RSM_BCAST_SHARD(short, short)
+RSM_BCAST_SHARD(int, int)
+RSM_BCAST_SHARD(long, long)
+#undef RSM_BCAST_SHARD
+
 __device__ __forceinline__ void a2a_call(roc_shmem_ctx_t c, roc_shmem_team_t t, char *d, const char *s, int n, int sh, int nsh) { roc_shmemx_ctx_char_wg_alltoall_shard(c, t, d, s, n, sh, nsh); }
 __device__ __forceinline__ void a2a_call(roc_shmem_ctx_t c, roc_shmem_team_t t, short *d, const short *s, int n, int sh, int nsh) { roc_shmemx_ctx_short_wg_alltoall_shard(c, t, d, s, n, sh, nsh); }
 __device__ __forceinline__ void a2a_call(roc_shmem_ctx_t c, roc_shmem_team_t t, int *d, const int *s, int n, int sh, int nsh) { roc_shmemx_ctx_int_wg_alltoall_shard(c, t, d, s, n, sh, nsh); }
@@ -56,13 +73,24 @@ __global__ void __launch_bounds__(1024)
     T *dest = roc_shmemx_my_addr(dest0);
     const T *source = roc_shmemx_my_addr(source0);
     long *pSync = pSync0 ? roc_shmemx_my_addr(pSync0) + w * ROC_SHMEM_BCAST_SYNC_SIZE : nullptr;
-    for (size_t off = w * tile; off < n; off += nw * tile) {
-      size_t cnt = n - off < tile ? n - off : tile;
+    if (tile == 0) {
+      // one broadcast shared by the PE's workgroups (sharded extension)
       if (team) {
-        bcast_team_call(ctx, team, dest + off, source + off, static_cast<int>(cnt), pe_root);
+        bcast_team_shard_call(ctx, team, dest, source, n, pe_root, static_cast<int>(w),
+                              static_cast<int>(nw));
       } else {
-        bcast_call(ctx, dest + off, source + off, static_cast<int>(cnt), pe_root, pe_start,
-                   log_stride, pe_size, pSync);
+        bcast_shard_call(ctx, dest, source, n, pe_root, pe_start, log_stride, pe_size, pSync,
+                         static_cast<int>(w), static_cast<int>(nw));
+      }
+    } else {
+      for (size_t off = w * tile; off < n; off += nw * tile) {
+        size_t cnt = n - off < tile ? n - off : tile;
+        if (team) {
+          bcast_team_call(ctx, team, dest + off, source + off, static_cast<int>(cnt), pe_root);
+        } else {
+          bcast_call(ctx, dest + off, source + off, static_cast<int>(cnt), pe_root, pe_start,
+                     log_stride, pe_size, pSync);
+        }
       }
     }
   }
@@ -121,10 +149,7 @@ void launch_bcast(const rsm::Launch &l, const BcastArgs &a) {
 
 int run_bcast(size_t elem_size, const rsm::Launch &l, BcastArgs a) {
   if (a.n == 0) return 0;
-  if (a.tile == 0) {
-    size_t t = (a.n + l.wgs_per_pe - 1) / l.wgs_per_pe;
-    a.tile = (t + 1023) / 1024 * 1024;
-  }
+  // tile == 0: the PE's workgroups share one broadcast through the sharded extension.
   if (a.tile > 0x7fffffffull) return rsm::fail("broadcast: tile does not fit the API's int nelem");
   switch (elem_size) {
     case 1: launch_bcast<char>(l, a); break;

@@ -499,6 +499,25 @@ ROCSHMEM_REDUCTION(__hip_bfloat16, bf16, min, ROC_SHMEM_MIN)
                                pe_root, t->wrt_world.pe_start, t->wrt_world.log_stride,        \
                                t->wrt_world.size, detail::team_psync(c, t->bcast_psync_off));  \
   }                                                                                            \
+  /* extension: `nshards` workgroups of every member share one broadcast (same */              \
+  /* arguments in all of them, nelem a size_t; complete when all have returned) */             \
+  __device__ inline void roc_shmemx_ctx_##TNAME##_wg_broadcast_shard(                          \
+      roc_shmem_ctx_t ctx, T *dest, const T *source, size_t nelem, int pe_root, int pe_start,  \
+      int log_pe_stride, int pe_size, long *p_sync, int shard, int nshards) {                  \
+    detail::wg_broadcast_bytes(detail::ctx_of(ctx)->my_pe, dest, source, nelem * sizeof(T),    \
+                               pe_root, pe_start, log_pe_stride, pe_size, p_sync, shard,       \
+                               nshards);                                                       \
+  }                                                                                            \
+  __device__ inline void roc_shmemx_ctx_##TNAME##_wg_broadcast_shard(                          \
+      roc_shmem_ctx_t ctx, roc_shmem_team_t team, T *dest, const T *source, size_t nelem,      \
+      int pe_root, int shard, int nshards) {                                                   \
+    const detail::DeviceCtx *c = detail::ctx_of(ctx);                                          \
+    const detail::Team *t = detail::team_of(team);                                             \
+    detail::wg_broadcast_bytes(c->my_pe, dest, source, nelem * sizeof(T), pe_root,             \
+                               t->wrt_world.pe_start, t->wrt_world.log_stride,                 \
+                               t->wrt_world.size, detail::team_psync(c, t->bcast_psync_off),   \
+                               shard, nshards);                                                \
+  }                                                                                            \
   /* extension: move only part `shard` of `nshards` of every block */                          \
   __device__ inline void roc_shmemx_ctx_##TNAME##_wg_alltoall_shard(                           \
       roc_shmem_ctx_t ctx, roc_shmem_team_t team, T *dest, const T *source, int nelem,         \

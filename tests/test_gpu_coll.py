@@ -65,6 +65,26 @@ def test_broadcast_shrinking_and_strided_sets(pe_start, log_stride, pe_size, roo
         compare(n_pes, dst, heap, nelem * 8, nelem * 8)
 
 
+@pytest.mark.parametrize("wgs,wg_size,tile,shift", [(2, 256, 0, 4), (3, 128, 0, 0), (4, 512, 0, 4),
+                                                    (2, 256, 100000, 4), (2, 256, 0, (4, 5))])
+def test_broadcast_large_payload_shared_by_several_workgroups(wgs, wg_size, tile, shift):
+    # tile 0: the PE's workgroups share one broadcast pass by pass (mutually aligned arrays, here
+    # 4 bytes past a 16-byte boundary) or range by range (arrays misaligned against each other);
+    # tile > 0: one standard call per tile.  3 MiB + 13 bytes, bytes around the payload untouched.
+    n_pes, nbytes = 4, (3 << 20) + 13
+    s_shift, d_shift = shift if isinstance(shift, tuple) else (shift, shift)
+    with runtime(n_pes):
+        src, dst, heap = setup(n_pes, nbytes + 64, nbytes + 64, seed=77)
+        psync = rs.sym_array(256 * wgs, np.int64, fill=0)
+        rs.roc_shmem_broadcast(1, dst.addr + d_shift, src.addr + s_shift, nbytes, 2, 0, 0, n_pes, psync,
+                               rs.Launch(wgs, wg_size, tile))
+        rs.synchronize()
+        oracle.broadcast(heap, nbytes + 64 + d_shift, s_shift, nbytes, 2)
+        compare(n_pes, dst, heap, nbytes + 64, nbytes + 64)
+        for p in range(n_pes):
+            assert not psync.read(p).any()
+
+
 def test_broadcast_reference_pattern_and_team_form():
     # clients/functional_tests/tester.cpp:236-271: source 1, dest 2, non-roots read 1, root keeps 2
     n_pes, nelem = 4, 512
