@@ -25,10 +25,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
 
 # HBM bytes per launch of the headline kernel measured with rocprofv3 --pmc:
-# FETCH_SIZE 1 048 914.8 KiB and WRITE_SIZE 2 099 013.0 KiB per dispatch, each scaled by
+# FETCH_SIZE 1 048 810.1 KiB and WRITE_SIZE 2 099 768.7 KiB per dispatch, each scaled by
 # what the same counter reads for a wg-putmem copy of known size (2 GiB read, 2 GiB
-# written: 1 048 669.0 and 2 097 724.2 KiB); see profiles/to_all_float_sum_8pe_2e26.md.
-MEASURED_TRAFFIC_BYTES = 4296790021
+# written: 1 048 667.0 and 2 097 754.6 KiB); see profiles/to_all_float_sum_8pe_2e26.md.
+MEASURED_TRAFFIC_BYTES = 4297322185
 
 # Launch shapes chosen by measurement on MI355X (256 CUs).
 TO_ALL_LAUNCH = dict(wgs_per_pe=32, wg_size=1024)
