@@ -518,17 +518,15 @@ ROCSHMEM_REDUCTION(__hip_bfloat16, bf16, min, ROC_SHMEM_MIN)
                                t->wrt_world.size, detail::team_psync(c, t->bcast_psync_off),   \
                                shard, nshards);                                                \
   }                                                                                            \
-  /* extension: move only part `shard` of `nshards` of every block */                          \
+  /* extension: `nshards` workgroups of every member share the exchange */                        \
   __device__ inline void roc_shmemx_ctx_##TNAME##_wg_alltoall_shard(                           \
       roc_shmem_ctx_t ctx, roc_shmem_team_t team, T *dest, const T *source, int nelem,         \
       int shard, int nshards) {                                                                \
     if (nelem <= 0) return;                                                                    \
     const detail::DeviceCtx *c = detail::ctx_of(ctx);                                          \
     const detail::Team *t = detail::team_of(team);                                             \
-    size_t b, e;                                                                               \
-    detail::split_range(static_cast<size_t>(nelem) * sizeof(T), nshards, shard, 256, b, e);    \
     detail::wg_alltoall_bytes(c->my_pe, dest, source, static_cast<size_t>(nelem) * sizeof(T),  \
-                              b, e, t->wrt_world.pe_start, t->wrt_world.log_stride,            \
+                              shard, nshards, t->wrt_world.pe_start, t->wrt_world.log_stride,  \
                               t->wrt_world.size, detail::team_psync(c, t->alltoall_psync_off)); \
   }                                                                                            \
   __device__ inline void roc_shmem_ctx_##TNAME##_wg_alltoall(                                  \
@@ -541,10 +539,8 @@ ROCSHMEM_REDUCTION(__hip_bfloat16, bf16, min, ROC_SHMEM_MIN)
     if (nelem <= 0) return;                                                                    \
     const detail::DeviceCtx *c = detail::ctx_of(ctx);                                          \
     const detail::Team *t = detail::team_of(team);                                             \
-    size_t b, e;                                                                               \
-    detail::split_range(static_cast<size_t>(nelem) * sizeof(T), nshards, shard, 256, b, e);    \
     detail::wg_fcollect_bytes(c->my_pe, dest, source, static_cast<size_t>(nelem) * sizeof(T),  \
-                              b, e, t->wrt_world.pe_start, t->wrt_world.log_stride,            \
+                              shard, nshards, t->wrt_world.pe_start, t->wrt_world.log_stride,  \
                               t->wrt_world.size, detail::team_psync(c, t->alltoall_psync_off)); \
   }                                                                                            \
   __device__ inline void roc_shmem_ctx_##TNAME##_wg_fcollect(                                  \

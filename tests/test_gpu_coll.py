@@ -134,6 +134,29 @@ def test_alltoall_and_fcollect(elem_size, nelem, wgs):
         compare(n_pes, dst, heap, block, block * n_pes + 32)
 
 
+@pytest.mark.parametrize("elem_size,nelem,wgs,wg_size", [(4, 30011, 3, 128), (8, 16384, 4, 128),
+                                                         (1, 200003, 2, 256)])
+def test_alltoall_and_fcollect_large_blocks_shared_by_several_workgroups(elem_size, nelem, wgs, wg_size):
+    # large blocks cut into one range per workgroup, with block sizes that leave sources and
+    # destinations misaligned against each other in some blocks and aligned in others
+    n_pes = 4
+    block = elem_size * nelem
+    with runtime(n_pes):
+        world = rs.roc_shmem_team_world()
+        src, dst, heap = setup(n_pes, block * n_pes, block * n_pes + 32, seed=nelem)
+        rs.roc_shmem_alltoall(elem_size, world, dst, src, nelem, rs.Launch(wgs, wg_size))
+        rs.synchronize()
+        oracle.alltoall(heap, block * n_pes, 0, block)
+        compare(n_pes, dst, heap, block * n_pes, block * n_pes + 32)
+        src.free()
+        dst.free()
+        src, dst, heap = setup(n_pes, block, block * n_pes + 32, seed=nelem + 1)
+        rs.roc_shmem_fcollect(elem_size, world, dst, src, nelem, rs.Launch(wgs, wg_size))
+        rs.synchronize()
+        oracle.fcollect(heap, block, 0, block)
+        compare(n_pes, dst, heap, block, block * n_pes + 32)
+
+
 def test_alltoall_reference_pattern_on_a_sub_team():
     # clients/functional_tests/tester.cpp:310-334: value (src_pe << 16) + dst_pe, int64
     n_pes, nelem = 8, 100
