@@ -189,6 +189,18 @@ def bench_putmem(rs, steps, n_pes, msg_bytes_list):
         moved = 2.0 * n_pes * tile * n_msgs
         res[str(m)] = {"GBps": moved / ms / 1e6, "ms": ms, "calls_per_pe": n_msgs, "bytes_per_call": tile,
                        "Mmsgs_per_s": n_pes * n_msgs / ms / 1e3}
+    # one 64 MiB message per PE moved by all of the PE's workgroups together (sharded extension)
+    msg = 64 << 20
+    launch = rs.Launch(**PUT_LAUNCH)
+
+    def shared():
+        rs.roc_shmem_rma(rs.PUT, rs.WG_SHARED, dst, src, msg, total // msg, msg, msg, 1, launch)
+
+    shared()
+    rs.synchronize()
+    ms = event_time_ms(rs, shared, steps) / steps
+    res["67108864_shared"] = {"GBps": 2.0 * n_pes * total / ms / 1e6, "ms": ms, "calls_per_pe": total // msg,
+                              "bytes_per_call": msg, "note": "roc_shmemx_ctx_putmem_wg_shard"}
     src.free()
     dst.free()
     return res

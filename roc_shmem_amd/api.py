@@ -26,7 +26,7 @@ __all__ = [
     "sym_array", "Event", "device_array", "heap_base",
     "SHORT", "INT", "LONG", "LONGLONG", "FLOAT", "DOUBLE", "BF16",
     "SUM", "MAX", "MIN", "PROD", "AND", "OR", "XOR",
-    "PUT", "GET", "PUT_NBI", "GET_NBI", "THREAD", "WAVE", "WG",
+    "PUT", "GET", "PUT_NBI", "GET_NBI", "THREAD", "WAVE", "WG", "WG_SHARED",
     "SMALL_OP_DTYPE", "OP_P64", "OP_FADD64", "OP_ADD64", "OP_FINC64", "OP_INC64", "OP_CSWAP64",
     "OP_FETCH64", "OP_SET64", "OP_SWAP64", "OP_P32", "OP_FADD32", "OP_PUTMEM", "OP_GETMEM",
     "OP_FAND64", "OP_FOR64", "OP_FXOR64", "OP_NONE",
@@ -36,7 +36,7 @@ __all__ = [
 SHORT, INT, LONG, LONGLONG, FLOAT, DOUBLE, BF16 = range(7)
 SUM, MAX, MIN, PROD, AND, OR, XOR = range(7)
 PUT, GET, PUT_NBI, GET_NBI = range(4)
-THREAD, WAVE, WG = range(3)
+THREAD, WAVE, WG, WG_SHARED = range(4)
 (OP_P64, OP_FADD64, OP_ADD64, OP_FINC64, OP_INC64, OP_CSWAP64, OP_FETCH64, OP_SET64, OP_SWAP64,
  OP_P32, OP_FADD32, OP_PUTMEM, OP_GETMEM, OP_FAND64, OP_FOR64, OP_FXOR64) = range(16)
 OP_NONE = 255

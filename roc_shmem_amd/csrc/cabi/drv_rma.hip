@@ -34,6 +34,18 @@ __global__ void __launch_bounds__(1024)
         default: roc_shmemx_ctx_getmem_nbi_wg(ctx, d, s, msg_bytes, target); break;
       }
     }
+  } else if (granularity == RSM_WG_SHARED) {
+    for (size_t m = 0; m < n_msgs; ++m) {
+      char *d = dest + m * dst_stride;
+      const char *s = source + m * src_stride;
+      if (kind == RSM_PUT || kind == RSM_PUT_NBI) {
+        roc_shmemx_ctx_putmem_wg_shard(ctx, d, s, msg_bytes, target, static_cast<int>(w),
+                                       static_cast<int>(nw));
+      } else {
+        roc_shmemx_ctx_getmem_wg_shard(ctx, d, s, msg_bytes, target, static_cast<int>(w),
+                                       static_cast<int>(nw));
+      }
+    }
   } else if (granularity == RSM_WAVE) {
     const size_t waves_per_wg = blockDim.x / 64;
     const size_t wave = w * waves_per_wg + threadIdx.x / 64;
@@ -62,7 +74,7 @@ __global__ void __launch_bounds__(1024)
       }
     }
   }
-  roc_shmem_ctx_quiet(ctx);
+  if (threadIdx.x == 0) roc_shmem_ctx_quiet(ctx);
   roc_shmem_wg_ctx_destroy(ctx);
   roc_shmem_wg_finalize();
 }
@@ -75,7 +87,8 @@ extern "C" int rsm_rma(int kind, int granularity, void *dest, const void *source
   rsm::Launch l;
   if (!rsm::resolve_launch(launch, &l)) return -1;
   if (kind < RSM_PUT || kind > RSM_GET_NBI) return rsm::fail("rma: unknown kind");
-  if (granularity < RSM_THREAD || granularity > RSM_WG) return rsm::fail("rma: unknown granularity");
+  if (granularity < RSM_THREAD || granularity > RSM_WG_SHARED)
+    return rsm::fail("rma: unknown granularity");
   if (!dest || !source) return rsm::fail("rma: NULL buffer");
   host::Runtime *rt = host::Runtime::get();
   // The remote side of the transfer must be symmetric.

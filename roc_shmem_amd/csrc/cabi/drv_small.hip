@@ -94,7 +94,7 @@ __global__ void __launch_bounds__(1024)
     }
     if (fetches && fetched) fetched[i] = got;
   }
-  roc_shmem_ctx_quiet(ctx);
+  if (threadIdx.x == 0) roc_shmem_ctx_quiet(ctx);
   roc_shmem_wg_ctx_destroy(ctx);
   roc_shmem_wg_finalize();
 }

@@ -253,6 +253,26 @@ __device__ inline void roc_shmemx_ctx_getmem_wg(roc_shmem_ctx_t ctx, void *dest,
   roc_shmemx_ctx_getmem_nbi_wg(ctx, dest, source, nelems, pe);
   if (nelems != 0) __syncthreads();
 }
+// extension: one transfer shared by `nshards` workgroups of the calling PE.
+// All of them pass the same dest / source / nelems / pe and their own shard
+// number; a large transfer between mutually aligned buffers is dealt to them
+// pass by pass.  Non-blocking in the sense of the _nbi forms: the source may
+// be reused and the destination read when all shards have returned and
+// roc_shmem_ctx_quiet (or the kernel's end) has passed.
+__device__ inline void roc_shmemx_ctx_putmem_wg_shard(roc_shmem_ctx_t ctx, void *dest,
+                                                      const void *source, size_t nelems, int pe,
+                                                      int shard, int nshards) {
+  if (nelems == 0) return;
+  const detail::DeviceCtx *c = detail::ctx_of(ctx);
+  detail::wg_copy_shard(detail::translate(dest, c->my_pe, pe), source, nelems, shard, nshards);
+}
+__device__ inline void roc_shmemx_ctx_getmem_wg_shard(roc_shmem_ctx_t ctx, void *dest,
+                                                      const void *source, size_t nelems, int pe,
+                                                      int shard, int nshards) {
+  if (nelems == 0) return;
+  const detail::DeviceCtx *c = detail::ctx_of(ctx);
+  detail::wg_copy_shard(dest, detail::translate(source, c->my_pe, pe), nelems, shard, nshards);
+}
 __device__ inline void roc_shmemx_ctx_putmem_nbi_wave(roc_shmem_ctx_t ctx, void *dest,
                                                       const void *source, size_t nelems,
                                                       int pe) {

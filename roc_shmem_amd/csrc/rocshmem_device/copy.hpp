@@ -148,11 +148,14 @@ constexpr int kRawBufferFlags = 0x00020000;  // untyped 32-bit data, no swizzle
 // `valid` load zeros and store nothing).
 template <int kAux, int U>
 __device__ __forceinline__ void stream_copy_uniform(char *d, const char *s, size_t nbytes,
-                                                    uint32_t tid, uint32_t nthr) {
+                                                    uint32_t tid, uint32_t nthr,
+                                                    size_t first_pass = 0, size_t pass_step = 1) {
   const uint32_t lane_off = tid * 16u;
   const uint32_t access_bytes = nthr * 16u;
   const uint32_t pass_bytes = access_bytes * U;
-  for (size_t b = 0; b < nbytes; b += pass_bytes) {
+  // This group takes passes first_pass, first_pass + pass_step, ...
+  const size_t step_bytes = pass_step * pass_bytes;
+  for (size_t b = first_pass * pass_bytes; b < nbytes; b += step_bytes) {
     const size_t left = nbytes - b;
     const int valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
     __amdgpu_buffer_rsrc_t rs =
@@ -211,9 +214,54 @@ __device__ __forceinline__ void group_copy_uniform(void *dst, const void *src, s
   for (size_t i = body + tid; i < n; i += nthr) d[i] = s[i];
 }
 
+// memcpy(dst, src, n) shared by `parts` groups that all pass the same
+// arguments and their own `part`: a large copy between mutually aligned
+// buffers is dealt pass by pass (the groups running at one moment then sweep
+// one compact window of both buffers), anything else is cut into contiguous
+// ranges.  Complete when every part has returned.
+__device__ __forceinline__ void group_copy_dealt(void *dst, const void *src, size_t n,
+                                                 uint32_t tid, uint32_t nthr, size_t part,
+                                                 size_t parts) {
+  if (parts <= 1) {
+    group_copy_uniform(dst, src, n, tid, nthr);
+    return;
+  }
+  char *d = static_cast<char *>(dst);
+  const char *s = static_cast<const char *>(src);
+  const size_t pass_bytes = static_cast<size_t>(nthr) * 16u * kStreamUnroll;
+  const bool coaligned =
+      ((reinterpret_cast<uintptr_t>(d) ^ reinterpret_cast<uintptr_t>(s)) & 15u) == 0;
+  if (coaligned && n >= 2 * parts * pass_bytes) {
+    const size_t head = (16u - (reinterpret_cast<uintptr_t>(d) & 15u)) & 15u;
+    const size_t body = (n - head) & ~static_cast<size_t>(15);
+    if (part == 0) {
+      for (size_t i = tid; i < head; i += nthr) d[i] = s[i];
+      for (size_t i = head + body + tid; i < n; i += nthr) d[i] = s[i];
+    }
+    stream_copy_uniform<2 /* nt */, kStreamUnroll>(d + head, s + head, body, tid, nthr, part, parts);
+  } else {
+    size_t share = (n + parts - 1) / parts;
+    share = (share + 255) / 256 * 256;
+    size_t b = share * part, e = b + share;
+    if (b > n) b = n;
+    if (e > n) e = n;
+    if (e > b) group_copy_uniform(d + b, s + b, e - b, tid, nthr);
+  }
+}
+
 __device__ __forceinline__ void wg_copy(void *dst, const void *src, size_t n) {
   // Workgroup-collective: the arguments are the same in every lane.
   group_copy_uniform(uniform(dst), uniform(src), uniform(n), flat_thread_id(), flat_block_size());
+}
+
+// One copy shared by `nshards` workgroups (workgroup-collective in each).
+__device__ __forceinline__ void wg_copy_shard(void *dst, const void *src, size_t n, int shard,
+                                              int nshards) {
+  shard = uniform(shard);
+  nshards = uniform(nshards);
+  if (nshards <= 0 || shard < 0 || shard >= nshards) return;
+  group_copy_dealt(uniform(dst), uniform(src), uniform(n), flat_thread_id(), flat_block_size(),
+                   static_cast<size_t>(shard), static_cast<size_t>(nshards));
 }
 
 __device__ __forceinline__ void wave_copy(void *dst, const void *src, size_t n) {

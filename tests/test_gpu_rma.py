@@ -75,6 +75,20 @@ def test_misaligned_buffers(src_mis, dst_mis, msg_bytes):
                     dst_mis=dst_mis, stride_pad=29)
 
 
+@pytest.mark.parametrize("kind", [rs.PUT, rs.GET])
+@pytest.mark.parametrize("msg_bytes,src_mis,dst_mis,wgs,wg_size", [
+    ((2 << 20) + 13, 0, 0, 4, 256),      # dealt pass by pass, tail bytes
+    ((2 << 20) + 13, 4, 4, 3, 128),      # mutually aligned, 4 bytes past a 16-byte boundary: head bytes too
+    ((1 << 20) + 5, 1, 7, 4, 256),       # misaligned against each other: one range per workgroup
+    (1000, 3, 3, 4, 256),                # too small to deal
+    (0, 0, 0, 2, 64)])
+def test_one_transfer_shared_by_the_workgroups_of_a_pe(kind, msg_bytes, src_mis, dst_mis, wgs, wg_size):
+    # roc_shmemx_ctx_{put,get}mem_wg_shard (extension)
+    with runtime(4):
+        run_rma(kind, rs.WG_SHARED, 4, msg_bytes, 2, seed=msg_bytes + src_mis, src_mis=src_mis,
+                dst_mis=dst_mis, wgs=wgs, wg_size=wg_size, stride_pad=48 if msg_bytes else 0)
+
+
 def test_zero_length_is_a_no_op():
     with runtime(4):
         run_rma(rs.PUT, rs.WG, 4, 0, 4, seed=1)
