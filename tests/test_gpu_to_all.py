@@ -149,6 +149,37 @@ def test_tiled_over_many_workgroups_int64_c1_shape():
             assert np.array_equal(got[p], expect[p])
 
 
+@pytest.mark.parametrize("dtype,op,n,wgs,wg_size,shift,in_place", [
+    (rs.INT, rs.XOR, 70001, 3, 128, 0, False),       # odd shard count, tail elements after the vectors
+    (rs.SHORT, rs.SUM, 123457, 5, 64, 0, False),     # more passes than parts, 2-byte elements
+    (rs.LONG, rs.MAX, 33333, 4, 256, 0, True),       # in place
+    (rs.INT, rs.SUM, 50001, 4, 128, 1, False),       # unaligned arrays: the element path, cut into parts
+    (rs.LONGLONG, rs.PROD, 9, 7, 64, 0, False),      # fewer elements than workgroups
+    (rs.INT, rs.OR, 1 << 16, 6, 1024, 0, False)])    # fewer passes than parts
+def test_one_reduction_shared_by_the_workgroups_of_a_pe(dtype, op, n, wgs, wg_size, shift, in_place):
+    # roc_shmemx_ctx_<T>_<op>_wg_to_all_shard (extension): launch->tile == 0 and wgs_per_pe > 1
+    with runtime(4):
+        got, expect, _ = run_case(dtype, op, 4, n, seed=n, wgs=wgs, wg_size=wg_size, elem_shift=shift,
+                                  in_place=in_place)
+        for p in range(4):
+            assert np.array_equal(got[p], expect[p]), "PE %d" % p
+
+
+@pytest.mark.parametrize("dtype", [rs.FLOAT, rs.BF16, rs.DOUBLE])
+def test_shared_reduction_floating_point_and_active_set(dtype):
+    with runtime(8):
+        got, expect, truth = run_case(dtype, rs.SUM, 8, 99991, seed=5, wgs=3, wg_size=256, pe_start=1,
+                                      log_stride=1, pe_size=3, kind="lognormal")
+        mem = members(8, 1, 1, 3)
+        for p in range(8):
+            if p in mem:
+                check_fp(dtype, got[p], truth[0], truth[1])
+                assert np.array_equal(got[p].view(np.uint8), got[mem[0]].view(np.uint8)), \
+                    "every member holds the same bits"
+            else:
+                assert np.array_equal(got[p].view(np.uint8), expect[p].view(np.uint8)), "PE %d was written" % p
+
+
 def test_repeated_tiles_reuse_one_psync_slice():
     with runtime(4):
         got, expect, _ = run_case(rs.INT, rs.SUM, 4, 40000, seed=9, wgs=2, wg_size=128, tile=1024)
