@@ -13,8 +13,13 @@
 // Device functions are defined inline (no relocatable device code needed);
 // host functions live in librocshmem_mi355x.so.
 //
-// Extensions over the reference interface are marked "extension" below:
-// bfloat16 reductions, sharded alltoall/fcollect, roc_shmemx_* host helpers.
+// Extensions over the reference interface are marked "extension" where they are
+// defined: bfloat16 reductions (roc_shmem_ctx_bf16_{sum,max,min}_wg_to_all);
+// the _shard forms, which let several workgroups of every member PE share one
+// operation (roc_shmemx_ctx_<T>_<op>_wg_to_all_shard, ..._wg_broadcast_shard,
+// ..._wg_alltoall_shard, ..._wg_fcollect_shard, roc_shmemx_ctx_{put,get}mem_wg_shard);
+// roc_shmemx_my_addr; swap / set / bitwise atomics; and the host helpers
+// roc_shmemx_set_pe, roc_shmemx_host_ptr, roc_shmemx_take_status.
 #ifndef ROCSHMEM_MI355X_ROC_SHMEM_HPP
 #define ROCSHMEM_MI355X_ROC_SHMEM_HPP
 
