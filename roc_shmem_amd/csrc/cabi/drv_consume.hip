@@ -41,20 +41,16 @@ int rsm_sq_consume(int pe, int block, void *target_arena, rsm_consume_totals_t *
       (block != -1 && (block < 0 || block >= rt->options().num_blocks)))
     return rsm::fail("rsm_sq_consume: pe / block out of range (-1 selects all)");
   static_assert(sizeof(rsm_consume_totals_t) == sizeof(detail::ConsumeTotals), "totals layout");
-  detail::ConsumeTotals *dev = nullptr;
-  CONSUME_HIP(hipMalloc(reinterpret_cast<void **>(&dev), sizeof(*dev)));
-  hipError_t e = hipMemset(dev, 0, sizeof(*dev));
-  if (e == hipSuccess) {
-    const unsigned rings = static_cast<unsigned>(rt->num_pes()) * rt->options().num_blocks;
-    hipLaunchKernelGGL(consume_kernel, dim3(rings), dim3(64), 0, nullptr, pe, block,
-                       static_cast<char *>(target_arena), dev);
-    e = hipGetLastError();
-  }
-  if (e == hipSuccess) e = hipDeviceSynchronize();
+  static_assert(sizeof(detail::ConsumeTotals) <= 256, "totals fit the runtime's result scratch");
+  detail::ConsumeTotals *dev = static_cast<detail::ConsumeTotals *>(rt->result_scratch());
+  CONSUME_HIP(hipMemset(dev, 0, sizeof(*dev)));
+  const unsigned rings = static_cast<unsigned>(rt->num_pes()) * rt->options().num_blocks;
+  hipLaunchKernelGGL(consume_kernel, dim3(rings), dim3(64), 0, nullptr, pe, block,
+                     static_cast<char *>(target_arena), dev);
+  CONSUME_HIP(hipGetLastError());
+  CONSUME_HIP(hipDeviceSynchronize());
   rsm_consume_totals_t host = {};
-  if (e == hipSuccess) e = hipMemcpy(&host, dev, sizeof(host), hipMemcpyDeviceToHost);
-  (void)hipFree(dev);
-  if (e != hipSuccess) return rsm::fail(std::string("rsm_sq_consume: ") + hipGetErrorString(e));
+  CONSUME_HIP(hipMemcpy(&host, dev, sizeof(host), hipMemcpyDeviceToHost));
   if (totals) *totals = host;
   return 0;
 }

@@ -3,6 +3,7 @@
 // VERIFY_BACKEND do (library/src/util.hpp:89-97, roc_shmem.cpp:54-61).
 #include <cstdio>
 #include <cstdlib>
+#include <mutex>
 
 #include "roc_shmem.hpp"
 #include "rocshmem_mi355x.h"
@@ -13,6 +14,12 @@ namespace rocshmem {
 roc_shmem_team_t ROC_SHMEM_TEAM_WORLD = nullptr;
 
 namespace {
+// The host interface reports ROC_SHMEM_THREAD_MULTIPLE: calls that change
+// library state (allocator, teams, read-modify-write emulation of the AMOs,
+// the shared pSync of host collectives) are serialised here.
+std::recursive_mutex g_host_lock;
+#define HOST_LOCKED std::lock_guard<std::recursive_mutex> host_guard_(g_host_lock)
+
 host::Runtime *runtime_or_die(const char *fn) {
   host::Runtime *rt = host::Runtime::get();
   if (!rt) {
@@ -54,6 +61,7 @@ __host__ void roc_shmem_global_exit(int status) {
 }
 
 __host__ void *roc_shmem_malloc(size_t size) {
+  HOST_LOCKED;
   host::Runtime *rt = runtime_or_die("roc_shmem_malloc");
   void *p = rt->sym_malloc(size);
   roc_shmem_barrier_all();  // reference: barrier after every allocation, roc_shmem.cpp:118-126
@@ -61,6 +69,7 @@ __host__ void *roc_shmem_malloc(size_t size) {
 }
 
 __host__ void roc_shmem_free(void *ptr) {
+  HOST_LOCKED;
   host::Runtime *rt = runtime_or_die("roc_shmem_free");
   roc_shmem_barrier_all();
   rt->sym_free(ptr);
@@ -114,6 +123,7 @@ __host__ int roc_shmem_team_translate_pe(roc_shmem_team_t src_team, int src_pe,
 __host__ int roc_shmem_team_split_strided(roc_shmem_team_t parent_team, int start, int stride,
                                           int size, const roc_shmem_team_config_t *, long,
                                           roc_shmem_team_t *new_team) {
+  HOST_LOCKED;
   host::Runtime *rt = runtime_or_die("roc_shmem_team_split_strided");
   *new_team = ROC_SHMEM_TEAM_INVALID;
   detail::Team *out = nullptr;
@@ -123,6 +133,7 @@ __host__ int roc_shmem_team_split_strided(roc_shmem_team_t parent_team, int star
 }
 
 __host__ void roc_shmem_team_destroy(roc_shmem_team_t team) {
+  HOST_LOCKED;
   if (team == ROC_SHMEM_TEAM_INVALID || team == ROC_SHMEM_TEAM_WORLD) return;
   runtime_or_die("roc_shmem_team_destroy")->team_destroy(reinterpret_cast<detail::Team *>(team));
 }
@@ -241,6 +252,7 @@ void getmem(void *dest, const void *source, size_t nbytes, int pe, bool blocking
 }
 
 uint64_t amo(int kind, void *dest, uint64_t value, uint64_t cond, int pe, int width) {
+  HOST_LOCKED;
   host::Runtime *rt = runtime_or_die("roc_shmem_atomic");
   void *remote = remote_of(rt, dest, pe, "roc_shmem_atomic");
   const uint64_t mask = width == 8 ? ~0ull : 0xffffffffull;
@@ -263,21 +275,10 @@ uint64_t amo(int kind, void *dest, uint64_t value, uint64_t cond, int pe, int wi
 namespace {
 // Library-owned pSync for host-initiated active-set collectives.
 long *host_psync(host::Runtime *rt) {
-  static long *psync = nullptr;
-  static host::Runtime *owner = nullptr;
-  if (owner != rt) {
-    const size_t bytes = static_cast<size_t>(rt->options().num_blocks) * detail::kSyncSlots * sizeof(long);
-    int keep = rt->current_pe();
-    rt->set_current_pe(0);
-    psync = static_cast<long *>(rt->sym_malloc(bytes));
-    rt->set_current_pe(keep);
-    if (!psync) {
-      fprintf(stderr, "rocshmem: no room for the host collectives' pSync\n");
-      abort();
-    }
-    for (int p = 0; p < rt->num_pes(); ++p)
-      check_hip(hipMemset(rt->translate(psync, p), 0, bytes), "pSync");
-    owner = rt;
+  long *psync = rt->host_psync();
+  if (!psync) {
+    fprintf(stderr, "rocshmem: no room for the host collectives' pSync\n");
+    abort();
   }
   return psync;
 }
@@ -285,6 +286,7 @@ long *host_psync(host::Runtime *rt) {
 
 void to_all(int dtype, int op, void *dest, const void *source, int nreduce, int pe_start,
             int log_pe_stride, int pe_size) {
+  HOST_LOCKED;
   if (nreduce <= 0) return;
   host::Runtime *rt = runtime_or_die("roc_shmem_to_all");
   rsm_launch_t l = collective_launch(rt, static_cast<size_t>(nreduce) * 4);
@@ -310,6 +312,7 @@ void to_all_team(int dtype, int op, roc_shmem_team_t team, void *dest, const voi
 
 void broadcast(size_t elem_size, void *dest, const void *source, int nelem, int pe_root,
                int pe_start, int log_pe_stride, int pe_size) {
+  HOST_LOCKED;
   if (nelem <= 0) return;
   host::Runtime *rt = runtime_or_die("roc_shmem_broadcast");
   rsm_launch_t l = collective_launch(rt, static_cast<size_t>(nelem) * elem_size);

@@ -221,8 +221,9 @@ std::string Runtime::init(const Options &opt) {
   RT_HIP(hipMemcpy(ctx_table_dev_, ctx_images_.data(), sizeof(detail::DeviceCtx) * rings,
                    hipMemcpyHostToDevice));
 
-  RT_HIP(hipMalloc(reinterpret_cast<void **>(&status_dev_), 64));
-  RT_HIP(hipMemset(status_dev_, 0, 64));
+  // status word (first 64 bytes) and, 256 bytes in, a scratch area for small kernel results
+  RT_HIP(hipMalloc(reinterpret_cast<void **>(&status_dev_), 512));
+  RT_HIP(hipMemset(status_dev_, 0, 512));
 
   RT_HIP(hipMalloc(reinterpret_cast<void **>(&teams_dev_), sizeof(detail::Team) * kMaxTeams));
   RT_HIP(hipMemset(teams_dev_, 0, sizeof(detail::Team) * kMaxTeams));
@@ -276,6 +277,7 @@ void Runtime::teardown() {
   arena_ = nullptr;
   teams_.clear();
   world_ = nullptr;
+  host_psync_ = nullptr;
   detail::DeviceState cleared{};
   (void)upload_state_everywhere(cleared);
 }
@@ -395,6 +397,19 @@ void Runtime::reset_queues(hipStream_t stream) {
                        sizeof(detail::SqCounters) * static_cast<size_t>(opt_.num_pes) *
                            opt_.num_blocks,
                        stream);
+}
+
+long *Runtime::host_psync() {
+  if (!host_psync_) {
+    const size_t bytes = static_cast<size_t>(opt_.num_blocks) * detail::kSyncSlots * sizeof(long);
+    size_t off = alloc_.alloc(bytes);
+    if (off == Pow2Allocator::kNoOffset) return nullptr;
+    for (int p = 0; p < opt_.num_pes; ++p) {
+      if (hipMemset(slice_base(p) + off, 0, bytes) != hipSuccess) return nullptr;
+    }
+    host_psync_ = reinterpret_cast<long *>(slice_base(0) + off);
+  }
+  return host_psync_;
 }
 
 uint32_t Runtime::take_status() {

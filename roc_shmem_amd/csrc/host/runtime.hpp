@@ -111,6 +111,13 @@ class Runtime {
   // Reads and clears the sticky device status word.
   uint32_t take_status();
 
+  // pSync slices (num_blocks x 256 longs, zeroed, in every PE's heap) that the
+  // host-initiated active-set collectives use; allocated on first use,
+  // nullptr when the heap has no room.
+  long *host_psync();
+  // 256 bytes of device memory for small results of library kernels.
+  void *result_scratch() const { return status_dev_ ? reinterpret_cast<char *>(status_dev_) + 256 : nullptr; }
+
   static constexpr int kMaxTeams = 40;  // reference: team_tracker.hpp:125
 
  private:
@@ -140,6 +147,7 @@ class Runtime {
   std::vector<int> free_team_slots_;
   std::map<const detail::Team *, TeamRecord> teams_;
   TeamRecord *world_ = nullptr;
+  long *host_psync_ = nullptr;
   detail::DeviceState state_{};
 };
 
