@@ -191,6 +191,40 @@ def test_wrapped_log_reports_overwritten_entries_as_lost():
         mem.free()
 
 
+def test_ring_shared_by_workgroups_on_different_xcds_keeps_the_newest_entries():
+    # 32 workgroups per PE feed one ring (ROC_SHMEM_NUM_BLOCKS = 1) and wrap it many times.  Every
+    # slot must end up holding the entry of the last lap (shared rings are written through to memory
+    # so that this does not depend on the order in which the XCDs' L2s are written back): the
+    # consumer pass finds each index field equal to the slot's position in the stream.
+    n_pes, sq, wgs, wg_size = 2, 256, 32, 256
+    with runtime(n_pes, heap_size=8 << 20, num_blocks=1, sq_size=sq):
+        mem = rs.sym_array(1 << 16, np.int64, fill=0)
+        n_ops = n_pes * wgs * wg_size * 6
+        rng = np.random.default_rng(3)
+        ops = np.zeros(n_ops, rs.SMALL_OP_DTYPE)
+        ops["kind"] = rng.choice([rs.OP_P64, rs.OP_FADD64, rs.OP_P32], n_ops)
+        ops["pe"] = rng.integers(0, n_pes, n_ops)
+        ops["offset"] = mem.offset + rng.integers(0, 1 << 16, n_ops) * 8
+        ops["value"] = rng.integers(-5, 5, n_ops)
+        dev_ops = rs.device_array(ops)
+        rs.sq_reset()
+        rs.roc_shmem_small_ops(dev_ops, n_ops, None, rs.Launch(wgs, wg_size))
+        rs.synchronize()
+        per_ring = n_ops // n_pes
+        for pe in range(n_pes):
+            st = rs.sq_state(pe, 0)
+            assert st["sq_counter"] == per_ring and st["published"] == per_ring
+            image = rs.sq_image(pe, 0, sq)
+            for k in range(sq):
+                newest = per_ring - sq + ((k - (per_ring - sq)) % sq)
+                assert int.from_bytes(bytes(image[k][1:3]), "big") == newest & 0xFFFF, (pe, k)
+        totals = rs.sq_consume()
+        assert totals["rejected"] == 0 and totals["retired"] == n_pes * sq
+        assert totals["lost"] == n_pes * (per_ring - sq)
+        dev_ops.free()
+        mem.free()
+
+
 def post_one_wave_per_ring(mem, n_pes, value):
     n_ops = n_pes * 64
     ops = np.zeros(n_ops, rs.SMALL_OP_DTYPE)
