@@ -189,6 +189,17 @@ def bench_putmem(rs, steps, n_pes, msg_bytes_list):
         moved = 2.0 * n_pes * tile * n_msgs
         res[str(m)] = {"GBps": moved / ms / 1e6, "ms": ms, "calls_per_pe": n_msgs, "bytes_per_call": tile,
                        "Mmsgs_per_s": n_pes * n_msgs / ms / 1e3}
+    # getmem in the same shape as the largest put
+    launch = rs.Launch(**PUT_LAUNCH)
+
+    def get_step():
+        rs.roc_shmem_rma(rs.GET, rs.WG, dst, src, PUT_TILE, total // PUT_TILE, PUT_TILE, PUT_TILE, 1, launch)
+
+    get_step()
+    rs.synchronize()
+    ms = event_time_ms(rs, get_step, steps) / steps
+    res["getmem_67108864"] = {"GBps": 2.0 * n_pes * total / ms / 1e6, "ms": ms,
+                              "calls_per_pe": total // PUT_TILE, "bytes_per_call": PUT_TILE}
     # one 64 MiB message per PE moved by all of the PE's workgroups together (sharded extension)
     msg = 64 << 20
     launch = rs.Launch(**PUT_LAUNCH)
@@ -235,6 +246,27 @@ def bench_small_ops(rs, n_pes, n_ops, wgs_total, wg_size, slice_bytes, seed):
         ms = event_time_ms(rs, step, 3) / 3
         res[name] = {"Mops_per_s": n_ops / ms / 1e3, "ms": ms}
         dev.free()
+    # Lane-contiguous 8-byte putmems: the coalescer merges each wave's 64 messages into one 512-byte
+    # WQE (wf_coal_policy.cpp:57-172); every lane still moves its own 8 bytes.
+    half = words // 2
+    ops = np.zeros(n_ops, rs.SMALL_OP_DTYPE)
+    i = np.arange(n_ops)
+    ops["kind"] = rs.OP_PUTMEM
+    ops["pe"] = (i // 64) % n_pes
+    ops["offset"] = mem.offset + (i % half) * 8
+    ops["value"] = mem.offset + (half + i % half) * 8
+    ops["aux"] = 8
+    dev = rs.device_array(ops)
+
+    def coalesced():
+        rs.roc_shmem_small_ops(dev, n_ops, None, launch)
+
+    coalesced()
+    rs.synchronize()
+    ms = event_time_ms(rs, coalesced, 3) / 3
+    res["putmem8_lane_contiguous"] = {"Mops_per_s": n_ops / ms / 1e3, "ms": ms,
+                                      "note": "64 lanes x 8 B coalesced into one 512-byte WQE per wave"}
+    dev.free()
     # Consumer pass over what the last stream left in the rings (each ring keeps its newest
     # sq_size entries): check + complete only, host-timed around the synchronous call.
     t0 = time.perf_counter()
