@@ -1,4 +1,4 @@
-"""The five BASELINE configurations at their full sizes, through the C ABI.
+"""The five benchmark workloads at their full sizes, through the C ABI.
 
 Small-size parity is covered elsewhere; here the same paths run at the sizes the
 throughput figures are quoted on and are compared with the oracle on the full data (or,

@@ -59,7 +59,7 @@ def test_kinds_and_granularities(kind, gran):
 
 @pytest.mark.parametrize("msg_bytes", [8, 16, 32, 63, 64, 65, 100, 256, 1024, 4096, 65536, 1 << 20])
 def test_message_size_sweep_wg(msg_bytes):
-    # second BASELINE configuration at reduced heap size: 8 slices, powers of two from 8 B up
+    # the put/get benchmark sweep at reduced heap size: 8 slices, powers of two from 8 B up
     with runtime(8):
         run_rma(rs.PUT, rs.WG, 8, msg_bytes, 3, seed=msg_bytes)
         run_rma(rs.GET, rs.WG, 8, msg_bytes, 3, seed=msg_bytes + 1)

@@ -146,7 +146,7 @@ def check_rings(shifted_ops, issue, n_pes, num_blocks, sq_size, masked_ce=True):
 
 
 def test_unique_puts_and_fetch_adds_heap_fetched_and_rings():
-    # fourth BASELINE configuration at reduced size: puts to unique offsets in the lower half of
+    # the small-operation benchmark workload at reduced size: puts to unique offsets in the lower half of
     # every slice, fetch-adds (collisions allowed) to the upper half.
     n_pes, wgs, wg_size, num_blocks, sq = 4, 4, 256, 4, 1024
     words = 1 << 14

@@ -140,7 +140,7 @@ def test_active_sets(pe_start, log_stride, pe_size):
 
 
 def test_tiled_over_many_workgroups_int64_c1_shape():
-    # The first BASELINE configuration at reduced length: int64 sum, 4 slices,
+    # The int64 benchmark workload at reduced length: int64 sum, 4 slices,
     # values uniform in [-2^30, 2^30], dest pre-filled 0x5A.
     with runtime(4, heap_size=64 << 20):
         n = 1 << 18
