@@ -323,6 +323,8 @@ def main():
     ap.add_argument("--counter-pair", action="store_true",
                     help="for rocprofv3 --pmc: a few launches of the headline kernel and of a "
                          "plain wg putmem copy of known size (2 GiB read + 2 GiB written), nothing else")
+    ap.add_argument("--small-ops", action="store_true",
+                    help="for rocprofv3 --pmc: the 10 M-operation streams and the consumer pass, nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: every PE slice lives in one GPU's HBM; this build measures one GPU only "
@@ -332,6 +334,12 @@ def main():
     import oracle
     import roc_shmem_amd as rs
 
+    if args.small_ops:
+        rs.roc_shmem_init(16, 256 << 20, 64, 1024)
+        out = bench_small_ops(rs, 16, 10_000_000, 1024, 256, 64 << 20, seed=4)
+        rs.roc_shmem_finalize()
+        print(json.dumps({"small_ops_16x64MiB_1024wg_x256": out}))
+        return
     device = device_report() if not args.counter_pair else {}
     # ---- headline: fp32 sum_to_all, 8 slices x 2^26 elements (4 GiB algorithmic traffic) ----
     n_pes, n = 8, 1 << 26
