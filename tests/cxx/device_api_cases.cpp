@@ -252,7 +252,17 @@ __global__ void TeamCtxPrimitiveTest(char *s_buf, char *r_buf, int size, int typ
   roc_shmem_wg_team_create_ctx(team, ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
   s_buf = roc_shmemx_my_addr(s_buf);
   r_buf = roc_shmemx_my_addr(r_buf);
-  if (threadIdx.x == 0 && roc_shmem_my_pe() == 1) {   // team PE 0
+  if (type >= 4) {
+    // The AMOs and the wg/wave calls take `pe` as a world PE even on a team
+    // context (roc_shmem_gpu.cpp:556-561,667-795): 2 is not a member of {1, 3}.
+    if (roc_shmem_my_pe() == 1) {
+      if (type == 4) {
+        roc_shmemx_ctx_putmem_wg(ctx, r_buf, s_buf, size, 2);
+      } else if (threadIdx.x == 0) {
+        roc_shmem_ctx_int_atomic_add(ctx, reinterpret_cast<int *>(r_buf), 0x01010101, 2);
+      }
+    }
+  } else if (threadIdx.x == 0 && roc_shmem_my_pe() == 1) {   // team PE 0
     switch (type) {
       case 0: roc_shmem_ctx_getmem(ctx, r_buf, s_buf, size, 1); break;
       case 1: roc_shmem_ctx_getmem_nbi(ctx, r_buf, s_buf, size, 1); break;
@@ -274,21 +284,25 @@ static void team_ctx_primitive() {
   roc_shmem_team_t team = ROC_SHMEM_TEAM_INVALID;
   roc_shmem_team_split_strided(ROC_SHMEM_TEAM_WORLD, 1, 2, 2, nullptr, 0, &team);
   EXPECT(team != ROC_SHMEM_TEAM_INVALID, "split {1, 3}");
-  for (int type = 0; type < 4; ++type) {
+  for (int type = 0; type < 6; ++type) {
     for (int pe = 0; pe < npes; ++pe) {
       fill(s_buf, size, static_cast<char>('a' + pe), pe);
       fill(r_buf, size, '1', pe);
     }
     TeamCtxPrimitiveTest<<<npes, 64>>>(s_buf, r_buf, size, type, team);
     finish_kernel("TeamCtxPrimitiveTest");
-    const bool is_get = type < 2;
     for (int pe = 0; pe < npes; ++pe) {
-      // get: world PE 1 receives PE 3's source; put: world PE 3 receives PE 1's source
-      char want = '1';
-      if (is_get && pe == 1) want = 'a' + 3;
-      if (!is_get && pe == 3) want = 'a' + 1;
+      // get: world PE 1 receives PE 3's source; put: world PE 3 receives PE 1's source;
+      // wg put / atomic add with pe = 2: world PE 2 is the target
       std::vector<char> got = load(r_buf, size, pe);
-      for (int i = 0; i < size; ++i) EXPECT(got[i] == want, "type %d PE %d byte %d = %c", type, pe, i, got[i]);
+      for (int i = 0; i < size; ++i) {
+        char want = '1';
+        if (type < 2 && pe == 1) want = 'a' + 3;
+        if ((type == 2 || type == 3) && pe == 3) want = 'a' + 1;
+        if (type == 4 && pe == 2) want = 'a' + 1;
+        if (type == 5 && pe == 2 && i < 4) want = '2';   // '1' + 1 in each byte of the first int
+        EXPECT(got[i] == want, "type %d PE %d byte %d = %c", type, pe, i, got[i]);
+      }
     }
   }
   roc_shmem_team_destroy(team);
