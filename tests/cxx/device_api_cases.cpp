@@ -403,6 +403,145 @@ static void swarm() {
   }
 }
 
+// ---- amo_standard_tester.cpp:117-163, amo_extended_tester.cpp:110-150, amo_bitwise_tester.cpp:125-170:
+// thread 0 of every workgroup of PE 0 issues `iters` operations on one word of PE 1; the closed
+// forms are the testers' verifyResults (num_msgs = iters * workgroups).
+enum AmoOp { FAdd, FInc, Add, Inc, FCswap, Fetch, Set, Swap, FAnd, And, FOr, Or, FXor, Xor };
+
+#define AMO_KERNEL_COMMON(T, TNAME, EXTRA)                                                        \
+  __global__ void AMOTest_##TNAME(int iters, int type, T *r_buf, T *s_buf, T *ret_val) {         \
+    __shared__ roc_shmem_ctx_t ctx;                                                               \
+    roc_shmem_wg_init();                                                                          \
+    roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);                                      \
+    r_buf = roc_shmemx_my_addr(r_buf);                                                            \
+    s_buf = roc_shmemx_my_addr(s_buf);                                                            \
+    if (threadIdx.x == 0 && roc_shmem_ctx_my_pe(ctx) == 0) {                                      \
+      T ret = 0;                                                                                  \
+      T cond = 0;                                                                                 \
+      for (int i = 0; i < iters; i++) {                                                           \
+        switch (type) {                                                                           \
+          case Fetch: ret = roc_shmem_ctx_##TNAME##_atomic_fetch(ctx, r_buf, 1); break;           \
+          case Set: roc_shmem_ctx_##TNAME##_atomic_set(ctx, r_buf, 44, 1); break;                 \
+          case Swap: ret = roc_shmem_ctx_##TNAME##_atomic_swap(ctx, r_buf, ret + 1, 1); break;    \
+          EXTRA                                                                                   \
+          default: break;                                                                         \
+        }                                                                                         \
+      }                                                                                           \
+      roc_shmem_ctx_quiet(ctx);                                                                   \
+      ret_val[wg_index()] = ret;                                                                  \
+      roc_shmem_ctx_getmem(ctx, &s_buf[wg_index()], r_buf, sizeof(T), 1);                         \
+    }                                                                                             \
+    roc_shmem_wg_ctx_destroy(ctx);                                                                \
+    roc_shmem_wg_finalize();                                                                      \
+  }
+#define AMO_STANDARD_OPS(TNAME)                                                                   \
+  case FAdd: ret = roc_shmem_ctx_##TNAME##_atomic_fetch_add(ctx, r_buf, 2, 1); break;             \
+  case FInc: ret = roc_shmem_ctx_##TNAME##_atomic_fetch_inc(ctx, r_buf, 1); break;                \
+  case FCswap:                                                                                    \
+    ret = roc_shmem_ctx_##TNAME##_atomic_compare_swap(ctx, r_buf, cond, i, 1);                    \
+    cond = i;                                                                                     \
+    break;                                                                                        \
+  case Add: roc_shmem_ctx_##TNAME##_atomic_add(ctx, r_buf, 2, 1); break;                          \
+  case Inc: roc_shmem_ctx_##TNAME##_atomic_inc(ctx, r_buf, 1); break;
+#define AMO_BITWISE_OPS(TNAME)                                                                    \
+  case FAnd: ret = roc_shmem_ctx_##TNAME##_atomic_fetch_and(ctx, r_buf, 0xFFFF, 1); break;        \
+  case And: roc_shmem_ctx_##TNAME##_atomic_and(ctx, r_buf, 0xFFFF, 1); break;                     \
+  case FOr: ret = roc_shmem_ctx_##TNAME##_atomic_fetch_or(ctx, r_buf, 0xFFFF, 1); break;          \
+  case Or: roc_shmem_ctx_##TNAME##_atomic_or(ctx, r_buf, 0xFFFF, 1); break;                       \
+  case FXor: ret = roc_shmem_ctx_##TNAME##_atomic_fetch_xor(ctx, r_buf, 0xFFFF, 1); break;        \
+  case Xor: roc_shmem_ctx_##TNAME##_atomic_xor(ctx, r_buf, 0xFFFF, 1); break;
+
+AMO_KERNEL_COMMON(float, float, )
+AMO_KERNEL_COMMON(double, double, )
+AMO_KERNEL_COMMON(int, int, AMO_STANDARD_OPS(int))
+AMO_KERNEL_COMMON(long, long, AMO_STANDARD_OPS(long))
+AMO_KERNEL_COMMON(long long, longlong, AMO_STANDARD_OPS(longlong))
+AMO_KERNEL_COMMON(unsigned int, uint, AMO_STANDARD_OPS(uint) AMO_BITWISE_OPS(uint))
+AMO_KERNEL_COMMON(unsigned long, ulong, AMO_STANDARD_OPS(ulong) AMO_BITWISE_OPS(ulong))
+AMO_KERNEL_COMMON(unsigned long long, ulonglong, AMO_STANDARD_OPS(ulonglong) AMO_BITWISE_OPS(ulonglong))
+
+template <typename T, typename Launch>
+static void amo_case(const char *tname, Launch launch, bool standard, bool bitwise) {
+  const int max_wgs = 8, iters = 25;
+  T *r_buf = static_cast<T *>(roc_shmem_malloc(sizeof(T)));
+  T *s_buf = static_cast<T *>(roc_shmem_malloc(sizeof(T) * max_wgs));
+  T *ret_val = nullptr;
+  (void)hipMalloc(reinterpret_cast<void **>(&ret_val), sizeof(T) * max_wgs);
+  for (int type = FAdd; type <= Xor; ++type) {
+    const bool is_standard = type <= FCswap, is_bitwise = type >= FAnd;
+    if ((is_standard && !standard) || (is_bitwise && !bitwise)) continue;
+    // compare-swap chains and swaps are only determined with one issuing workgroup
+    const int wgs = (type == FCswap || type == Swap) ? 1 : max_wgs;
+    const long num_msgs = static_cast<long>(iters) * wgs;
+    for (int pe = 0; pe < npes; ++pe) {
+      fill(r_buf, 1, static_cast<T>(0), pe);
+      fill(s_buf, max_wgs, static_cast<T>(0), pe);
+    }
+    (void)hipMemset(ret_val, 0, sizeof(T) * max_wgs);
+    launch(wgs * npes, iters, type, r_buf, s_buf, ret_val);
+    finish_kernel("AMOTest");
+    double expected = 0;
+    bool fetch_op = false;
+    switch (type) {
+      case FAdd: expected = 2 * (num_msgs - 1); fetch_op = true; break;
+      case FInc: expected = num_msgs - 1; fetch_op = true; break;
+      case Add: expected = 2 * num_msgs; break;
+      case Inc: expected = num_msgs; break;
+      case FCswap: expected = (num_msgs - 2) / wgs; fetch_op = true; break;
+      case Fetch: expected = 0; fetch_op = true; break;
+      case Set: expected = 44; break;
+      case Swap: expected = num_msgs / 2; fetch_op = true; break;
+      case FAnd: case And: expected = 0; fetch_op = type == FAnd; break;
+      case FOr: case Or: expected = 0xFFFF; fetch_op = type == FOr; break;
+      case FXor: expected = 0xFFFF; fetch_op = true; break;
+      case Xor: expected = (num_msgs % 2) ? 0xFFFF : 0; break;
+    }
+    std::vector<T> got(max_wgs);
+    if (fetch_op) {
+      (void)hipMemcpy(got.data(), ret_val, sizeof(T) * max_wgs, hipMemcpyDeviceToHost);
+    } else {
+      // The testers take the largest value the workgroups read back after their own operations;
+      // that is the final value for add / inc / set / or, but not for xor, which toggles.  The
+      // word itself, read after the kernel, is what every non-fetching operation is checked on.
+      got.assign(max_wgs, load(r_buf, 1, 1)[0]);
+      if (type != Xor && type != And) {
+        std::vector<T> seen = load(s_buf, max_wgs, 0);
+        T top = seen[0];
+        for (T v : seen) top = v > top ? v : top;
+        EXPECT(top == got[0], "%s op %d: largest value read back differs from the final one", tname, type);
+      }
+    }
+    T best = got[0];
+    for (T v : got) best = v > best ? v : best;
+    EXPECT(static_cast<double>(best) == expected, "%s op %d: got %g, expected %g", tname, type,
+           static_cast<double>(best), expected);
+    for (int pe = 0; pe < npes; ++pe)
+      if (pe != 1) EXPECT(load(r_buf, 1, pe)[0] == static_cast<T>(0), "%s op %d touched PE %d", tname, type, pe);
+  }
+  (void)hipFree(ret_val);
+  roc_shmem_free(s_buf);
+  roc_shmem_free(r_buf);
+}
+
+static void amo_testers() {
+  current_case = "amo_standard / amo_extended / amo_bitwise testers";
+#define RUN_AMO(T, TNAME, STD, BIT)                                                              \
+  amo_case<T>(#TNAME,                                                                             \
+              [](int grid, int iters, int type, T *r, T *s, T *rv) {                              \
+                AMOTest_##TNAME<<<grid, 64>>>(iters, type, r, s, rv);                             \
+              },                                                                                  \
+              STD, BIT);
+  RUN_AMO(float, float, false, false)
+  RUN_AMO(double, double, false, false)
+  RUN_AMO(int, int, true, false)
+  RUN_AMO(long, long, true, false)
+  RUN_AMO(long long, longlong, true, false)
+  RUN_AMO(unsigned int, uint, true, true)
+  RUN_AMO(unsigned long, ulong, true, true)
+  RUN_AMO(unsigned long long, ulonglong, true, true)
+#undef RUN_AMO
+}
+
 // ---- the context-less forms (ROC_SHMEM_CTX_DEFAULT; roc_shmem.hpp:907-1147) ------------------------
 __global__ void DefaultCtxTest(long *data, long *counter, int n) {
   roc_shmem_wg_init();
@@ -466,7 +605,8 @@ int main() {
   } cases[] = {{"ping_pong", ping_pong},       {"compare_ops", compare_ops},
                {"shmem_ptr", shmem_ptr},       {"team_ctx_infra", team_ctx_infra},
                {"team_ctx_primitive", team_ctx_primitive}, {"sync_and_barrier", sync_and_barrier},
-               {"swarm", swarm},               {"default_ctx", default_ctx}};
+               {"swarm", swarm},               {"amo_testers", amo_testers},
+               {"default_ctx", default_ctx}};
   for (auto &c : cases) {
     const int before = failures;
     c.run();
