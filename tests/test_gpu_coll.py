@@ -179,6 +179,24 @@ def test_alltoall_reference_pattern_on_a_sub_team():
         rs.roc_shmem_team_destroy(team)
 
 
+def test_fcollect_reference_pattern():
+    # clients/functional_tests/tester.cpp:336-355 (FcollectTester<int64_t>): source = own rank,
+    # dest = -1; afterwards block i of every PE's dest holds i.
+    n_pes, nelem = 8, 333
+    with runtime(n_pes):
+        world = rs.roc_shmem_team_world()
+        src = rs.sym_array(nelem, np.int64)
+        dst = rs.sym_array(nelem * n_pes, np.int64)
+        for p in range(n_pes):
+            src.write(p, np.full(nelem, p, np.int64))
+            dst.write(p, np.full(nelem * n_pes, -1, np.int64))
+        rs.roc_shmem_fcollect(8, world, dst, src, nelem, rs.Launch(2, 256))
+        rs.synchronize()
+        exp = np.repeat(np.arange(n_pes, dtype=np.int64), nelem)
+        for p in range(n_pes):
+            assert np.array_equal(dst.read(p), exp), "PE %d" % p
+
+
 def test_barrier_all_many_rounds():
     with runtime(8, num_blocks=8):
         rs.roc_shmem_wg_barrier_all(200, rs.Launch(4, 64))
