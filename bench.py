@@ -61,6 +61,20 @@ def per_launch_ms(rs, fn, iters):
     return out
 
 
+def hbm_ceilings():
+    """What bare streaming kernels reach on this card (roc_shmem_amd/csrc/probes/hbm_ceiling.hip),
+    run as a child process before this process touches the GPU."""
+    import subprocess
+    probe = os.path.join(ROOT, "roc_shmem_amd", "hbm_ceiling")
+    if not os.path.exists(probe):
+        return {"unavailable": "roc_shmem_amd/hbm_ceiling is not built"}
+    try:
+        out = subprocess.run([probe], capture_output=True, text=True, timeout=120)
+        return json.loads(out.stdout.strip().splitlines()[-1])
+    except Exception as e:
+        return {"unavailable": str(e)}
+
+
 def device_report():
     """Clock and power state of the GPU as rocm-smi prints it (run as a child process)."""
     import subprocess
@@ -341,6 +355,7 @@ def main():
         print(json.dumps({"small_ops_16x64MiB_1024wg_x256": out}))
         return
     device = device_report() if not args.counter_pair else {}
+    ceilings = hbm_ceilings() if not (args.counter_pair or args.quick) else {}
     # ---- headline: fp32 sum_to_all, 8 slices x 2^26 elements (4 GiB algorithmic traffic) ----
     n_pes, n = 8, 1 << 26
     rs.roc_shmem_init(n_pes, 1 << 30, 64, 1024)
@@ -406,6 +421,7 @@ def main():
         "per_launch_ms": {"median": round(head["ms_median"], 4), "min": round(head["ms_min"], 4),
                           "max": round(head["ms_max"], 4)},
         "device": device,
+        "hbm_ceilings_of_bare_kernels": ceilings,
         "extra": extra,
     }
     print(json.dumps(line))
