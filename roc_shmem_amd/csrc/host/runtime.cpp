@@ -101,6 +101,7 @@ Options Options::from_env() {
     if (d > 0) o.wait_limit_s = d;
   }
   if (const char *s = getenv("ROC_SHMEM_SQ_MODE")) o.sq_queue_mode = strcmp(s, "queue") == 0;
+  if (env_u64("ROC_SHMEM_HEAP_HOST_VISIBLE", &v)) o.heap_host_visible = v != 0;
   return o;
 }
 
@@ -157,7 +158,12 @@ std::string Runtime::init(const Options &opt) {
   const int P = opt_.num_pes;
   const int B = opt_.num_blocks;
   stride_ = opt_.heap_size + opt_.slice_pad;
-  RT_HIP(hipMalloc(reinterpret_cast<void **>(&arena_), stride_ * P));
+  if (opt_.heap_host_visible) {
+    RT_HIP(hipExtMallocWithFlags(reinterpret_cast<void **>(&arena_), stride_ * P,
+                                 hipDeviceMallocFinegrained));
+  } else {
+    RT_HIP(hipMalloc(reinterpret_cast<void **>(&arena_), stride_ * P));
+  }
   alloc_ = Pow2Allocator(opt_.heap_size);
 
   // Slice base table (reference: RemoteHeapInfo's base_heap[], remote_heap_info.hpp:142-152).

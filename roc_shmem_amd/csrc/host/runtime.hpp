@@ -52,6 +52,10 @@ struct Options {
   size_t slice_pad = 0;            // ROC_SHMEM_SLICE_PAD, extra bytes between slices
   double wait_limit_s = 2.0;       // ROC_SHMEM_WAIT_LIMIT_S, bound of a device flag wait
   bool sq_queue_mode = false;      // ROC_SHMEM_SQ_MODE=queue: slots are freed by the consumer pass
+  // ROC_SHMEM_HEAP_HOST_VISIBLE (default 1): the arena is fine-grained device memory, which host
+  // code can dereference like the reference's heap (hipExtMallocWithFlags, heap_type.hpp:50) and
+  // which kernels stream as fast as ordinary device memory; 0: plain hipMalloc.
+  bool heap_host_visible = true;
   static Options from_env();
 };
 

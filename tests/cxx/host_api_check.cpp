@@ -167,6 +167,20 @@ int main() {
   EXPECT(roc_shmem_uint_atomic_fetch_add(ucounter, 3u, 1) == 0xfffffffeu, "uint fetch_add");
   EXPECT(roc_shmem_uint_g(ucounter, 1) == 1u, "uint wrap");
 
+  // The heap is host-visible, as the reference's is: host code may read and write symmetric
+  // objects through plain pointers (roc_shmemx_host_ptr gives PE pe's address), with
+  // roc_shmem_barrier_all between host and device accesses.
+  for (int pe = 0; pe < np; ++pe) {
+    long *mine = static_cast<long *>(roc_shmemx_host_ptr(src, pe));
+    for (int i = 0; i < n; ++i) mine[i] = 7L * pe + i;
+  }
+  roc_shmem_barrier_all();
+  roc_shmem_ctx_long_max_to_all(ctx, dst, src, n, 0, 0, np, nullptr, nullptr);
+  for (int pe = 0; pe < np; ++pe) {
+    const long *mine = static_cast<const long *>(roc_shmemx_host_ptr(dst, pe));
+    for (int i = 0; i < n; ++i) EXPECT(mine[i] == 7L * (np - 1) + i, "host-visible dst pe %d i %d: %ld", pe, i, mine[i]);
+  }
+
   // A kernel written against the public header: ring put + device AMO.
   roc_shmem_long_p(counter, 0, 0);
   ring_put<<<np, 256>>>(dst, src, counter, n);
@@ -176,7 +190,7 @@ int main() {
   for (int pe = 0; pe < np; ++pe) {
     roc_shmem_long_get(back.data(), dst, n, pe);
     const int from = (pe + np - 1) % np;
-    for (int i = 0; i < n; ++i) EXPECT(back[i] == 1000L * from + i, "ring pe %d i %d: %ld", pe, i, back[i]);
+    for (int i = 0; i < n; ++i) EXPECT(back[i] == 7L * from + i, "ring pe %d i %d: %ld", pe, i, back[i]);
   }
   EXPECT(roc_shmem_long_g(counter, 0) == np * (np + 1) / 2, "device atomic_add: %ld", roc_shmem_long_g(counter, 0));
 

@@ -2,10 +2,10 @@
 // process that hosts every PE.  Each case keeps the reference's inputs and its
 // closed-form expectation and cites the file it follows.  Where the
 // reference's SPMD code says "every PE does X", the case loops over the PEs
-// with roc_shmemx_set_pe; where it dereferences symmetric memory on the host
-// (the reference's heap is host-visible), the case goes through
-// roc_shmem_<T>_put / _get on the calling PE, because the arena here is
-// ordinary device memory.  A collective is called once for all members.
+// with roc_shmemx_set_pe; where it dereferences symmetric memory on the host,
+// the case goes through roc_shmem_<T>_put / _get, which also works when the
+// arena is not host-visible (ROC_SHMEM_HEAP_HOST_VISIBLE=0).  A collective is
+// called once for all members.
 // Exit code 0 and a final line "SOS_CASES_OK" mean every case passed.
 #include <cstdio>
 #include <cstdlib>
