@@ -180,6 +180,22 @@ def test_shared_reduction_floating_point_and_active_set(dtype):
                 assert np.array_equal(got[p].view(np.uint8), expect[p].view(np.uint8)), "PE %d was written" % p
 
 
+def test_arena_in_plain_device_memory():
+    # ROC_SHMEM_HEAP_HOST_VISIBLE=0: hipMalloc instead of fine-grained memory; same results.
+    import os
+    os.environ["ROC_SHMEM_HEAP_HOST_VISIBLE"] = "0"
+    try:
+        with runtime(4):
+            got, expect, _ = run_case(rs.LONG, rs.SUM, 4, 100003, seed=12, wgs=4, wg_size=256, kind="c1")
+            for p in range(4):
+                assert np.array_equal(got[p], expect[p])
+            got, expect, truth = run_case(rs.FLOAT, rs.SUM, 4, 40000, seed=13, wgs=2)
+            for p in range(4):
+                check_fp(rs.FLOAT, got[p], truth[0], truth[1])
+    finally:
+        del os.environ["ROC_SHMEM_HEAP_HOST_VISIBLE"]
+
+
 def test_repeated_tiles_reuse_one_psync_slice():
     with runtime(4):
         got, expect, _ = run_case(rs.INT, rs.SUM, 4, 40000, seed=9, wgs=2, wg_size=128, tile=1024)
