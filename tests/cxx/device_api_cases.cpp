@@ -542,6 +542,113 @@ static void amo_testers() {
 #undef RUN_AMO
 }
 
+// ---- random_access_tester.cpp:32-93,103-126,178-221: every wave of PE 0's workgroup holds a few
+// "bins" of coal_coef neighbouring lanes; the lanes of a bin put (or get) `size` bytes each to
+// consecutive addresses of one randomly chosen PE, so the coalescer merges a bin into one message.
+__device__ bool thread_passing(int num_bins, const uint32_t *bin_threads, const uint32_t *off_bins,
+                               const uint32_t *pe_bins, int *offset, int *pe, int coal_coef, int size_ints) {
+  bool pass = false;
+  const int wave_id = threadIdx.x / 64;
+  const int off = wave_id * num_bins;
+  const uint32_t lane = threadIdx.x % 64;
+  for (int i = 0; i < num_bins; i++) {
+    if (lane >= bin_threads[i + off] && lane < bin_threads[i + off] + coal_coef) {
+      pass = true;
+      *offset = off_bins[i + off] + (lane - bin_threads[i + off]) * size_ints;
+      *pe = pe_bins[i + off];
+    }
+  }
+  return pass;
+}
+
+__global__ void RandomAccessTest(int loop, int *s_buf, int *r_buf, int size, int is_get, int coal_coef,
+                                 int num_bins, const uint32_t *threads_bins, const uint32_t *off_bins,
+                                 const uint32_t *pe_bins) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  s_buf = roc_shmemx_my_addr(s_buf);
+  r_buf = roc_shmemx_my_addr(r_buf);
+  int offset = 0, pe = 0;
+  if (roc_shmem_ctx_my_pe(ctx) == 0 &&
+      thread_passing(num_bins, threads_bins, off_bins, pe_bins, &offset, &pe, coal_coef,
+                     size / static_cast<int>(sizeof(int)))) {
+    for (int i = 0; i < loop; i++) {
+      if (is_get) {
+        roc_shmem_ctx_getmem(ctx, r_buf + offset, s_buf + offset, size, pe);
+      } else {
+        roc_shmem_ctx_putmem(ctx, r_buf + offset, s_buf + offset, size, pe);
+      }
+    }
+    roc_shmem_ctx_quiet(ctx);
+  }
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+static void random_access() {
+  current_case = "random_access_tester.cpp";
+  const int wg_size = 256, num_waves = wg_size / 64, space = 8;
+  uint32_t seed = 12345;
+  auto next = [&seed]() { seed = seed * 1664525u + 1013904223u; return seed >> 8; };
+  for (int size : {4, 8, 16, 64}) {
+    for (int coal_coef : {1, 4, 8}) {
+      const int thread_access = 16, num_bins = thread_access / coal_coef;   // bins per wave
+      if (num_bins < 1 || 64 / num_bins - coal_coef - 1 < 0) continue;
+      const int size_ints = size / static_cast<int>(sizeof(int));
+      const int total_ints = space * size_ints * wg_size;
+      std::vector<uint32_t> threads_bins(num_waves * num_bins), off_bins(num_waves * num_bins),
+          pe_bins(num_waves * num_bins);
+      for (int j = 0; j < num_waves; j++)
+        for (int i = 0; i < num_bins; i++) {
+          const int bin = j * num_bins + i;
+          int quad = 64 / num_bins;
+          const int range = quad - coal_coef - 1;
+          threads_bins[bin] = (range ? next() % range : 0) + i * quad;
+          quad = total_ints / (num_bins * num_waves);                 // one region of the buffer per bin
+          off_bins[bin] = next() % (quad - (size_ints * coal_coef - 1)) + bin * quad;
+          pe_bins[bin] = next() % npes;
+        }
+      uint32_t *d_threads = nullptr, *d_off = nullptr, *d_pe = nullptr;
+      const size_t bin_bytes = sizeof(uint32_t) * threads_bins.size();
+      (void)hipMalloc(reinterpret_cast<void **>(&d_threads), bin_bytes);
+      (void)hipMalloc(reinterpret_cast<void **>(&d_off), bin_bytes);
+      (void)hipMalloc(reinterpret_cast<void **>(&d_pe), bin_bytes);
+      (void)hipMemcpy(d_threads, threads_bins.data(), bin_bytes, hipMemcpyHostToDevice);
+      (void)hipMemcpy(d_off, off_bins.data(), bin_bytes, hipMemcpyHostToDevice);
+      (void)hipMemcpy(d_pe, pe_bins.data(), bin_bytes, hipMemcpyHostToDevice);
+      int *s_buf = static_cast<int *>(roc_shmem_malloc(total_ints * sizeof(int)));
+      int *r_buf = static_cast<int *>(roc_shmem_malloc(total_ints * sizeof(int)));
+      for (int is_get = 0; is_get < 2; ++is_get) {
+        for (int pe = 0; pe < npes; ++pe) {
+          fill(s_buf, total_ints, 1, pe);
+          fill(r_buf, total_ints, 0, pe);
+        }
+        RandomAccessTest<<<npes, wg_size>>>(2, s_buf, r_buf, size, is_get, coal_coef, num_bins, d_threads,
+                                            d_off, d_pe);
+        finish_kernel("RandomAccessTest");
+        for (int pe = 0; pe < npes; ++pe) {
+          std::vector<int> want(total_ints, 0);
+          for (size_t bin = 0; bin < off_bins.size(); ++bin) {
+            const bool lands_here = is_get ? pe == 0 : static_cast<int>(pe_bins[bin]) == pe;
+            if (!lands_here) continue;
+            for (int j = 0; j < size_ints * coal_coef; j++) want[off_bins[bin] + j] = 1;
+          }
+          std::vector<int> got = load(r_buf, total_ints, pe);
+          for (int i = 0; i < total_ints; ++i)
+            EXPECT(got[i] == want[i], "size %d coal %d %s PE %d int %d: got %d", size, coal_coef,
+                   is_get ? "get" : "put", pe, i, got[i]);
+        }
+      }
+      roc_shmem_free(r_buf);
+      roc_shmem_free(s_buf);
+      (void)hipFree(d_pe);
+      (void)hipFree(d_off);
+      (void)hipFree(d_threads);
+    }
+  }
+}
+
 // ---- the context-less forms (ROC_SHMEM_CTX_DEFAULT; roc_shmem.hpp:907-1147) ------------------------
 __global__ void DefaultCtxTest(long *data, long *counter, int n) {
   roc_shmem_wg_init();
@@ -606,6 +713,7 @@ int main() {
                {"shmem_ptr", shmem_ptr},       {"team_ctx_infra", team_ctx_infra},
                {"team_ctx_primitive", team_ctx_primitive}, {"sync_and_barrier", sync_and_barrier},
                {"swarm", swarm},               {"amo_testers", amo_testers},
+               {"random_access", random_access},
                {"default_ctx", default_ctx}};
   for (auto &c : cases) {
     const int before = failures;
