@@ -164,8 +164,22 @@ __host__ void debug_print_sq(int dest_pe, int src_wg, int index_wqe) {
   printf("\n");
 }
 
-__host__ void debug_print_cq(int, int, int) {
-  printf("CQ: this build has no completion queue (operations complete in program order)\n");
+__host__ void debug_print_cq(int dest_pe, int src_wg, int cqe_num) {
+  host::Runtime *rt = runtime_or_die("debug_print_cq");
+  if (dest_pe < 0 || dest_pe >= rt->num_pes() || src_wg < 0 ||
+      src_wg >= rt->options().num_blocks || cqe_num < 0 ||
+      static_cast<uint32_t>(cqe_num) >= rt->options().sq_size) {
+    fprintf(stderr, "debug_print_cq: arguments out of range\n");
+    return;
+  }
+  // Completion entries are written by the consumer pass (rsm_sq_consume).
+  uint64_t words[8];
+  const detail::DeviceCtx &c = rt->ctx_image(dest_pe, src_wg);
+  (void)hipDeviceSynchronize();
+  (void)hipMemcpy(words, c.ring.cq + 8ull * cqe_num, sizeof(words), hipMemcpyDeviceToHost);
+  printf("CQ pe %d block %d entry %d:", dest_pe, src_wg, cqe_num);
+  for (int i = 0; i < 8; ++i) printf(" %016llx", static_cast<unsigned long long>(words[i]));
+  printf("\n");
 }
 
 __host__ void roc_shmemx_set_pe(int pe) {
