@@ -11,7 +11,10 @@
  * library/src/memory/bin.hpp (a bin is a LIFO stack).
  * Pinned by: clients/unit_tests/single_heap_gtest.cpp:26-142 and
  * pow2_bins_gtest.cpp:26-157 (alloc(1) takes 128 bytes, alloc(4097) takes 8192,
- * alloc(0) yields nothing, a fresh 1 GiB heap satisfies one 1 GiB request).
+ * alloc(0) yields nothing, a fresh 1 GiB heap satisfies one 1 GiB request), and
+ * offset for offset by the reference's own Pow2Bins compiled from its sources
+ * (build_ref.sh, ref_alloc_wrapper.cpp) on fresh heaps and random alloc/free
+ * sequences (tests/test_host_allocator.py).
  */
 #include <stdlib.h>
 #include <string.h>

@@ -1,8 +1,10 @@
 """The symmetric-heap allocator of the library against the reference's unit-test
 expectations and the oracle's model of the same strategy."""
 import ctypes as C
+import os
 
 import numpy as np
+import pytest
 
 import oracle
 from roc_shmem_amd import _lib
@@ -76,4 +78,91 @@ def test_random_sequences_agree_with_the_model():
             if a != NONE:
                 live.append(a)
         assert lib.in_use() == model.in_use()
+    lib.close()
+
+
+# --- against the reference's own allocator, built from its sources where they lie ---------------
+# oracle/build_ref.sh compiles library/src/memory/pow2_bins.hpp (with binner.hpp, bin.hpp,
+# address_record.hpp) behind the C entry points of oracle/ref_alloc_wrapper.cpp into
+# oracle/_ref/libref_alloc.so.  Where that library is absent these tests are skipped and the
+# closed-form tests above are what pins the model.
+
+REF_LIB = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                       "oracle", "_ref", "libref_alloc.so")
+
+
+class RefAlloc:
+    _lib = None
+
+    def __init__(self, heap):
+        if RefAlloc._lib is None:
+            lib = C.CDLL(REF_LIB)
+            lib.ref_alloc_create.restype = C.c_void_p
+            lib.ref_alloc_create.argtypes = [C.c_size_t]
+            lib.ref_alloc_destroy.argtypes = [C.c_void_p]
+            lib.ref_alloc_alloc.restype = C.c_size_t
+            lib.ref_alloc_alloc.argtypes = [C.c_void_p, C.c_size_t]
+            lib.ref_alloc_free.argtypes = [C.c_void_p, C.c_size_t]
+            lib.ref_alloc_in_use.restype = C.c_size_t
+            lib.ref_alloc_in_use.argtypes = [C.c_void_p]
+            RefAlloc._lib = lib
+        self.h = self._lib.ref_alloc_create(heap)
+
+    def alloc(self, n):
+        return self._lib.ref_alloc_alloc(self.h, n)
+
+    def free(self, off):
+        self._lib.ref_alloc_free(self.h, off)   # the reference asserts on an unknown address
+        return 0
+
+    def in_use(self):
+        return self._lib.ref_alloc_in_use(self.h)
+
+    def close(self):
+        self._lib.ref_alloc_destroy(self.h)
+
+
+needs_ref = pytest.mark.skipif(not os.path.exists(REF_LIB),
+                               reason="oracle/_ref/libref_alloc.so not built (no reference tree)")
+
+
+@needs_ref
+@pytest.mark.parametrize("heap", [1 << 30, 1 << 20, (1 << 20) + 128 * 37, 3 << 16, 128, 1000])
+def test_fresh_heap_matches_the_reference(heap):
+    # whole-heap, half-heap and minimum requests on heaps that are and are not powers of two
+    for requests in ([heap, 1], [heap // 2, heap // 2, 128], [1, 4097, 0, 129, heap // 4],
+                     [heap // 3] * 4, [128] * 9):
+        ref, lib, model = RefAlloc(heap), HostAlloc(heap), oracle.Allocator(heap)
+        for n in requests:
+            r = ref.alloc(n)
+            assert lib.alloc(n) == r and model.alloc(n) == r, (heap, requests, n)
+            assert lib.in_use() == model.in_use() == ref.in_use()
+        ref.close()
+        lib.close()
+
+
+@needs_ref
+@pytest.mark.parametrize("seed,heap,p_free", [(1, 1 << 24, 0.45), (2, 1 << 22, 0.3), (3, (1 << 22) + 4224, 0.5),
+                                              (4, 1 << 16, 0.4)])
+def test_random_sequences_match_the_reference(seed, heap, p_free):
+    # the offsets depend on split order, stack order inside a bin and the no-merge rule, so a
+    # model that differs in any of them diverges within a few hundred steps
+    rng = np.random.default_rng(seed)
+    ref, lib, model = RefAlloc(heap), HostAlloc(heap), oracle.Allocator(heap)
+    sizes = [1, 64, 128, 129, 255, 256, 1000, 4096, 4097, 70000, 1 << 18, 1 << 20, heap // 8]
+    live = []
+    for step in range(6000):
+        if live and rng.random() < p_free:
+            off = live.pop(int(rng.integers(0, len(live))))
+            assert lib.free(off) == 0 and model.free(off) == 0
+            ref.free(off)
+        else:
+            n = int(rng.choice(sizes))
+            r = ref.alloc(n)
+            assert lib.alloc(n) == r, "library, step %d, request %d" % (step, n)
+            assert model.alloc(n) == r, "model, step %d, request %d" % (step, n)
+            if r != NONE:
+                live.append(r)
+        assert lib.in_use() == model.in_use() == ref.in_use()
+    ref.close()
     lib.close()
