@@ -58,7 +58,11 @@ __device__ __forceinline__ bool in_set(int me, int pe_start, int stride, int pe_
   return rel >= 0 && rel % stride == 0 && rel / stride < pe_size;
 }
 
-template <typename T>
+// kTeam: the team form of the call; kShard: the PE's workgroups share one broadcast (sharded
+// extension), otherwise one standard call per tile.  Four kernels rather than branches: with
+// all four calls inlined into one kernel the compiler ran out of scalar registers and the
+// store loop ran a sixth slower.
+template <typename T, bool kTeam, bool kShard>
 __global__ void __launch_bounds__(1024)
     broadcast_kernel(roc_shmem_team_t team, T *dest0, const T *source0, size_t n, size_t tile,
                      int pe_root, int pe_start, int log_stride, int pe_size, long *pSync0) {
@@ -72,10 +76,9 @@ __global__ void __launch_bounds__(1024)
   if (in_set(me, pe_start, 1 << log_stride, pe_size)) {
     T *dest = roc_shmemx_my_addr(dest0);
     const T *source = roc_shmemx_my_addr(source0);
-    long *pSync = pSync0 ? roc_shmemx_my_addr(pSync0) + w * ROC_SHMEM_BCAST_SYNC_SIZE : nullptr;
-    if (tile == 0) {
-      // one broadcast shared by the PE's workgroups (sharded extension)
-      if (team) {
+    long *pSync = kTeam ? nullptr : roc_shmemx_my_addr(pSync0) + w * ROC_SHMEM_BCAST_SYNC_SIZE;
+    if constexpr (kShard) {
+      if constexpr (kTeam) {
         bcast_team_shard_call(ctx, team, dest, source, n, pe_root, static_cast<int>(w),
                               static_cast<int>(nw));
       } else {
@@ -85,7 +88,7 @@ __global__ void __launch_bounds__(1024)
     } else {
       for (size_t off = w * tile; off < n; off += nw * tile) {
         size_t cnt = n - off < tile ? n - off : tile;
-        if (team) {
+        if constexpr (kTeam) {
           bcast_team_call(ctx, team, dest + off, source + off, static_cast<int>(cnt), pe_root);
         } else {
           bcast_call(ctx, dest + off, source + off, static_cast<int>(cnt), pe_root, pe_start,
@@ -140,11 +143,21 @@ struct BcastArgs {
   long *pSync;
 };
 
+template <typename T, bool kTeam, bool kShard>
+void launch_bcast_form(const rsm::Launch &l, const BcastArgs &a) {
+  hipLaunchKernelGGL((broadcast_kernel<T, kTeam, kShard>), dim3(l.grid), dim3(l.wg_size), 0,
+                     l.stream, a.team, static_cast<T *>(a.dest), static_cast<const T *>(a.source),
+                     a.n, a.tile, a.root, a.pe_start, a.log_stride, a.pe_size, a.pSync);
+}
+
 template <typename T>
 void launch_bcast(const rsm::Launch &l, const BcastArgs &a) {
-  hipLaunchKernelGGL(broadcast_kernel<T>, dim3(l.grid), dim3(l.wg_size), 0, l.stream, a.team,
-                     static_cast<T *>(a.dest), static_cast<const T *>(a.source), a.n, a.tile,
-                     a.root, a.pe_start, a.log_stride, a.pe_size, a.pSync);
+  const bool shard = a.tile == 0;
+  if (a.team) {
+    shard ? launch_bcast_form<T, true, true>(l, a) : launch_bcast_form<T, true, false>(l, a);
+  } else {
+    shard ? launch_bcast_form<T, false, true>(l, a) : launch_bcast_form<T, false, false>(l, a);
+  }
 }
 
 int run_bcast(size_t elem_size, const rsm::Launch &l, BcastArgs a) {

@@ -63,7 +63,10 @@ RSM_TO_ALL(__hip_bfloat16, bf16, sum, ROC_SHMEM_SUM)
 RSM_TO_ALL(__hip_bfloat16, bf16, max, ROC_SHMEM_MAX)
 RSM_TO_ALL(__hip_bfloat16, bf16, min, ROC_SHMEM_MIN)
 
-template <typename T, ROC_SHMEM_OP Op>
+// kShard: the PE's workgroups share one reduction (sharded extension); otherwise one standard
+// call per tile, tiles dealt round-robin to the PE's workgroups.  Two kernels rather than a
+// branch: with both forms inlined into one kernel the compiler ran out of scalar registers.
+template <typename T, ROC_SHMEM_OP Op, bool kShard>
 __global__ void __launch_bounds__(1024)
     to_all_kernel(T *dest0, const T *source0, size_t n, size_t tile, int pe_start, int log_stride,
                   int pe_size, T *pWrk0, long *pSync0) {
@@ -82,12 +85,10 @@ __global__ void __launch_bounds__(1024)
     const T *source = roc_shmemx_my_addr(source0);
     T *pWrk = roc_shmemx_my_addr(pWrk0);
     long *pSync = roc_shmemx_my_addr(pSync0) + w * ROC_SHMEM_REDUCE_SYNC_SIZE;
-    if (tile == 0) {
-      // one reduction shared by the PE's workgroups (sharded extension)
+    if constexpr (kShard) {
       ToAll<T, Op>::active_set_shard(ctx, dest, source, n, pe_start, log_stride, pe_size, pWrk,
                                      pSync, static_cast<int>(w), static_cast<int>(nw));
     } else {
-      // one standard call per tile, tiles dealt round-robin to the PE's workgroups
       for (size_t off = w * tile; off < n; off += nw * tile) {
         size_t cnt = n - off < tile ? n - off : tile;
         ToAll<T, Op>::active_set(ctx, dest + off, source + off, static_cast<int>(cnt), pe_start,
@@ -99,7 +100,7 @@ __global__ void __launch_bounds__(1024)
   roc_shmem_wg_finalize();
 }
 
-template <typename T, ROC_SHMEM_OP Op>
+template <typename T, ROC_SHMEM_OP Op, bool kShard>
 __global__ void __launch_bounds__(1024)
     to_all_team_kernel(roc_shmem_team_t team, T *dest0, const T *source0, size_t n, size_t tile,
                        int pe_start, int stride, int pe_size) {
@@ -115,7 +116,7 @@ __global__ void __launch_bounds__(1024)
   if (member) {
     T *dest = roc_shmemx_my_addr(dest0);
     const T *source = roc_shmemx_my_addr(source0);
-    if (tile == 0) {
+    if constexpr (kShard) {
       ToAll<T, Op>::team_shard(ctx, team, dest, source, n, static_cast<int>(w),
                                static_cast<int>(nw));
     } else {
@@ -141,16 +142,26 @@ struct ReduceArgs {
   int stride;
 };
 
-template <typename T, ROC_SHMEM_OP Op>
-void launch_one(const rsm::Launch &l, const ReduceArgs &a) {
+template <typename T, ROC_SHMEM_OP Op, bool kShard>
+void launch_form(const rsm::Launch &l, const ReduceArgs &a) {
   if (a.team) {
-    hipLaunchKernelGGL((to_all_team_kernel<T, Op>), dim3(l.grid), dim3(l.wg_size), 0, l.stream,
-                       a.team, static_cast<T *>(a.dest), static_cast<const T *>(a.source), a.n,
-                       a.tile, a.pe_start, a.stride, a.pe_size);
+    hipLaunchKernelGGL((to_all_team_kernel<T, Op, kShard>), dim3(l.grid), dim3(l.wg_size), 0,
+                       l.stream, a.team, static_cast<T *>(a.dest),
+                       static_cast<const T *>(a.source), a.n, a.tile, a.pe_start, a.stride,
+                       a.pe_size);
   } else {
-    hipLaunchKernelGGL((to_all_kernel<T, Op>), dim3(l.grid), dim3(l.wg_size), 0, l.stream,
+    hipLaunchKernelGGL((to_all_kernel<T, Op, kShard>), dim3(l.grid), dim3(l.wg_size), 0, l.stream,
                        static_cast<T *>(a.dest), static_cast<const T *>(a.source), a.n, a.tile,
                        a.pe_start, a.log_stride, a.pe_size, static_cast<T *>(a.pWrk), a.pSync);
+  }
+}
+
+template <typename T, ROC_SHMEM_OP Op>
+void launch_one(const rsm::Launch &l, const ReduceArgs &a) {
+  if (a.tile == 0) {
+    launch_form<T, Op, true>(l, a);
+  } else {
+    launch_form<T, Op, false>(l, a);
   }
 }
 

@@ -138,6 +138,19 @@ __device__ __forceinline__ void group_copy(void *dst, const void *src, size_t n,
 constexpr int kStreamUnroll = 8;          // 16-byte accesses per lane per pass
 constexpr int kRawBufferFlags = 0x00020000;  // untyped 32-bit data, no swizzle
 
+// Descriptor over [base, base + bytes) for a group whose lanes all pass the
+// same `base` and `bytes`.  Both go through readfirstlane here even though the
+// callers' values are uniform already: when the compiler has moved such a
+// value into vector registers (a 64-bit unsigned compare has no scalar form,
+// and everything computed from its result follows it to the vector unit) it
+// no longer knows the descriptor is uniform and wraps every buffer access in
+// a loop over the distinct values it might hold - a dozen extra instructions
+// per access, which cost the 1 -> 15 broadcast a sixth of its bandwidth.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t uniform_rsrc(const void *base, int bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(uniform(base)), 0, uniform(bytes),
+                                           kRawBufferFlags);
+}
+
 // Body of a group copy whose arguments are the same in every lane
 // (workgroup- and wave-collective calls): `d` 16-byte aligned, `s` 4-byte
 // aligned, `nbytes` a multiple of 16.  One pass moves U*nthr*16
@@ -158,9 +171,8 @@ __device__ __forceinline__ void stream_copy_uniform(char *d, const char *s, size
   for (size_t b = first_pass * pass_bytes; b < nbytes; b += step_bytes) {
     const size_t left = nbytes - b;
     const int valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
-    __amdgpu_buffer_rsrc_t rs =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(s) + b, 0, valid, kRawBufferFlags);
-    __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(d + b, 0, valid, kRawBufferFlags);
+    __amdgpu_buffer_rsrc_t rs = uniform_rsrc(s + b, valid);
+    __amdgpu_buffer_rsrc_t rd = uniform_rsrc(d + b, valid);
     u32x4 v[U];
 #pragma unroll
     for (int u = 0; u < U; ++u)

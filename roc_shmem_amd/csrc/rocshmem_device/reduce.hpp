@@ -187,7 +187,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
     const int valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
     Acc acc[U][E];
     {
-      __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(src0 + b, 0, valid, kRawBufferFlags);
+      __amdgpu_buffer_rsrc_t rs = uniform_rsrc(src0 + b, valid);
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         typename V::Pack p;
@@ -201,8 +201,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
       typename V::Pack p[C][U];
 #pragma unroll
       for (int c = 0; c < C; ++c) {
-        __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-            src0 + (k + c) * member_step + b, 0, valid, kRawBufferFlags);
+        __amdgpu_buffer_rsrc_t rs = uniform_rsrc(src0 + (k + c) * member_step + b, valid);
 #pragma unroll
         for (int u = 0; u < U; ++u)
           p[c][u].raw = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * access_bytes, kNt);
@@ -216,8 +215,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
             acc[u][e] = fold<Op, Acc>(acc[u][e], to_acc<T, Acc>(p[c][u].e[e]));
     }
     for (; k < as.size; ++k) {
-      __amdgpu_buffer_rsrc_t rs =
-          __builtin_amdgcn_make_buffer_rsrc(src0 + k * member_step + b, 0, valid, kRawBufferFlags);
+      __amdgpu_buffer_rsrc_t rs = uniform_rsrc(src0 + k * member_step + b, valid);
       typename V::Pack p[U];
 #pragma unroll
       for (int u = 0; u < U; ++u)
@@ -233,8 +231,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
 #pragma unroll
       for (int e = 0; e < E; ++e) out[u].e[e] = from_acc<T, Acc>(acc[u][e]);
     for (int m = 0; m < as.size; ++m) {
-      __amdgpu_buffer_rsrc_t rd =
-          __builtin_amdgcn_make_buffer_rsrc(dst0 + m * member_step + b, 0, valid, kRawBufferFlags);
+      __amdgpu_buffer_rsrc_t rd = uniform_rsrc(dst0 + m * member_step + b, valid);
 #pragma unroll
       for (int u = 0; u < U; ++u)
         __builtin_amdgcn_raw_buffer_store_b128(out[u].raw, rd, lane_off, u * access_bytes, kNt);
