@@ -28,7 +28,7 @@ HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
 # FETCH_SIZE 1 048 810.1 KiB and WRITE_SIZE 2 099 768.7 KiB per dispatch, each scaled by
 # what the same counter reads for a wg-putmem copy of known size (2 GiB read, 2 GiB
 # written: 1 048 667.0 and 2 097 754.6 KiB); see profiles/to_all_float_sum_8pe_2e26.md.
-MEASURED_TRAFFIC_BYTES = 4297322185
+MEASURED_TRAFFIC_BYTES = 4297372262
 
 # Launch shapes chosen by measurement on MI355X (256 CUs).
 TO_ALL_LAUNCH = dict(wgs_per_pe=32, wg_size=1024)

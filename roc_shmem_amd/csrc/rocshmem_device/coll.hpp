@@ -112,8 +112,8 @@ __device__ __forceinline__ void wg_copy_to_members(char *dst_mine, const char *s
 // `shard` / `nshards`: several workgroups of every member share the call.  A
 // large, mutually aligned payload is dealt to them pass by pass (the
 // workgroups running at one moment then write one compact window of every
-// destination: 1 -> 15 broadcast of 64 MiB on MI355X, 5.07 TB/s with 8
-// workgroups of 1024 lanes per PE against 4.83 TB/s with a contiguous range
+// destination: 1 -> 15 broadcast of 64 MiB on MI355X, 5.8 TB/s with 8
+// workgroups of 1024 lanes per PE against 5.6 TB/s with a contiguous range
 // per workgroup); anything else is cut into contiguous ranges.
 __device__ __forceinline__ void wg_broadcast_bytes(int my_pe, void *dest, const void *source,
                                                    size_t nbytes, int root_idx, int pe_start,
@@ -167,7 +167,7 @@ __device__ __forceinline__ void wg_broadcast_bytes(int my_pe, void *dest, const 
 // context_ib_tmpl_device.hpp:528-558).  `block_bytes` is the size of one
 // block; `nshards` workgroups of every member share the call, each moving
 // one contiguous range of every block (dealing the blocks pass by pass was
-// measured slower here: 5.2 against 5.46 TB/s for 16 x 16 blocks of 4 MiB).
+// measured slower here: 5.9 against 6.1 TB/s for 16 x 16 blocks of 4 MiB).
 __device__ __forceinline__ void wg_alltoall_bytes(int my_pe, void *dest, const void *source,
                                                   size_t block_bytes, int shard, int nshards,
                                                   int pe_start, int log_stride, int pe_size,
@@ -239,7 +239,7 @@ __device__ __forceinline__ void wg_fcollect_bytes(int my_pe, void *dest, const v
 
   // The member's own block goes to block my_idx of everybody; the member's
   // workgroups take one contiguous range of it each (dealing a 4 MiB block
-  // pass by pass was measured slower: 4.8 against 5.2 TB/s).
+  // pass by pass was measured slower: 5.4 against 5.9 TB/s).
   char *dst_mine = static_cast<char *>(dest) + static_cast<size_t>(my_idx) * block_bytes;
   const char *src = static_cast<const char *>(source);
   size_t b, e;
