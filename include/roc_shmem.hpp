@@ -174,6 +174,10 @@ void getmem(void *dest, const void *source, size_t nbytes, int pe, bool blocking
 // kind: 0 fetch_add, 1 compare_swap, 2 swap, 3 fetch_and, 4 fetch_or, 5 fetch_xor; width 4 or 8.
 // Returns the previous value of the word, zero-extended.
 uint64_t amo(int kind, void *dest, uint64_t value, uint64_t cond, int pe, int width);
+// The current PE's copy of the naturally aligned word of `width` (1, 2, 4 or 8) bytes at the
+// symmetric address `ptr`, zero-extended, as a kernel that is still running has left it.
+uint64_t fetch_own(const void *ptr, int width);
+double wait_limit_seconds();  // bound of a host-side wait (ROC_SHMEM_WAIT_LIMIT_S)
 // dtype / op use the codes of rsm_dtype / rsm_op (rocshmem_mi355x.h).
 void to_all(int dtype, int op, void *dest, const void *source, int nreduce, int pe_start,
             int log_pe_stride, int pe_size);

@@ -15,6 +15,9 @@
 #ifndef ROCSHMEM_MI355X_ROC_SHMEM_HOST_HPP
 #define ROCSHMEM_MI355X_ROC_SHMEM_HOST_HPP
 
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 namespace rocshmem {
@@ -181,6 +184,55 @@ inline T from_bits(uint64_t b) {
   return v;
 }
 }  // namespace hostx
+
+// ---- wait_until / test ------------------------------------------------------------------
+// Reference: HostInterface::wait_until / test / test_and_compare, library/src/host/
+// host_templates.hpp:426-487 (an atomic fetch of the calling PE's own copy of the word, compared
+// on the host; wait_until repeats it until the comparison holds); declared for the 13 standard
+// types at library/include/roc_shmem.hpp:1152-1163,1973-2019.  The calling PE is the host's
+// current PE.  Where the reference would spin for ever, the wait gives up after
+// ROC_SHMEM_WAIT_LIMIT_S seconds, prints a message and exits like the library's other fatal errors.
+namespace hostx {
+template <typename T>
+inline T own_value(const T *ptr) {
+  const uint64_t bits = fetch_own(ptr, static_cast<int>(sizeof(T)));
+  T v;
+  std::memcpy(&v, &bits, sizeof(T));  // little-endian host: the low bytes hold the word
+  return v;
+}
+template <typename T>
+inline bool compare(roc_shmem_cmps cmp, T have, T want) {
+  switch (cmp) {
+    case ROC_SHMEM_CMP_EQ: return have == want;
+    case ROC_SHMEM_CMP_NE: return have != want;
+    case ROC_SHMEM_CMP_GT: return have > want;
+    case ROC_SHMEM_CMP_GE: return have >= want;
+    case ROC_SHMEM_CMP_LT: return have < want;
+    default: return have <= want;
+  }
+}
+template <typename T>
+inline void wait_until(const T *ptr, roc_shmem_cmps cmp, T val) {
+  const auto start = std::chrono::steady_clock::now();
+  const double limit = wait_limit_seconds();
+  while (!compare(cmp, own_value(ptr), val)) {
+    if (std::chrono::duration<double>(std::chrono::steady_clock::now() - start).count() > limit) {
+      fprintf(stderr, "rocshmem: roc_shmem_wait_until: condition not met after %.1f s\n", limit);
+      exit(EXIT_FAILURE);
+    }
+  }
+}
+}  // namespace hostx
+
+#define ROCSHMEM_HOST_WAIT(T, TNAME)                                                           \
+  __host__ inline void roc_shmem_##TNAME##_wait_until(T *ptr, roc_shmem_cmps cmp, T val) {     \
+    hostx::wait_until<T>(ptr, cmp, val);                                                       \
+  }                                                                                            \
+  __host__ inline int roc_shmem_##TNAME##_test(T *ptr, roc_shmem_cmps cmp, T val) {            \
+    return hostx::compare<T>(cmp, hostx::own_value<T>(ptr), val) ? 1 : 0;                      \
+  }
+ROCSHMEM_HOST_STANDARD_TYPES(ROCSHMEM_HOST_WAIT)
+#undef ROCSHMEM_HOST_WAIT
 
 #define ROCSHMEM_HOST_AMO_TYPES(X) \
   X(int, int)                      \

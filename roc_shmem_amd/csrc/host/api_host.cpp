@@ -265,6 +265,33 @@ void getmem(void *dest, const void *source, size_t nbytes, int pe, bool blocking
   }
 }
 
+uint64_t fetch_own(const void *ptr, int width) {
+  host::Runtime *rt = runtime_or_die("roc_shmem_test");
+  const void *mine = remote_of(rt, ptr, rt->current_pe(), "roc_shmem_test");
+  if (reinterpret_cast<uintptr_t>(mine) & static_cast<uintptr_t>(width - 1)) {
+    fprintf(stderr, "rocshmem: roc_shmem_test: the word is not naturally aligned\n");
+    abort();
+  }
+  uint64_t bits = 0;
+  if (rt->options().heap_host_visible) {
+    // The arena is host-visible: one atomic load over the bus sees what a
+    // kernel that is still running has stored with device or system scope.
+    switch (width) {
+      case 1: bits = __atomic_load_n(static_cast<const uint8_t *>(mine), __ATOMIC_ACQUIRE); break;
+      case 2: bits = __atomic_load_n(static_cast<const uint16_t *>(mine), __ATOMIC_ACQUIRE); break;
+      case 4: bits = __atomic_load_n(static_cast<const uint32_t *>(mine), __ATOMIC_ACQUIRE); break;
+      default: bits = __atomic_load_n(static_cast<const uint64_t *>(mine), __ATOMIC_ACQUIRE); break;
+    }
+  } else {
+    // Plain device memory: a copy on the null stream, which runs after the
+    // kernels launched before it.
+    check_hip(hipMemcpy(&bits, mine, width, hipMemcpyDeviceToHost), "roc_shmem_test");
+  }
+  return bits;
+}
+
+double wait_limit_seconds() { return runtime_or_die("roc_shmem_wait_until")->options().wait_limit_s; }
+
 uint64_t amo(int kind, void *dest, uint64_t value, uint64_t cond, int pe, int width) {
   HOST_LOCKED;
   host::Runtime *rt = runtime_or_die("roc_shmem_atomic");

@@ -39,6 +39,22 @@ __global__ void ring_put(long *dst, const long *src, long *counter, int n) {
   roc_shmem_wg_finalize();
 }
 
+// PE 0 lets `ticks` of the 100 MHz device timer pass and then puts 5 into `flag` on PE 1.
+__global__ void late_signal(long *flag, uint64_t ticks) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  flag = roc_shmemx_my_addr(flag);
+  if (roc_shmem_ctx_my_pe(ctx) == 0 && threadIdx.x == 0) {
+    const uint64_t start = roc_shmem_timer();
+    for (int spins = 0; spins < (1 << 24) && roc_shmem_timer() - start < ticks; ++spins) {
+    }
+    roc_shmem_ctx_long_p(ctx, flag, 5, 1);
+  }
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
 int main() {
   setenv("ROC_SHMEM_NUM_PES", "4", 1);
   setenv("ROC_SHMEM_HEAP_SIZE", "67108864", 1);
@@ -193,6 +209,33 @@ int main() {
     for (int i = 0; i < n; ++i) EXPECT(back[i] == 7L * from + i, "ring pe %d i %d: %ld", pe, i, back[i]);
   }
   EXPECT(roc_shmem_long_g(counter, 0) == np * (np + 1) / 2, "device atomic_add: %ld", roc_shmem_long_g(counter, 0));
+
+  // Host-side wait_until / test on the current PE's copy of a word (reference:
+  // host_templates.hpp:426-487), first on values that are already there ...
+  roc_shmem_long_p(counter, 17, 2);
+  roc_shmemx_set_pe(2);
+  EXPECT(roc_shmem_long_test(counter, ROC_SHMEM_CMP_EQ, 17) == 1, "test EQ");
+  EXPECT(roc_shmem_long_test(counter, ROC_SHMEM_CMP_GT, 17) == 0, "test GT");
+  EXPECT(roc_shmem_long_test(counter, ROC_SHMEM_CMP_LT, 18) == 1, "test LT");
+  roc_shmem_long_wait_until(counter, ROC_SHMEM_CMP_GE, 17);
+  // ... then on a word that a kernel still running on another stream sets three milliseconds
+  // after its launch: the wait has to see the store while the kernel runs (host-visible heap).
+  const char *visible = getenv("ROC_SHMEM_HEAP_HOST_VISIBLE");
+  if (!visible || atoi(visible) != 0) {
+    roc_shmem_long_p(counter, 0, 1);
+    roc_shmem_barrier_all();
+    hipStream_t side;
+    EXPECT(hipStreamCreateWithFlags(&side, hipStreamNonBlocking) == hipSuccess, "stream");
+    late_signal<<<np, 64, 0, side>>>(counter, 300000);
+    roc_shmemx_set_pe(1);
+    EXPECT(roc_shmem_long_test(counter, ROC_SHMEM_CMP_EQ, 5) == 0, "the flag is set too early");
+    roc_shmem_long_wait_until(counter, ROC_SHMEM_CMP_EQ, 5);
+    EXPECT(hipStreamSynchronize(side) == hipSuccess, "late_signal");
+    EXPECT(roc_shmem_long_g(counter, 1) == 5, "flag after the kernel");
+    EXPECT(hipStreamDestroy(side) == hipSuccess, "stream destroy");
+    EXPECT(roc_shmemx_take_status() == 0, "device status");
+  }
+  roc_shmemx_set_pe(0);
 
   roc_shmem_free(counter);
   roc_shmem_free(idst);

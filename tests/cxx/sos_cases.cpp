@@ -561,6 +561,240 @@ static void broadcast_active_set() {
   }
 }
 
+// ---- point-to-point synchronisation ---------------------------------------------------------
+
+// clients/sos_tests/cxx_test_shmem_wait_until.cpp:42-60 and cxx_test_shmem_test.cpp:42-61: every PE
+// puts (TYPE)me + 1 into its right-hand neighbour and waits on its own copy for a value other
+// than zero, which must be that of its left-hand neighbour.  In one process all puts are made
+// first; each PE's wait then finds its condition already true.
+template <typename T, typename P, typename W, typename Tst>
+static void wait_case(const char *name, P p, W wait_until, Tst test) {
+  current_case = name;
+  Sym<T> remote(1);
+  for (int use_test = 0; use_test < 2; ++use_test) {
+    for (int me = 0; me < npes; ++me) remote.fill(me, 0);
+    roc_shmemx_set_pe(0);
+    EXPECT(test(remote.ptr, ROC_SHMEM_CMP_NE, static_cast<T>(0)) == 0, "test true before any put");
+    EXPECT(test(remote.ptr, ROC_SHMEM_CMP_EQ, static_cast<T>(0)) == 1, "test of the initial value");
+    for (int me = 0; me < npes; ++me) {
+      roc_shmemx_set_pe(me);
+      p(remote.ptr, static_cast<T>(static_cast<T>(me) + 1), (me + 1) % npes);
+    }
+    for (int me = 0; me < npes; ++me) {
+      roc_shmemx_set_pe(me);
+      if (use_test) {
+        int spins = 0;
+        while (!test(remote.ptr, ROC_SHMEM_CMP_NE, static_cast<T>(0)) && ++spins < 1000000) {
+        }
+        EXPECT(spins < 1000000, "test never became true on PE %d", me);
+      } else {
+        wait_until(remote.ptr, ROC_SHMEM_CMP_NE, static_cast<T>(0));
+      }
+      const T want = static_cast<T>(static_cast<T>((me + npes - 1) % npes) + 1);
+      EXPECT(remote.load(me)[0] == want, "PE %d holds the wrong value", me);
+      // the remaining comparisons, on the value that is there now
+      EXPECT(test(remote.ptr, ROC_SHMEM_CMP_EQ, want) == 1, "EQ on PE %d", me);
+      EXPECT(test(remote.ptr, ROC_SHMEM_CMP_GE, want) == 1, "GE on PE %d", me);
+      EXPECT(test(remote.ptr, ROC_SHMEM_CMP_LE, want) == 1, "LE on PE %d", me);
+      EXPECT(test(remote.ptr, ROC_SHMEM_CMP_GT, want) == 0, "GT on PE %d", me);
+      EXPECT(test(remote.ptr, ROC_SHMEM_CMP_LT, static_cast<T>(want + 1)) == 1, "LT on PE %d", me);
+    }
+  }
+}
+
+static void wait_until_and_test() {
+#define WAIT_CASE(T, TNAME)                                                                    \
+  wait_case<T>("cxx_test_shmem_wait_until.cpp / cxx_test_shmem_test.cpp " #TNAME,              \
+               [](T *d, T v, int pe) { roc_shmem_##TNAME##_p(d, v, pe); },                      \
+               [](T *ptr, roc_shmem_cmps c, T v) { roc_shmem_##TNAME##_wait_until(ptr, c, v); }, \
+               [](T *ptr, roc_shmem_cmps c, T v) { return roc_shmem_##TNAME##_test(ptr, c, v); });
+  WAIT_CASE(short, short)
+  WAIT_CASE(int, int)
+  WAIT_CASE(long, long)
+  WAIT_CASE(long long, longlong)
+  WAIT_CASE(unsigned short, ushort)
+  WAIT_CASE(unsigned int, uint)
+  WAIT_CASE(unsigned long, ulong)
+  WAIT_CASE(unsigned long long, ulonglong)
+#undef WAIT_CASE
+}
+
+// clients/sos_tests/waituntil.cpp:58-137: PE 0 clears `target` everywhere, puts 1..10 into every
+// other PE, waits for pong > 666 (PE 1 sets it to 999 once its target[9] reads 10) and then puts
+// 0xDD into t2[9] of the others, which wait for it.  The steps run here in an order in which every
+// wait finds its condition met by a put made earlier.
+static void waituntil() {
+  current_case = "waituntil.cpp";
+  long source[10] = {1, 2, 3, 4, 5, 6, 7, 8, 9, 10};
+  Sym<long> target(10), pong(1), t2(10);
+  for (int me = 0; me < npes; ++me) {
+    pong.fill(me, 666);
+    target.fill(me, 0xFF);
+    t2.fill(me, 0xFF);
+  }
+  roc_shmem_barrier_all();
+  roc_shmemx_set_pe(0);
+  long zeros[10] = {0};
+  for (int pe = 1; pe < npes; ++pe) roc_shmem_long_put(target.ptr, zeros, 10, pe);
+  for (int pe = 1; pe < npes; ++pe) roc_shmem_long_put(target.ptr, source, 10, pe);
+  for (int me = 1; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    roc_shmem_long_wait_until(&target.ptr[9], ROC_SHMEM_CMP_NE, 0xFF);
+    roc_shmem_long_wait_until(&target.ptr[9], ROC_SHMEM_CMP_EQ, 10);
+    if (me == 1) {
+      EXPECT(roc_shmem_long_g(pong.ptr, 0) == 666, "pong on PE 0 before the reply");
+      roc_shmem_long_p(pong.ptr, 999, 0);
+    }
+  }
+  roc_shmemx_set_pe(0);
+  roc_shmem_long_wait_until(pong.ptr, ROC_SHMEM_CMP_GT, 666);
+  EXPECT(pong.load(0)[0] == 999, "pong on PE 0 = %ld", pong.load(0)[0]);
+  for (int pe = 1; pe < npes; ++pe) roc_shmem_long_p(&t2.ptr[9], 0xDD, pe);
+  for (int me = 1; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    roc_shmem_long_wait_until(&t2.ptr[9], ROC_SHMEM_CMP_NE, 0xFF);
+    EXPECT(t2.load(me)[9] == 0xDD, "t2[9] on PE %d = %ld", me, t2.load(me)[9]);
+    std::vector<long> got = target.load(me);
+    for (int i = 0; i < 10; ++i) EXPECT(got[i] == i + 1, "target[%d] on PE %d = %ld", i, me, got[i]);
+  }
+  EXPECT(t2.load(0)[9] == 0xFF, "PE 0's own t2 was written");
+}
+
+// ---- small programs -------------------------------------------------------------------------
+
+// clients/sos_tests/circular_shift.cpp:38-62: every PE stores its rank and gets its right-hand
+// neighbour's; get1.cpp:44-80: PE 0 gets ten longs i + 1 from PE 1.
+static void circular_shift_and_get1() {
+  current_case = "circular_shift.cpp";
+  Sym<int> bbb(1);
+  for (int me = 0; me < npes; ++me) bbb.fill(me, me);
+  roc_shmem_barrier_all();
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    const int neighbor = (me + 1) % npes;
+    int aaa = -1;
+    roc_shmem_int_get(&aaa, bbb.ptr, 1, neighbor);
+    EXPECT(aaa == neighbor, "PE %d got %d from PE %d", me, aaa, neighbor);
+  }
+  current_case = "get1.cpp";
+  Sym<long> source(10);
+  std::vector<long> pattern(10);
+  for (int i = 0; i < 10; ++i) pattern[i] = i + 1;
+  for (int me = 0; me < npes; ++me) source.store(me, pattern);
+  roc_shmem_barrier_all();
+  roc_shmemx_set_pe(0);
+  long target[10] = {0};
+  roc_shmem_long_get(target, source.ptr, 10, 1);
+  roc_shmem_barrier_all();
+  EXPECT(memcmp(target, pattern.data(), sizeof(target)) == 0, "source and target differ");
+}
+
+// clients/sos_tests/pi.cpp:40-110: every PE counts the random points that fall inside the unit
+// circle; PE 0 gets and adds the others' counters.  The reference checks |pi - estimate| < 0.1;
+// here the gathered totals are also compared with the counts made on the host.
+static void pi() {
+  current_case = "pi.cpp";
+  const long long points = 10000;
+  Sym<long long> inside(1), total(1);
+  long long want_inside = 0;
+  for (int me = 0; me < npes; ++me) {
+    srand(1 + me);
+    long long in = 0;
+    for (long long t = 0; t < points; ++t) {
+      const double x = rand() / static_cast<double>(RAND_MAX), y = rand() / static_cast<double>(RAND_MAX);
+      if (x * x + y * y < 1) ++in;
+    }
+    inside.fill(me, in);
+    total.fill(me, points);
+    want_inside += in;
+  }
+  roc_shmem_barrier_all();
+  roc_shmemx_set_pe(0);
+  long long sum_inside = inside.load(0)[0], sum_total = total.load(0)[0];
+  for (int i = 1; i < npes; ++i) {
+    long long remote_inside = 0, remote_total = 0;
+    roc_shmem_longlong_get(&remote_inside, inside.ptr, 1, i);
+    roc_shmem_longlong_get(&remote_total, total.ptr, 1, i);
+    sum_inside += remote_inside;
+    sum_total += remote_total;
+  }
+  EXPECT(sum_total == points * npes && sum_inside == want_inside, "gathered %lld of %lld", sum_inside, sum_total);
+  const double approx = 4.0 * sum_inside / static_cast<double>(sum_total);
+  EXPECT(approx > 3.04 && approx < 3.25, "pi estimate %f", approx);
+}
+
+// clients/sos_tests/many-ctx.cpp:36-80: every PE creates NUM_CTX contexts and increments a
+// counter on its right-hand neighbour once through each; after quiet on every context and
+// sync_all each counter holds NUM_CTX.
+static void many_ctx() {
+  current_case = "many-ctx.cpp";
+  const int kNumCtx = 32;
+  Sym<int64_t> data(1);
+  for (int me = 0; me < npes; ++me) data.fill(me, 0);
+  roc_shmem_barrier_all();
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    roc_shmem_ctx_t ctx[kNumCtx];
+    for (int i = 0; i < kNumCtx; ++i) {
+      if (roc_shmem_ctx_create(0, &ctx[i]) != 0) ctx[i] = ROC_SHMEM_CTX_DEFAULT;  // as the reference does
+    }
+    for (int i = 0; i < kNumCtx; ++i) roc_shmem_ctx_int64_atomic_inc(ctx[i], data.ptr, (me + 1) % npes);
+    for (int i = 0; i < kNumCtx; ++i) roc_shmem_ctx_quiet(ctx[i]);
+    for (int i = 0; i < kNumCtx; ++i)
+      if (ctx[i].ctx_opaque != ROC_SHMEM_CTX_DEFAULT.ctx_opaque) roc_shmem_ctx_destroy(ctx[i]);
+  }
+  roc_shmem_sync_all();
+  for (int me = 0; me < npes; ++me)
+    EXPECT(data.load(me)[0] == kNumCtx, "PE %d counted %ld", me, static_cast<long>(data.load(me)[0]));
+}
+
+// ---- teams ------------------------------------------------------------------------------------
+
+// clients/sos_tests/shmem_team_b2b_collectives.cpp:68-100: NITERS back-to-back broadcasts and then
+// reductions on the world team with src = me, no barrier in between; the last results must be
+// those of a single call.
+static void team_b2b_collectives() {
+  current_case = "shmem_team_b2b_collectives.cpp";
+  const int kIters = 100, kElems = 10;
+  Sym<long> dest(kElems), src(kElems);
+  for (int me = 0; me < npes; ++me) {
+    src.fill(me, me);
+    dest.fill(me, -7);
+  }
+  for (int i = 0; i < kIters; ++i)
+    roc_shmem_ctx_long_broadcast(ROC_SHMEM_CTX_DEFAULT, ROC_SHMEM_TEAM_WORLD, dest.ptr, src.ptr, kElems, 0);
+  for (int me = 0; me < npes; ++me)
+    for (long x : dest.load(me)) EXPECT(x == (me == 0 ? -7 : 0), "broadcast: PE %d holds %ld", me, x);
+  for (int i = 0; i < kIters; ++i)
+    roc_shmem_ctx_long_sum_to_all(ROC_SHMEM_CTX_DEFAULT, ROC_SHMEM_TEAM_WORLD, dest.ptr, src.ptr, kElems);
+  const long want = static_cast<long>(npes) * (npes - 1) / 2;
+  for (int me = 0; me < npes; ++me)
+    for (long x : dest.load(me)) EXPECT(x == want, "reduce: PE %d holds %ld", me, x);
+}
+
+// clients/sos_tests/shmem_team_reuse_teams.cpp:35-75: npes - 1 rounds in which the team loses its
+// first member (split (1, 1, n - 1) of the previous team) and the previous team is destroyed.
+static void team_reuse_teams() {
+  current_case = "shmem_team_reuse_teams.cpp";
+  roc_shmem_team_t old_team, new_team;
+  int ret = roc_shmem_team_split_strided(ROC_SHMEM_TEAM_WORLD, 0, 1, npes, nullptr, 0, &old_team);
+  EXPECT(ret == 0, "first split returned %d", ret);
+  for (int i = 1; i < npes; ++i) {
+    EXPECT(roc_shmem_team_translate_pe(old_team, 1, ROC_SHMEM_TEAM_WORLD) == i,
+           "round %d: second member is world PE %d", i,
+           roc_shmem_team_translate_pe(old_team, 1, ROC_SHMEM_TEAM_WORLD));
+    const int size = roc_shmem_team_n_pes(old_team);
+    EXPECT(size == npes - i + 1, "round %d: team of %d", i, size);
+    ret = roc_shmem_team_split_strided(old_team, 1, 1, size - 1, nullptr, 0, &new_team);
+    EXPECT(ret == 0 && new_team != ROC_SHMEM_TEAM_INVALID, "round %d: split returned %d", i, ret);
+    roc_shmem_team_destroy(old_team);
+    old_team = new_team;
+  }
+  EXPECT(roc_shmem_team_n_pes(old_team) == 1, "last team has %d members", roc_shmem_team_n_pes(old_team));
+  EXPECT(roc_shmem_team_translate_pe(old_team, 0, ROC_SHMEM_TEAM_WORLD) == npes - 1, "last team's member");
+  roc_shmem_team_destroy(old_team);
+}
+
 int main() {
   if (!getenv("ROC_SHMEM_NUM_PES")) setenv("ROC_SHMEM_NUM_PES", "6", 1);
   setenv("ROC_SHMEM_HEAP_SIZE", "134217728", 0);
@@ -583,7 +817,14 @@ int main() {
                {"mt_a2a", mt_a2a},
                {"bcast", bcast},
                {"bcast_flood", bcast_flood},
-               {"broadcast_active_set", broadcast_active_set}};
+               {"broadcast_active_set", broadcast_active_set},
+               {"wait_until_and_test", wait_until_and_test},
+               {"waituntil", waituntil},
+               {"circular_shift_get1", circular_shift_and_get1},
+               {"pi", pi},
+               {"many_ctx", many_ctx},
+               {"team_b2b_collectives", team_b2b_collectives},
+               {"team_reuse_teams", team_reuse_teams}};
   for (auto &c : cases) {
     const int before = failures;
     c.run();
