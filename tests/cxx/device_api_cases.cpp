@@ -701,6 +701,145 @@ static void default_ctx() {
   roc_shmem_free(data);
 }
 
+// ---- primitive_mr_tester.cpp:32-58,102-118: thread 0 of every workgroup of PE 0 issues 64 * loop
+// windows of 64 putmem_nbi of `size` bytes to PE 1, with a quiet after every window; afterwards
+// r_buf on PE 1 holds the source's '0' characters.  8192 posts per workgroup and launch, so the
+// 1024-entry send queue wraps several times.
+__global__ void PrimitiveMRTest(int loop, uint64_t *timer, char *s_buf, char *r_buf, int size) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  s_buf = roc_shmemx_my_addr(s_buf);
+  r_buf = roc_shmemx_my_addr(r_buf);
+  if (threadIdx.x == 0 && roc_shmem_ctx_my_pe(ctx) == 0) {
+    uint64_t start = roc_shmem_timer();
+    for (int win_i = 0; win_i < 64 * loop; win_i++) {
+      for (int i = 0; i < 64; i++) roc_shmem_ctx_putmem_nbi(ctx, r_buf, s_buf, size, 1);
+      roc_shmem_ctx_quiet(ctx);
+    }
+    timer[wg_index()] = roc_shmem_timer() - start;
+  }
+  __syncthreads();
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+static void primitive_mr() {
+  current_case = "primitive_mr_tester.cpp";
+  const int wgs = 4, max_size = 1024;
+  uint64_t *timer;
+  EXPECT(hipMalloc(&timer, wgs * sizeof(uint64_t)) == hipSuccess, "hipMalloc");
+  char *s_buf = static_cast<char *>(roc_shmem_malloc(max_size));
+  char *r_buf = static_cast<char *>(roc_shmem_malloc(max_size));
+  for (int size : {1, 8, 9, 64, 1000}) {
+    for (int pe = 0; pe < npes; ++pe) {
+      fill(s_buf, max_size, '0', pe);
+      fill(r_buf, max_size, '1', pe);
+    }
+    for (int launch = 0; launch < 2; ++launch)  // warm-up and benchmark launch, as the tester does
+      PrimitiveMRTest<<<wgs * npes, 64>>>(2, timer, s_buf, r_buf, size);
+    finish_kernel("PrimitiveMRTest");
+    std::vector<char> got = load(r_buf, max_size, 1);
+    for (int i = 0; i < max_size; ++i)
+      EXPECT(got[i] == (i < size ? '0' : '1'), "size %d: r_buf[%d] on PE 1 = %c", size, i, got[i]);
+    for (int pe = 0; pe < npes; ++pe)
+      if (pe != 1)
+        for (char c : load(r_buf, max_size, pe)) EXPECT(c == '1', "size %d: PE %d was written", size, pe);
+  }
+  uint64_t ticks[wgs];
+  EXPECT(hipMemcpy(ticks, timer, sizeof(ticks), hipMemcpyDeviceToHost) == hipSuccess, "timer copy");
+  printf("  putmem_nbi(1000 B) + quiet per 64: %.0f ns per message in one lane\n",
+         ticks[0] * 10.0 / (64 * 2 * 64));
+  roc_shmem_free(r_buf);
+  roc_shmem_free(s_buf);
+  EXPECT(hipFree(timer) == hipSuccess, "hipFree");
+}
+
+// ---- primitive_amo_tester.cpp:30-100,160-215: thread 0 of every workgroup of PE 0 issues
+// loop + skip int64 operations on one word of PE 1, then quiet, and reads the word back with
+// getmem; verifyResults' closed forms with num_msgs = (loop + skip) * workgroups.
+enum PrimAmo { PFAdd, PFInc, PFetch, PFCswap, PAdd, PInc };
+__global__ void PrimitiveAMOTest(int loop, int skip, char *r_buf, int64_t *s_buf, int64_t *ret_val, int type) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  r_buf = roc_shmemx_my_addr(r_buf);
+  s_buf = roc_shmemx_my_addr(s_buf);
+  if (threadIdx.x == 0 && roc_shmem_ctx_my_pe(ctx) == 0) {
+    int64_t ret = 0, cond = 0;
+    for (int i = 0; i < loop + skip; i++) {
+      switch (type) {
+        case PFAdd: ret = roc_shmem_ctx_int64_atomic_fetch_add(ctx, (int64_t *)r_buf, 2, 1); break;
+        case PFInc: ret = roc_shmem_ctx_int64_atomic_fetch_inc(ctx, (int64_t *)r_buf, 1); break;
+        case PFetch: ret = roc_shmem_ctx_int64_atomic_fetch(ctx, (int64_t *)r_buf, 1); break;
+        case PFCswap:
+          ret = roc_shmem_ctx_int64_atomic_compare_swap(ctx, (int64_t *)r_buf, cond, (int64_t)i, 1);
+          cond = i;
+          break;
+        case PAdd: roc_shmem_ctx_int64_atomic_add(ctx, (int64_t *)r_buf, 2, 1); break;
+        case PInc: roc_shmem_ctx_int64_atomic_inc(ctx, (int64_t *)r_buf, 1); break;
+        default: break;
+      }
+    }
+    roc_shmem_ctx_quiet(ctx);
+    ret_val[wg_index()] = ret;
+    // a get to check the result of the ops that fetch nothing
+    roc_shmem_ctx_getmem(ctx, &s_buf[wg_index()], r_buf, sizeof(int64_t), 1);
+  }
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+static void primitive_amo() {
+  current_case = "primitive_amo_tester.cpp";
+  const int loop = 100, skip = 10, max_wgs = 8;
+  int64_t *ret_val;
+  EXPECT(hipMalloc(&ret_val, max_wgs * sizeof(int64_t)) == hipSuccess, "hipMalloc");
+  char *r_buf = static_cast<char *>(roc_shmem_malloc(sizeof(int64_t)));
+  int64_t *s_buf = static_cast<int64_t *>(roc_shmem_malloc(max_wgs * sizeof(int64_t)));
+  for (int type = PFAdd; type <= PInc; ++type) {
+    // the compare-and-swap chain (cond = previous i) has a closed form for one workgroup only
+    for (int wgs : {1, max_wgs}) {
+      if (type == PFCswap && wgs > 1) continue;
+      for (int pe = 0; pe < npes; ++pe) {
+        fill(reinterpret_cast<int64_t *>(r_buf), 1, int64_t{0}, pe);
+        fill(s_buf, max_wgs, int64_t{0}, pe);
+      }
+      EXPECT(hipMemset(ret_val, 0, max_wgs * sizeof(int64_t)) == hipSuccess, "memset");
+      PrimitiveAMOTest<<<wgs * npes, 64>>>(loop, skip, r_buf, s_buf, ret_val, type);
+      finish_kernel("PrimitiveAMOTest");
+      const int64_t num_msgs = static_cast<int64_t>(loop + skip) * wgs;
+      int64_t expected = 0;
+      switch (type) {
+        case PFAdd: expected = 2 * (num_msgs - 1); break;
+        case PFInc: expected = num_msgs - 1; break;
+        case PAdd: expected = 2 * num_msgs; break;
+        case PInc: expected = num_msgs; break;
+        case PFCswap: expected = (num_msgs - 2) / wgs; break;
+        default: break;
+      }
+      int64_t fetched[max_wgs];
+      EXPECT(hipMemcpy(fetched, ret_val, sizeof(fetched), hipMemcpyDeviceToHost) == hipSuccess, "copy");
+      std::vector<int64_t> read_back = load(s_buf, max_wgs, 0);
+      int64_t best_ret = fetched[0], best_read = read_back[0];
+      for (int w = 1; w < wgs; ++w) {
+        best_ret = fetched[w] > best_ret ? fetched[w] : best_ret;
+        best_read = read_back[w] > best_read ? read_back[w] : best_read;
+      }
+      if (type <= PFCswap) {
+        EXPECT(best_ret == expected, "type %d, %d workgroups: fetched %ld, expected %ld", type, wgs,
+               static_cast<long>(best_ret), static_cast<long>(expected));
+      } else {
+        EXPECT(best_read == expected, "type %d, %d workgroups: read back %ld, expected %ld", type, wgs,
+               static_cast<long>(best_read), static_cast<long>(expected));
+      }
+    }
+  }
+  roc_shmem_free(s_buf);
+  roc_shmem_free(r_buf);
+  EXPECT(hipFree(ret_val) == hipSuccess, "hipFree");
+}
+
 int main() {
   if (!getenv("ROC_SHMEM_NUM_PES")) setenv("ROC_SHMEM_NUM_PES", "4", 1);
   setenv("ROC_SHMEM_HEAP_SIZE", "67108864", 0);
@@ -714,7 +853,8 @@ int main() {
                {"team_ctx_primitive", team_ctx_primitive}, {"sync_and_barrier", sync_and_barrier},
                {"swarm", swarm},               {"amo_testers", amo_testers},
                {"random_access", random_access},
-               {"default_ctx", default_ctx}};
+               {"default_ctx", default_ctx},   {"primitive_mr", primitive_mr},
+               {"primitive_amo", primitive_amo}};
   for (auto &c : cases) {
     const int before = failures;
     c.run();
