@@ -298,6 +298,44 @@ def bench_small_ops(rs, n_pes, n_ops, wgs_total, wg_size, slice_bytes, seed):
     return res
 
 
+def bench_small_collectives(rs, n_pes, n, calls):
+    """A launch-bound sequence: `calls` int64 sum_to_all of `n` elements back to back, issued call by
+    call and as one recorded graph.  Microseconds per collective."""
+    stream = rs.Stream()
+    src = rs.sym_array(n, np.int64, fill=1)
+    dst = rs.sym_array(n, np.int64, fill=0)
+    psync = rs.sym_array(rs.ROC_SHMEM_REDUCE_SYNC_SIZE, np.int64, fill=0)
+    launch = rs.Launch(1, 512, 0, stream)
+
+    def eager():
+        for _ in range(calls):
+            rs.roc_shmem_to_all(rs.LONG, rs.SUM, dst, src, n, 0, 0, n_pes, None, psync, launch)
+
+    with rs.Graph.capture(stream) as graph:
+        eager()
+    out = {}
+    for name, fn in (("eager_us", eager), ("graph_us", graph.launch)):
+        fn()
+        rs.synchronize()
+        start, stop = rs.Event(), rs.Event()
+        start.record(stream)
+        for _ in range(5):
+            fn()
+        stop.record(stream)
+        out[name] = start.elapsed_ms(stop) / 5 / calls * 1e3
+        start.destroy()
+        stop.destroy()
+    got = dst.read(n_pes - 1)
+    # every source byte is 1, so every byte of the sum over n_pes <= 255 slices is n_pes
+    if not (got.view(np.uint8) == n_pes).all() or rs.take_status():
+        raise RuntimeError("small collectives: wrong sum after the graph replays")
+    graph.destroy()
+    stream.destroy()
+    for a in (psync, dst, src):
+        a.free()
+    return out
+
+
 def bench_bcast_a2a(rs, n_pes, slice_bytes):
     world = rs.roc_shmem_team_world()
     res = {}
@@ -388,6 +426,7 @@ def main():
         barriers()
         rs.synchronize()
         extra["wg_barrier_all_4pe_us"] = event_time_ms(rs, barriers, 3) / 3 / rounds * 1e3
+        extra["sum_to_all_4096_int64_x100"] = bench_small_collectives(rs, 4, 4096, 100)
         rs.roc_shmem_finalize()
 
         rs.roc_shmem_init(16, 256 << 20, 64, 1024)

@@ -138,6 +138,20 @@ int rsm_event_destroy(void *event);
 int rsm_event_record(void *event, void *stream);
 int rsm_event_elapsed_ms(void *start, void *stop, float *ms);   /* synchronises on `stop` */
 
+/* Graphs (no counterpart in the reference; for launch-bound sequences of small
+ * operations).  The data-path entry points below (rsm_to_all*, rsm_broadcast*,
+ * rsm_alltoall, rsm_fcollect, rsm_barrier_all, rsm_putmem/rsm_getmem, rsm_small_ops)
+ * only launch kernels on launch->stream: between rsm_capture_begin(stream) and
+ * rsm_capture_end(stream) they are recorded instead of run.  rsm_capture_end returns
+ * an executable graph (NULL on error); rsm_graph_launch replays it on any stream.
+ * `stream` must come from rsm_stream_create.  Symmetric objects named by the
+ * recorded calls must stay allocated while the graph is in use; calls that copy,
+ * allocate or synchronise (lifecycle, memory, inspection) must stay outside. */
+int rsm_capture_begin(void *stream);
+void *rsm_capture_end(void *stream);
+int rsm_graph_launch(void *graph, void *stream);
+int rsm_graph_destroy(void *graph);
+
 /* ---- reductions ------------------------------------------------------------
  * roc_shmem_ctx_<T>_<op>_wg_to_all, active-set form (roc_shmem.hpp:837-851;
  * GPUIBContext::to_all, gpu_ib/context_ib_tmpl_device.hpp:262-307).  With

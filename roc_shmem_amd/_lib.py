@@ -47,6 +47,10 @@ SIGNATURES = {
     "rsm_event_destroy": (i32, [vp]),
     "rsm_event_record": (i32, [vp, vp]),
     "rsm_event_elapsed_ms": (i32, [vp, vp, C.POINTER(C.c_float)]),
+    "rsm_capture_begin": (i32, [vp]),
+    "rsm_capture_end": (vp, [vp]),
+    "rsm_graph_launch": (i32, [vp, vp]),
+    "rsm_graph_destroy": (i32, [vp]),
     "rsm_to_all": (i32, [i32, i32, vp, vp, sz, i32, i32, i32, vp, vp, LP]),
     "rsm_to_all_team": (i32, [i32, i32, u64, vp, vp, sz, LP]),
     "rsm_rma": (i32, [i32, i32, vp, vp, sz, sz, sz, sz, i32, LP]),

@@ -12,7 +12,7 @@ import numpy as np
 from . import _lib as L
 
 __all__ = [
-    "RocShmemError", "SymArray", "Launch",
+    "RocShmemError", "SymArray", "Launch", "Stream", "Graph",
     "roc_shmem_init", "roc_shmem_finalize", "roc_shmem_n_pes", "roc_shmem_malloc",
     "roc_shmem_free", "roc_shmem_ptr", "roc_shmem_team_world", "roc_shmem_team_split_strided",
     "roc_shmem_team_destroy", "roc_shmem_team_n_pes", "roc_shmem_team_translate_pe",
@@ -60,7 +60,7 @@ def _check(rc):
 
 
 def Launch(wgs_per_pe=1, wg_size=256, tile=0, stream=None):
-    return L.Launch(wgs_per_pe, wg_size, tile, stream)
+    return L.Launch(wgs_per_pe, wg_size, tile, getattr(stream, "h", stream))
 
 
 def _launch(launch):
@@ -229,7 +229,7 @@ class Event:
         self.h = L.load().rsm_event_create()
 
     def record(self, stream=None):
-        _check(L.load().rsm_event_record(self.h, stream))
+        _check(L.load().rsm_event_record(self.h, getattr(stream, "h", stream)))
 
     def elapsed_ms(self, stop):
         ms = C.c_float(0)
@@ -239,6 +239,50 @@ class Event:
     def destroy(self):
         if self.h:
             L.load().rsm_event_destroy(self.h)
+            self.h = None
+
+
+class Stream:
+    def __init__(self):
+        self.h = L.load().rsm_stream_create()
+        if not self.h:
+            raise RocShmemError(L.load().rsm_last_error().decode())
+
+    def destroy(self):
+        if self.h:
+            L.load().rsm_stream_destroy(self.h)
+            self.h = None
+
+
+class Graph:
+    """A recorded run of data-path calls: ``with Graph.capture(stream) as g:`` records every
+    data-path call whose launch names ``stream``; ``g.launch(stream)`` replays them as one
+    submission."""
+
+    def __init__(self, stream):
+        self.stream = stream
+        self.h = None
+
+    @classmethod
+    def capture(cls, stream):
+        return cls(stream)
+
+    def __enter__(self):
+        _check(L.load().rsm_capture_begin(self.stream.h))
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        self.h = L.load().rsm_capture_end(self.stream.h)
+        if not self.h and exc_type is None:
+            raise RocShmemError(L.load().rsm_last_error().decode())
+        return False
+
+    def launch(self, stream=None):
+        _check(L.load().rsm_graph_launch(self.h, (stream or self.stream).h))
+
+    def destroy(self):
+        if self.h:
+            L.load().rsm_graph_destroy(self.h)
             self.h = None
 
 

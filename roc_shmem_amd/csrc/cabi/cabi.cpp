@@ -257,6 +257,43 @@ int rsm_event_elapsed_ms(void *start, void *stop, float *ms) {
   return 0;
 }
 
+// ---- graphs --------------------------------------------------------------------
+// The data-path entry points only launch kernels on launch->stream, so a run of
+// them can be recorded once and replayed as one submission.
+
+int rsm_capture_begin(void *stream) {
+  if (!stream) return rsm::fail("rsm_capture_begin: capture needs a stream of its own, not the default stream");
+  RSM_HIP(hipStreamBeginCapture(static_cast<hipStream_t>(stream), hipStreamCaptureModeThreadLocal));
+  return 0;
+}
+
+void *rsm_capture_end(void *stream) {
+  hipGraph_t graph = nullptr;
+  hipError_t e = hipStreamEndCapture(static_cast<hipStream_t>(stream), &graph);
+  if (e != hipSuccess || !graph) {
+    rsm::fail(std::string("rsm_capture_end: ") + hipGetErrorString(e));
+    return nullptr;
+  }
+  hipGraphExec_t exec = nullptr;
+  e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  if (e != hipSuccess) {
+    rsm::fail(std::string("rsm_capture_end: hipGraphInstantiate: ") + hipGetErrorString(e));
+    return nullptr;
+  }
+  return exec;
+}
+
+int rsm_graph_launch(void *graph, void *stream) {
+  RSM_HIP(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), static_cast<hipStream_t>(stream)));
+  return 0;
+}
+
+int rsm_graph_destroy(void *graph) {
+  RSM_HIP(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)));
+  return 0;
+}
+
 // ---- send-queue inspection ---------------------------------------------------
 
 static bool sq_args_ok(Runtime *rt, int pe, int block) {
