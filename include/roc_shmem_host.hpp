@@ -309,6 +309,66 @@ ROCSHMEM_HOST_STANDARD_TYPES(ROCSHMEM_HOST_WAIT)
 ROCSHMEM_HOST_AMO_TYPES(ROCSHMEM_HOST_AMO)
 #undef ROCSHMEM_HOST_AMO
 
+// fetch / set / swap also exist for float and double (reference: roc_shmem.hpp:1647-1648,
+// 1713-1714,1747-1748): the word is moved as its bit pattern.
+#define ROCSHMEM_HOST_AMO_FLOATING(T, TNAME)                                                   \
+  __host__ inline T roc_shmem_ctx_##TNAME##_atomic_fetch(roc_shmem_ctx_t, T *dest, int pe) {   \
+    return hostx::from_bits<T>(hostx::amo(0, dest, 0, 0, pe, sizeof(T)));                      \
+  }                                                                                            \
+  __host__ inline T roc_shmem_##TNAME##_atomic_fetch(T *dest, int pe) {                        \
+    return hostx::from_bits<T>(hostx::amo(0, dest, 0, 0, pe, sizeof(T)));                      \
+  }                                                                                            \
+  __host__ inline T roc_shmem_ctx_##TNAME##_atomic_swap(roc_shmem_ctx_t, T *dest, T value,     \
+                                                        int pe) {                              \
+    return hostx::from_bits<T>(hostx::amo(2, dest, hostx::to_bits(value), 0, pe, sizeof(T)));  \
+  }                                                                                            \
+  __host__ inline T roc_shmem_##TNAME##_atomic_swap(T *dest, T value, int pe) {                \
+    return hostx::from_bits<T>(hostx::amo(2, dest, hostx::to_bits(value), 0, pe, sizeof(T)));  \
+  }                                                                                            \
+  __host__ inline void roc_shmem_ctx_##TNAME##_atomic_set(roc_shmem_ctx_t, T *dest, T value,   \
+                                                          int pe) {                            \
+    (void)hostx::amo(2, dest, hostx::to_bits(value), 0, pe, sizeof(T));                        \
+  }                                                                                            \
+  __host__ inline void roc_shmem_##TNAME##_atomic_set(T *dest, T value, int pe) {              \
+    (void)hostx::amo(2, dest, hostx::to_bits(value), 0, pe, sizeof(T));                        \
+  }
+ROCSHMEM_HOST_AMO_FLOATING(float, float)
+ROCSHMEM_HOST_AMO_FLOATING(double, double)
+#undef ROCSHMEM_HOST_AMO_FLOATING
+
+// Bitwise operations (reference: roc_shmem.hpp:1068-1147,1781-1953): seven types.
+#define ROCSHMEM_HOST_AMO_BITWISE_TYPES(X) \
+  X(unsigned int, uint)                    \
+  X(unsigned long, ulong)                  \
+  X(unsigned long long, ulonglong)         \
+  X(int32_t, int32)                        \
+  X(int64_t, int64)                        \
+  X(uint32_t, uint32)                      \
+  X(uint64_t, uint64)
+
+#define ROCSHMEM_HOST_AMO_BITWISE_ONE(T, TNAME, OP, KIND)                                      \
+  __host__ inline T roc_shmem_ctx_##TNAME##_atomic_fetch_##OP(roc_shmem_ctx_t, T *dest,        \
+                                                              T value, int pe) {               \
+    return hostx::from_bits<T>(hostx::amo(KIND, dest, hostx::to_bits(value), 0, pe, sizeof(T))); \
+  }                                                                                            \
+  __host__ inline T roc_shmem_##TNAME##_atomic_fetch_##OP(T *dest, T value, int pe) {          \
+    return hostx::from_bits<T>(hostx::amo(KIND, dest, hostx::to_bits(value), 0, pe, sizeof(T))); \
+  }                                                                                            \
+  __host__ inline void roc_shmem_ctx_##TNAME##_atomic_##OP(roc_shmem_ctx_t, T *dest, T value,  \
+                                                           int pe) {                           \
+    (void)hostx::amo(KIND, dest, hostx::to_bits(value), 0, pe, sizeof(T));                     \
+  }                                                                                            \
+  __host__ inline void roc_shmem_##TNAME##_atomic_##OP(T *dest, T value, int pe) {             \
+    (void)hostx::amo(KIND, dest, hostx::to_bits(value), 0, pe, sizeof(T));                     \
+  }
+#define ROCSHMEM_HOST_AMO_BITWISE(T, TNAME)          \
+  ROCSHMEM_HOST_AMO_BITWISE_ONE(T, TNAME, and, 3)    \
+  ROCSHMEM_HOST_AMO_BITWISE_ONE(T, TNAME, or, 4)     \
+  ROCSHMEM_HOST_AMO_BITWISE_ONE(T, TNAME, xor, 5)
+ROCSHMEM_HOST_AMO_BITWISE_TYPES(ROCSHMEM_HOST_AMO_BITWISE)
+#undef ROCSHMEM_HOST_AMO_BITWISE
+#undef ROCSHMEM_HOST_AMO_BITWISE_ONE
+
 }  // namespace rocshmem
 
 #endif

@@ -727,6 +727,11 @@ ROCSHMEM_AMO_BITWISE_TYPES(ROCSHMEM_AMO_BITWISE)
 #define ROCSHMEM_WAIT_TYPES(X) \
   X(float, float)              \
   X(double, double)            \
+  X(char, char)                \
+  X(signed char, schar)        \
+  X(short, short)              \
+  X(unsigned char, uchar)      \
+  X(unsigned short, ushort)    \
   X(int, int)                  \
   X(long, long)                \
   X(long long, longlong)       \
@@ -740,7 +745,7 @@ ROCSHMEM_AMO_BITWISE_TYPES(ROCSHMEM_AMO_BITWISE)
     detail::fence_acquire_agent();                                                             \
   }                                                                                            \
   __device__ inline int roc_shmem_##TNAME##_test(T *ptr, roc_shmem_cmps cmp, T val) {          \
-    using W = typename detail::AtomicWord<T>::type;                                            \
+    using W = typename detail::WaitWord<T>::type;                                              \
     W raw = __hip_atomic_load(reinterpret_cast<W *>(ptr), __ATOMIC_RELAXED,                    \
                               __HIP_MEMORY_SCOPE_AGENT);                                       \
     T have;                                                                                    \

@@ -67,9 +67,19 @@ __device__ __forceinline__ bool compare_for_wait(T have, int cmp, T want) {
 // (the reference polls with uncached loads, context_tmpl_device.hpp:199-246).
 // Returns false on timeout or when the status word is already raised.
 template <typename T>
+struct WaitWord {
+  static_assert(sizeof(T) == 1 || sizeof(T) == 2 || sizeof(T) == 4 || sizeof(T) == 8,
+                "wait on naturally aligned words of 1, 2, 4 or 8 bytes");
+  using type = typename std::conditional<
+      sizeof(T) == 8, uint64_t,
+      typename std::conditional<sizeof(T) == 4, uint32_t,
+                                typename std::conditional<sizeof(T) == 2, uint16_t,
+                                                          uint8_t>::type>::type>::type;
+};
+
+template <typename T>
 __device__ __forceinline__ bool bounded_wait(const T *ptr, int cmp, T want) {
-  using Word = typename std::conditional<sizeof(T) == 8, uint64_t, uint32_t>::type;
-  static_assert(sizeof(T) == 4 || sizeof(T) == 8, "wait on 4- or 8-byte words");
+  using Word = typename WaitWord<T>::type;
   const Word *wptr = reinterpret_cast<const Word *>(ptr);
   uint64_t start = wall_clock64();
   uint32_t spins = 0;

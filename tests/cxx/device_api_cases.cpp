@@ -155,6 +155,71 @@ static void compare_ops() {
   roc_shmem_free(word);
 }
 
+// ---- the ping-pong of ping_pong_tester.cpp on 1- and 2-byte words (roc_shmem.hpp:1973-2019 declares
+// wait_until / test for char, schar, short, uchar and ushort as well): neighbouring workgroups
+// use neighbouring bytes, so four flags share one 32-bit word.
+#define NARROW_PING_PONG(T, TNAME)                                                        \
+  __global__ void PingPong_##TNAME(int loop, T *r_buf, int *bad) {                       \
+    __shared__ roc_shmem_ctx_t ctx;                                                       \
+    roc_shmem_wg_init();                                                                  \
+    roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);                              \
+    int pe = roc_shmem_ctx_my_pe(ctx);                                                    \
+    r_buf = roc_shmemx_my_addr(r_buf);                                                    \
+    const int w = wg_index();                                                             \
+    if (threadIdx.x == 0 && pe < 2) {                                                     \
+      for (int i = 0; i < loop; i++) {                                                    \
+        const T v = static_cast<T>(i + 1);                                                \
+        if (pe == 0) {                                                                    \
+          roc_shmem_ctx_##TNAME##_p(ctx, &r_buf[w], v, 1);                                \
+          roc_shmem_##TNAME##_wait_until(&r_buf[w], ROC_SHMEM_CMP_EQ, v);                 \
+        } else {                                                                          \
+          for (int spins = 0; spins < (1 << 22); ++spins) /* bounded: never hangs */      \
+            if (roc_shmem_##TNAME##_test(&r_buf[w], ROC_SHMEM_CMP_GE, v)) break;          \
+          if (r_buf[w] != v) atomicAdd(bad, 1);                                           \
+          roc_shmem_ctx_##TNAME##_p(ctx, &r_buf[w], v, 0);                                \
+        }                                                                                 \
+      }                                                                                   \
+    }                                                                                     \
+    roc_shmem_wg_ctx_destroy(ctx);                                                        \
+    roc_shmem_wg_finalize();                                                              \
+  }                                                                                       \
+  static void narrow_ping_pong_##TNAME() {                                                \
+    const int wgs = 4, loop = 100;                                                        \
+    T *r_buf = static_cast<T *>(roc_shmem_malloc(16));                                    \
+    int *bad = nullptr;                                                                   \
+    (void)hipMalloc(reinterpret_cast<void **>(&bad), sizeof(int));                        \
+    (void)hipMemset(bad, 0, sizeof(int));                                                 \
+    for (int pe = 0; pe < npes; ++pe) fill(r_buf, static_cast<int>(16 / sizeof(T)), static_cast<T>(0), pe); \
+    PingPong_##TNAME<<<wgs * npes, 64>>>(loop, r_buf, bad);                               \
+    finish_kernel("PingPong_" #TNAME);                                                    \
+    int h = -1;                                                                           \
+    (void)hipMemcpy(&h, bad, sizeof(int), hipMemcpyDeviceToHost);                         \
+    EXPECT(h == 0, #TNAME ": %d rounds saw a value other than the one sent", h);          \
+    for (int pe = 0; pe < 2; ++pe) {                                                      \
+      std::vector<T> got = load(r_buf, static_cast<int>(16 / sizeof(T)), pe);             \
+      for (int w = 0; w < wgs; ++w)                                                       \
+        EXPECT(got[w] == static_cast<T>(loop), #TNAME ": PE %d flag %d ends at %d", pe, w, (int)got[w]); \
+      EXPECT(got[wgs] == 0, #TNAME ": the word after the flags was written on PE %d", pe); \
+    }                                                                                     \
+    (void)hipFree(bad);                                                                   \
+    roc_shmem_free(r_buf);                                                                \
+  }
+NARROW_PING_PONG(short, short)
+NARROW_PING_PONG(unsigned char, uchar)
+NARROW_PING_PONG(signed char, schar)
+NARROW_PING_PONG(unsigned short, ushort)
+NARROW_PING_PONG(char, char)
+#undef NARROW_PING_PONG
+
+static void narrow_ping_pong() {
+  current_case = "wait_until / test on 1- and 2-byte words";
+  narrow_ping_pong_short();
+  narrow_ping_pong_uchar();
+  narrow_ping_pong_schar();
+  narrow_ping_pong_ushort();
+  narrow_ping_pong_char();
+}
+
 // ---- shmem_ptr_tester.cpp:31-44 ------------------------------------------------------------------
 __global__ void ShmemPtrTest(char *r_buf, int *available) {
   roc_shmem_wg_init();
@@ -849,6 +914,7 @@ int main() {
     const char *name;
     void (*run)();
   } cases[] = {{"ping_pong", ping_pong},       {"compare_ops", compare_ops},
+               {"narrow_ping_pong", narrow_ping_pong},
                {"shmem_ptr", shmem_ptr},       {"team_ctx_infra", team_ctx_infra},
                {"team_ctx_primitive", team_ctx_primitive}, {"sync_and_barrier", sync_and_barrier},
                {"swarm", swarm},               {"amo_testers", amo_testers},

@@ -2,6 +2,7 @@
 // header, checked against closed forms (the style of the reference's
 // functional tests, clients/functional_tests/*_tester.cpp verify_results).
 // Exit code 0 and a final line "HOST_API_OK" mean every check passed.
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <vector>
@@ -182,6 +183,30 @@ int main() {
   roc_shmem_uint_p(ucounter, 0xfffffffeu, 1);
   EXPECT(roc_shmem_uint_atomic_fetch_add(ucounter, 3u, 1) == 0xfffffffeu, "uint fetch_add");
   EXPECT(roc_shmem_uint_g(ucounter, 1) == 1u, "uint wrap");
+
+  // Bitwise and floating-point AMOs of the host interface (roc_shmem.hpp:1647-1648,1713-1714,
+  // 1747-1748,1781-1953).
+  roc_shmem_uint_p(ucounter, 0xf0f0u, 2);
+  EXPECT(roc_shmem_uint_atomic_fetch_and(ucounter, 0xff00u, 2) == 0xf0f0u, "fetch_and");
+  EXPECT(roc_shmem_uint_atomic_fetch_or(ucounter, 0x000fu, 2) == 0xf000u, "fetch_or");
+  EXPECT(roc_shmem_uint_atomic_fetch_xor(ucounter, 0xffffu, 2) == 0xf00fu, "fetch_xor");
+  roc_shmem_uint_atomic_and(ucounter, 0x0ff0u, 2);
+  roc_shmem_uint_atomic_or(ucounter, 0x1000u, 2);
+  roc_shmem_uint_atomic_xor(ucounter, 0x0001u, 2);
+  EXPECT(roc_shmem_uint_g(ucounter, 2) == 0x1ff1u, "and/or/xor: %x", roc_shmem_uint_g(ucounter, 2));
+  uint64_t *wide = reinterpret_cast<uint64_t *>(dst);
+  roc_shmem_ctx_uint64_atomic_set(ctx, wide, 0xffff0000ffff0000ull, 1);
+  EXPECT(roc_shmem_ctx_uint64_atomic_fetch_xor(ctx, wide, ~0ull, 1) == 0xffff0000ffff0000ull, "uint64 fetch_xor");
+  EXPECT(roc_shmem_uint64_atomic_fetch(wide, 1) == 0x0000ffff0000ffffull, "uint64 after xor");
+  roc_shmem_float_atomic_set(fdst, 2.5f, 3);
+  EXPECT(roc_shmem_float_atomic_fetch(fdst, 3) == 2.5f, "float fetch");
+  EXPECT(roc_shmem_float_atomic_swap(fdst, -7.25f, 3) == 2.5f, "float swap");
+  EXPECT(roc_shmem_float_g(fdst, 3) == -7.25f, "float after swap");
+  double *dword = reinterpret_cast<double *>(dst) + 8;
+  roc_shmem_ctx_double_atomic_set(ctx, dword, 1e300, 0);
+  EXPECT(roc_shmem_ctx_double_atomic_swap(ctx, dword, -0.0, 0) == 1e300, "double swap");
+  EXPECT(roc_shmem_double_atomic_fetch(dword, 0) == 0.0 && std::signbit(roc_shmem_double_atomic_fetch(dword, 0)),
+         "double keeps its bit pattern");
 
   // The heap is host-visible, as the reference's is: host code may read and write symmetric
   // objects through plain pointers (roc_shmemx_host_ptr gives PE pe's address), with
