@@ -1,0 +1,45 @@
+"""Function names a roc_shmem header declares, per side (__host__ / __device__), found by
+expanding the header's own function-like macros textually.  Used to write
+reference_api_names.json from the reference's public header and, in
+tests/test_api_surface.py, to read the same from this repository's headers."""
+import re
+
+
+def names_of(paths):
+    txt = "\n".join(open(p).read() for p in paths)
+    txt = re.sub(r"//[^\n]*", "", txt)
+    txt = re.sub(r"/\*.*?\*/", "", txt, flags=re.S)
+    txt = re.sub(r"\\\n", " ", txt)
+    macros = {}
+    for m in re.finditer(r"#define\s+(\w+)\(([^)]*)\)\s+(.*)", txt):
+        macros[m.group(1)] = ([p.strip() for p in m.group(2).split(",")], m.group(3))
+    host, device = set(), set()
+
+    def collect(s):
+        host.update(re.findall(r"__host__[^;({]*?\b(roc_shmemx?_\w+)\s*\(", s))
+        device.update(re.findall(r"__device__[^;({]*?\b(roc_shmemx?_\w+)\s*\(", s))
+
+    plain = re.sub(r"#define[^\n]*", "", txt)
+    collect(plain)
+
+    def expand(text, depth=0):
+        for m in re.finditer(r"\b(\w+)\(([^()]*)\)", text):
+            mac, args = m.group(1), [a.strip() for a in m.group(2).split(",")]
+            if mac not in macros:
+                continue
+            params, body = macros[mac]
+            if len(params) != len(args):
+                continue
+            for p, a in zip(params, args):
+                p = re.escape(p)
+                body = re.sub(r"##\s*%s\s*##" % p, a, body)
+                body = re.sub(r"##\s*%s\b" % p, a, body)
+                body = re.sub(r"\b%s\s*##" % p, a, body)
+                body = re.sub(r"\b%s\b" % p, a, body)
+            body = body.replace("##", "")
+            collect(body)
+            if depth < 3:
+                expand(body, depth + 1)
+
+    expand(plain)
+    return sorted(host), sorted(device)
