@@ -32,3 +32,37 @@ def test_the_scan_sees_macro_generated_names():
     for name in ("roc_shmem_malloc", "roc_shmem_long_wait_until", "roc_shmem_uint64_atomic_fetch_xor",
                  "roc_shmem_ctx_double_prod_to_all"):
         assert name in host, name
+
+
+def test_every_reference_declaration_resolves_with_its_exact_signature(tmp_path):
+    """tests/golden/reference_api_signatures.json holds side, return type, name and parameter types
+    of the reference header's 1454 declarations (tests/golden/make_api_signatures.py).  A program
+    that initialises a function pointer of exactly that type from each name must compile against
+    this repository's header, in a __device__ function for the device side and in a host function
+    for the host side: a missing overload or a parameter of another type is a compile error."""
+    import shutil
+    import subprocess
+
+    import pytest
+
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not found")
+    with open(os.path.join(ROOT, "tests", "golden", "reference_api_signatures.json")) as f:
+        decls = json.load(f)["declarations"]
+    assert len(decls) > 1400
+    lines = ['#include "roc_shmem.hpp"', "using namespace rocshmem;"]
+    for side, opener in (("device", "__device__ void device_side() {"), ("host", "void host_side() {")):
+        lines.append(opener)
+        for s, ret, name, params in decls:
+            if s == side:
+                lines.append("  { %s (*f)(%s) = %s; (void)f; }" % (ret, ", ".join(params), name))
+        lines.append("}")
+    src = tmp_path / "signatures.cpp"
+    src.write_text("\n".join(lines) + "\n")
+    cmd = [hipcc, "-x", "hip", "--offload-arch=gfx950", "-std=c++17", "-DROCSHMEM_NO_MPI", "-fsyntax-only",
+           "-Wno-unused-command-line-argument", "-I", os.path.join(ROOT, "include"),
+           "-I", os.path.join(ROOT, "roc_shmem_amd", "csrc"), str(src)]
+    run = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+    errors = [ln for ln in run.stderr.splitlines() if "error" in ln]
+    assert run.returncode == 0 and not errors, "\n".join(errors[:20])
