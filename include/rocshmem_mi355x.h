@@ -85,6 +85,14 @@ typedef struct rsm_small_op {
   int64_t aux;
 } rsm_small_op_t;
 
+/* Argument checks of the data-path entry points.  A symmetric operand must lie
+ * inside a live allocation of rsm_malloc and the bytes the call touches
+ * (elements x element size, team size x block, messages x stride, wgs_per_pe
+ * pSync slices) must fit that allocation; otherwise the call returns non-zero
+ * with a message in rsm_last_error() and launches nothing.  The reference
+ * checks none of this; a kernel that runs past an allocation overwrites its
+ * neighbours or faults the device. */
+
 /* Launch shape shared by the data-path entry points. */
 typedef struct rsm_launch {
   int wgs_per_pe;   /* workgroups acting for each PE (>= 1)                        */
@@ -206,7 +214,9 @@ int rsm_barrier_all(int iterations, const rsm_launch_t *launch);
  * context_ib_tmpl_device.hpp:365-453), every op also leaving its 64-byte WQE
  * in the issuing workgroup's send queue (queue_pair.cpp:205-273).  `ops` is
  * device memory.  `fetched` (device, n_ops int64, may be NULL) receives the
- * value returned by fetching operations. */
+ * value returned by fetching operations.  An operation that names a PE that
+ * does not exist or bytes outside the heap is skipped and raises the status
+ * word (rsm_take_status() == 2) instead of faulting the device. */
 int rsm_small_ops(const rsm_small_op_t *ops, size_t n_ops, int64_t *fetched,
                   const rsm_launch_t *launch);
 

@@ -63,6 +63,27 @@ bool check_symmetric(const void *p, const char *what, bool allow_null) {
   return true;
 }
 
+bool check_extent(const void *p, size_t bytes, const char *what) {
+  using rocshmem::host::Pow2Allocator;
+  using rocshmem::host::Runtime;
+  Runtime *rt = Runtime::get();
+  if (!rt || !p || !rt->owns(p)) return true;  // not symmetric: nothing to compare with
+  const size_t offset = (static_cast<const char *>(p) - rt->arena()) % rt->slice_stride();
+  const size_t end = rt->allocation_end(offset);
+  if (end == Pow2Allocator::kNoOffset) {
+    fail(std::string(what) + ": the address (heap offset " + std::to_string(offset) +
+         ") is not inside a live symmetric allocation");
+    return false;
+  }
+  if (bytes > end - offset) {
+    fail(std::string(what) + ": " + std::to_string(bytes) + " bytes at heap offset " +
+         std::to_string(offset) + " do not fit the symmetric allocation that holds them (it ends at offset " +
+         std::to_string(end) + ")");
+    return false;
+  }
+  return true;
+}
+
 int after_launch(const char *what) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(std::string(what) + ": " + hipGetErrorString(e));

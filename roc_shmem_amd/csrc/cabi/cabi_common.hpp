@@ -27,6 +27,10 @@ bool resolve_launch(const rsm_launch_t *in, Launch *out);
 
 // True when `p` is a symmetric address in PE 0's slice (or NULL when allowed).
 bool check_symmetric(const void *p, const char *what, bool allow_null = false);
+// `bytes` starting at the symmetric address `p` stay inside the live symmetric allocation that
+// contains `p` (a kernel that ran past it would overwrite its neighbours or fault the device);
+// true for addresses outside the arena, which cannot be judged here.
+bool check_extent(const void *p, size_t bytes, const char *what);
 
 // hipGetLastError() after a launch, folded into the error convention.
 int after_launch(const char *what);

@@ -162,6 +162,12 @@ void launch_bcast(const rsm::Launch &l, const BcastArgs &a) {
 
 int run_bcast(size_t elem_size, const rsm::Launch &l, BcastArgs a) {
   if (a.n == 0) return 0;
+  if (elem_size == 0 || elem_size > 8 || a.n > (~size_t{0} >> 4) ||
+      !rsm::check_extent(a.dest, a.n * elem_size, "broadcast: dest") ||
+      !rsm::check_extent(a.source, a.n * elem_size, "broadcast: source") ||
+      !rsm::check_extent(a.pSync, static_cast<size_t>(l.wgs_per_pe) * ROC_SHMEM_BCAST_SYNC_SIZE * sizeof(long),
+                         "broadcast: pSync (wgs_per_pe slices of ROC_SHMEM_BCAST_SYNC_SIZE longs)"))
+    return -1;
   // tile == 0: the PE's workgroups share one broadcast through the sharded extension.
   if (a.tile > 0x7fffffffull) return rsm::fail("broadcast: tile does not fit the API's int nelem");
   switch (elem_size) {
@@ -190,6 +196,11 @@ int run_exchange(size_t elem_size, uint64_t team, void *dest, const void *source
   const detail::TeamInfo &ti = rec->image.wrt_world;
   roc_shmem_team_t t = reinterpret_cast<roc_shmem_team_t>(team);
   const int n = static_cast<int>(nelem);
+  if (elem_size == 0 || elem_size > 8) return rsm::fail("alltoall/fcollect: element size must be 1, 2, 4 or 8");
+  const size_t block = nelem * elem_size, all_blocks = block * static_cast<size_t>(ti.size);
+  if (!rsm::check_extent(dest, all_blocks, "alltoall/fcollect: dest (team size blocks)") ||
+      !rsm::check_extent(source, kFcollect ? block : all_blocks, "alltoall/fcollect: source"))
+    return -1;
 #define RSM_EXCHANGE(T)                                                                        \
   hipLaunchKernelGGL((exchange_kernel<T, kFcollect>), dim3(l.grid), dim3(l.wg_size), 0,        \
                      l.stream, t, static_cast<T *>(dest), static_cast<const T *>(source), n,   \

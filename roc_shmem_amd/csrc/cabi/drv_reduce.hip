@@ -208,6 +208,11 @@ int run(int dtype, int op, const rsm::Launch &l, ReduceArgs a) {
   const size_t es = dtype_size(dtype);
   if (!es) return rsm::fail("to_all: unknown dtype");
   if (a.n == 0) return 0;  // zero-element reductions are no-ops (context_tmpl_device.hpp:68-70)
+  if (a.n > (~size_t{0} >> 4) || !rsm::check_extent(a.dest, a.n * es, "to_all: dest") ||
+      !rsm::check_extent(a.source, a.n * es, "to_all: source") ||
+      !rsm::check_extent(a.pSync, static_cast<size_t>(l.wgs_per_pe) * ROC_SHMEM_REDUCE_SYNC_SIZE * sizeof(long),
+                         "to_all: pSync (wgs_per_pe slices of ROC_SHMEM_REDUCE_SYNC_SIZE longs)"))
+    return -1;
   // tile == 0: the PE's workgroups share one reduction through the sharded
   // extension; otherwise each standard call covers `tile` elements.
   if (a.tile > 0x7fffffffull) return rsm::fail("to_all: tile does not fit the API's int nreduce");

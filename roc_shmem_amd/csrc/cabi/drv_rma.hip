@@ -96,6 +96,12 @@ extern "C" int rsm_rma(int kind, int granularity, void *dest, const void *source
   if (rt->pe_of(remote) != 0) return rsm::fail("rma: the remote buffer is not a symmetric address of PE 0");
   if (pe_shift < 0) return rsm::fail("rma: pe_shift must be non-negative");
   if (n_msgs == 0) return 0;
+  // Both sides of every message must stay inside the heap when they are symmetric.
+  if (msg_bytes > (~size_t{0} >> 2) || n_msgs > (~size_t{0} >> 2) / (dst_stride | src_stride | 1))
+    return rsm::fail("rma: sizes overflow");
+  if (!rsm::check_extent(dest, (n_msgs - 1) * dst_stride + msg_bytes, "rma: dest") ||
+      !rsm::check_extent(source, (n_msgs - 1) * src_stride + msg_bytes, "rma: source"))
+    return -1;
   hipLaunchKernelGGL(rma_kernel, dim3(l.grid), dim3(l.wg_size), 0, l.stream, kind, granularity,
                      static_cast<char *>(dest), static_cast<const char *>(source), msg_bytes,
                      n_msgs, dst_stride, src_stride, pe_shift);

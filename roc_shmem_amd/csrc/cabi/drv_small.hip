@@ -22,6 +22,18 @@ __global__ void __launch_bounds__(1024)
        i += total) {
     const rsm_small_op_t op = ops[i];
     const int pe = static_cast<int>(op.pe);
+    // An operation that names a PE or bytes outside the heap is skipped and reported through
+    // the status word; issued, it would fault the device.
+    const uint64_t heap_bytes = detail::g_state.heap_size;
+    const bool bulk = op.kind == RSM_OP_PUTMEM || op.kind == RSM_OP_GETMEM;
+    const uint64_t width = bulk ? static_cast<uint64_t>(op.aux)
+                                : (op.kind == RSM_OP_P32 || op.kind == RSM_OP_FADD32 ? 4u : 8u);
+    const uint64_t local = bulk ? static_cast<uint64_t>(op.value) : 0u;
+    if (op.pe >= static_cast<uint32_t>(detail::g_state.num_pes) || width > heap_bytes ||
+        op.offset > heap_bytes - width || local > heap_bytes - width) {
+      detail::status_raise(detail::kStatusBadArgument);
+      continue;
+    }
     char *sym = heap + op.offset;
     int64_t got = 0;
     bool fetches = false;

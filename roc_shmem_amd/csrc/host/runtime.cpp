@@ -68,6 +68,13 @@ bool Pow2Allocator::free(size_t offset) {
   return true;
 }
 
+size_t Pow2Allocator::block_end(size_t offset) const {
+  auto it = outstanding_.upper_bound(offset);
+  if (it == outstanding_.begin()) return kNoOffset;
+  --it;
+  return offset < it->first + it->second ? it->first + it->second : kNoOffset;
+}
+
 size_t Pow2Allocator::bytes_in_use() const {
   size_t total = 0;
   for (const auto &kv : outstanding_) total += kv.second;
@@ -299,7 +306,11 @@ int Runtime::pe_of(const void *p) const {
 }
 
 void *Runtime::sym_malloc(size_t bytes) {
-  size_t off = alloc_.alloc(bytes);
+  size_t off;
+  {
+    std::lock_guard<std::mutex> alloc_guard(alloc_mu_);
+    off = alloc_.alloc(bytes);
+  }
   if (off == Pow2Allocator::kNoOffset) return nullptr;
   return slice_base(current_pe_) + off;
 }
@@ -307,6 +318,7 @@ void *Runtime::sym_malloc(size_t bytes) {
 bool Runtime::sym_free(void *ptr) {
   if (!ptr || !owns(ptr)) return false;
   size_t off = (static_cast<char *>(ptr) - arena_) % stride_;
+  std::lock_guard<std::mutex> alloc_guard(alloc_mu_);
   return alloc_.free(off);
 }
 
@@ -321,7 +333,9 @@ TeamRecord *Runtime::make_team(const detail::TeamInfo &info) {
   // Four pSync pools, one kSyncSlots-long slice per context block each
   // (reference: per-team pool slices, gpu_ib_team.cpp:30-52, backend_ib.cpp:335-381).
   const size_t pool_bytes = static_cast<size_t>(opt_.num_blocks) * detail::kSyncSlots * sizeof(long);
+  std::unique_lock<std::mutex> alloc_guard(alloc_mu_);
   size_t off = alloc_.alloc(4 * pool_bytes);
+  alloc_guard.unlock();
   if (off == Pow2Allocator::kNoOffset) return nullptr;
   for (int p = 0; p < opt_.num_pes; ++p) {
     if (hipMemset(slice_base(p) + off, 0, 4 * pool_bytes) != hipSuccess) return nullptr;
@@ -377,7 +391,9 @@ int Runtime::team_split(detail::Team *parent, int start, int stride, int size,
 void Runtime::team_destroy(detail::Team *team) {
   auto it = teams_.find(team);
   if (it == teams_.end() || &it->second == world_) return;
+  std::unique_lock<std::mutex> alloc_guard(alloc_mu_);
   alloc_.free(it->second.pool_offset);
+  alloc_guard.unlock();
   free_team_slots_.push_back(static_cast<int>(it->second.device - teams_dev_));
   teams_.erase(it);
 }
@@ -408,7 +424,9 @@ void Runtime::reset_queues(hipStream_t stream) {
 long *Runtime::host_psync() {
   if (!host_psync_) {
     const size_t bytes = static_cast<size_t>(opt_.num_blocks) * detail::kSyncSlots * sizeof(long);
+    std::unique_lock<std::mutex> alloc_guard(alloc_mu_);
     size_t off = alloc_.alloc(bytes);
+    alloc_guard.unlock();
     if (off == Pow2Allocator::kNoOffset) return nullptr;
     for (int p = 0; p < opt_.num_pes; ++p) {
       if (hipMemset(slice_base(p) + off, 0, bytes) != hipSuccess) return nullptr;

@@ -9,6 +9,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <map>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -35,6 +36,8 @@ class Pow2Allocator {
   size_t alloc(size_t request);  // kNoOffset when nothing fits (or request == 0)
   bool free(size_t offset);      // false when `offset` is not an outstanding allocation
   size_t bytes_in_use() const;
+  // End offset of the outstanding block that contains `offset`, kNoOffset when there is none.
+  size_t block_end(size_t offset) const;
   size_t heap_bytes() const { return heap_bytes_; }
 
  private:
@@ -85,7 +88,10 @@ class Runtime {
   void *sym_malloc(size_t bytes);   // address in the current PE's slice, nullptr on failure
   bool sym_free(void *ptr);
   void *translate(const void *ptr, int pe) const;
-  size_t bytes_in_use() const { return alloc_.bytes_in_use(); }
+  size_t bytes_in_use() const {
+    std::lock_guard<std::mutex> lk(alloc_mu_);
+    return alloc_.bytes_in_use();
+  }
 
   detail::Team *team_world() const { return world_->device; }
   // 0 on success (handle in *out, nullptr if arguments describe no team), -1 on bad arguments.
@@ -110,6 +116,12 @@ class Runtime {
   bool sq_queue_mode() const { return state_.sq_queue_mode != 0; }
   const detail::DeviceState &device_state() const { return state_; }
   char *arena() const { return arena_; }
+  // End (as a heap offset) of the live symmetric allocation that contains heap offset `offset`,
+  // Pow2Allocator::kNoOffset when no allocation does.
+  size_t allocation_end(size_t offset) const {
+    std::lock_guard<std::mutex> lk(alloc_mu_);
+    return alloc_.block_end(offset);
+  }
   size_t arena_bytes() const { return stride_ * static_cast<size_t>(opt_.num_pes); }
 
   // Reads and clears the sticky device status word.
@@ -135,6 +147,7 @@ class Runtime {
   size_t stride_ = 0;
   char *arena_ = nullptr;
   Pow2Allocator alloc_;
+  mutable std::mutex alloc_mu_;  // guards alloc_: entry points look allocations up while other threads allocate
   int current_pe_ = 0;
 
   char **base_heap_dev_ = nullptr;
