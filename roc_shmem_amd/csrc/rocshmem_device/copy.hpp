@@ -39,19 +39,19 @@ __device__ __forceinline__ void store_vec(u32x4 v, u32x4 *p) {
   }
 }
 
-// dst and src both 16-byte aligned.
-template <bool kNt>
+// dst and src both 16-byte aligned; kDepth loads are in flight per lane.
+template <bool kNt, int kDepth = kCopyUnroll>
 __device__ __forceinline__ void copy_vec_aligned(u32x4 *__restrict__ d,
                                                  const u32x4 *__restrict__ s, size_t nvec,
                                                  uint32_t tid, uint32_t nthr) {
   size_t i = tid;
   const size_t step = nthr;
-  for (; i + (kCopyUnroll - 1) * step < nvec; i += kCopyUnroll * step) {
-    u32x4 v[kCopyUnroll];
+  for (; i + (kDepth - 1) * step < nvec; i += kDepth * step) {
+    u32x4 v[kDepth];
 #pragma unroll
-    for (int k = 0; k < kCopyUnroll; ++k) v[k] = load_vec<kNt>(&s[i + k * step]);
+    for (int k = 0; k < kDepth; ++k) v[k] = load_vec<kNt>(&s[i + k * step]);
 #pragma unroll
-    for (int k = 0; k < kCopyUnroll; ++k) store_vec<kNt>(v[k], &d[i + k * step]);
+    for (int k = 0; k < kDepth; ++k) store_vec<kNt>(v[k], &d[i + k * step]);
   }
   for (; i < nvec; i += step) store_vec<kNt>(load_vec<kNt>(&s[i]), &d[i]);
 }
@@ -297,6 +297,96 @@ __device__ __forceinline__ W coherent_load(const void *src) {
   return __hip_atomic_load(static_cast<const W *>(src), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// One naturally aligned piece of W bytes, if `take`: load now, store later.
+template <typename W>
+struct LanePiece {
+  W bits;
+  bool take;
+  __device__ __forceinline__ void load(const char *s, bool t) {
+    take = t;
+    if (take) bits = *reinterpret_cast<const W *>(s);
+  }
+  __device__ __forceinline__ void store(char *d) const {
+    if (take) *reinterpret_cast<W *>(d) = bits;
+  }
+};
+
+// memcpy(d, s, n) by one lane for buffers that are aligned alike modulo 16
+// (n >= 32).  A lane has no neighbours to share the message with, so what
+// counts is how many memory round trips it makes: the bytes in front of the
+// first and behind the last 16-byte vector are moved as at most four
+// naturally aligned pieces each, all loaded before any is stored, and the
+// vectors go eight at a time, the last partial group included.  A 1000-byte
+// message takes 9 round trips this way, 21 when every leftover vector and
+// byte makes its own.
+__device__ __forceinline__ void lane_copy_coaligned(char *d, const char *s, size_t n) {
+  constexpr int kDepth = 2 * kCopyUnroll;
+  const uint32_t lead = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(d)) & 15u;
+  const size_t head = (16u - lead) & 15u;
+  const size_t nvec = (n - head) / 16;
+  const size_t tail = n - head - nvec * 16;
+  {
+    // Head pieces rise in size (1, 2, 4, 8 bytes bring the address to the next
+    // boundary), tail pieces fall (8, 4, 2, 1 bytes of what is left).
+    LanePiece<uint8_t> h1, t1;
+    LanePiece<uint16_t> h2, t2;
+    LanePiece<uint32_t> h4, t4;
+    LanePiece<uint64_t> h8, t8;
+    size_t o = 0;
+    h1.load(s + o, (head & 1u) != 0);
+    const size_t o1 = o;
+    o += head & 1u;
+    h2.load(s + o, (head & 2u) != 0);
+    const size_t o2 = o;
+    o += head & 2u;
+    h4.load(s + o, (head & 4u) != 0);
+    const size_t o4 = o;
+    o += head & 4u;
+    h8.load(s + o, (head & 8u) != 0);
+    const size_t o8 = o;
+    size_t q = head + nvec * 16;
+    t8.load(s + q, (tail & 8u) != 0);
+    const size_t q8 = q;
+    q += tail & 8u;
+    t4.load(s + q, (tail & 4u) != 0);
+    const size_t q4 = q;
+    q += tail & 4u;
+    t2.load(s + q, (tail & 2u) != 0);
+    const size_t q2 = q;
+    q += tail & 2u;
+    t1.load(s + q, (tail & 1u) != 0);
+    const size_t q1 = q;
+    h1.store(d + o1);
+    h2.store(d + o2);
+    h4.store(d + o4);
+    h8.store(d + o8);
+    t8.store(d + q8);
+    t4.store(d + q4);
+    t2.store(d + q2);
+    t1.store(d + q1);
+  }
+  const u32x4 *sv = reinterpret_cast<const u32x4 *>(s + head);
+  u32x4 *dv = reinterpret_cast<u32x4 *>(d + head);
+  size_t i = 0;
+  for (; i + kDepth <= nvec; i += kDepth) {
+    u32x4 v[kDepth];
+#pragma unroll
+    for (int k = 0; k < kDepth; ++k) v[k] = sv[i + k];
+#pragma unroll
+    for (int k = 0; k < kDepth; ++k) dv[i + k] = v[k];
+  }
+  const size_t left = nvec - i;
+  if (left) {
+    u32x4 v[kDepth - 1];
+#pragma unroll
+    for (int k = 0; k < kDepth - 1; ++k)
+      if (static_cast<size_t>(k) < left) v[k] = sv[i + k];
+#pragma unroll
+    for (int k = 0; k < kDepth - 1; ++k)
+      if (static_cast<size_t>(k) < left) dv[i + k] = v[k];
+  }
+}
+
 // Single-lane copy used by the thread-level put/get: the common 4- and 8-byte
 // naturally aligned messages are one coherent load and one coherent store.
 __device__ __forceinline__ void lane_copy(void *dst, const void *src, size_t n) {
@@ -305,6 +395,9 @@ __device__ __forceinline__ void lane_copy(void *dst, const void *src, size_t n) 
     coherent_store<uint64_t>(dst, coherent_load<uint64_t>(src));
   } else if (n == 4 && (both & 3u) == 0) {
     coherent_store<uint32_t>(dst, coherent_load<uint32_t>(src));
+  } else if (n >= 32 && n < kNonTemporalBytes &&
+             ((reinterpret_cast<uintptr_t>(dst) ^ reinterpret_cast<uintptr_t>(src)) & 15u) == 0) {
+    lane_copy_coaligned(static_cast<char *>(dst), static_cast<const char *>(src), n);
   } else {
     group_copy(dst, src, n, 0u, 1u);
   }

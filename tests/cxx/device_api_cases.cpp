@@ -810,11 +810,11 @@ static void primitive_mr() {
     for (int pe = 0; pe < npes; ++pe)
       if (pe != 1)
         for (char c : load(r_buf, max_size, pe)) EXPECT(c == '1', "size %d: PE %d was written", size, pe);
+    uint64_t ticks[wgs];
+    EXPECT(hipMemcpy(ticks, timer, sizeof(ticks), hipMemcpyDeviceToHost) == hipSuccess, "timer copy");
+    printf("  putmem_nbi(%d B), quiet after every 64: %.0f ns per message issued by one lane\n", size,
+           ticks[0] * 10.0 / (64 * 2 * 64));
   }
-  uint64_t ticks[wgs];
-  EXPECT(hipMemcpy(ticks, timer, sizeof(ticks), hipMemcpyDeviceToHost) == hipSuccess, "timer copy");
-  printf("  putmem_nbi(1000 B) + quiet per 64: %.0f ns per message in one lane\n",
-         ticks[0] * 10.0 / (64 * 2 * 64));
   roc_shmem_free(r_buf);
   roc_shmem_free(s_buf);
   EXPECT(hipFree(timer) == hipSuccess, "hipFree");
