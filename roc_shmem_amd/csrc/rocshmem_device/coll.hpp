@@ -38,7 +38,7 @@ __device__ __forceinline__ void split_range(size_t n, int parts, int idx, size_t
 
 // Copy `n` bytes from `src` into the same symmetric address `dst_mine` of
 // every member for which `skip_idx != member index`.  When source and
-// destinations are mutually 16-byte aligned every source vector is loaded
+// destinations are aligned alike modulo 4 every source vector is loaded
 // once and stored to each destination (raw-buffer addressing as in
 // stream_copy_uniform); otherwise each destination is copied on its own.
 // Arguments are workgroup-uniform.
@@ -56,8 +56,9 @@ __device__ __forceinline__ void wg_copy_to_members(char *dst_mine, const char *s
   const int64_t stride = static_cast<int64_t>(g_state.slice_stride);
   char *dst0 = dst_mine + (static_cast<int64_t>(as.pe_start) - my_pe) * stride;
   const int64_t member_step = stride << as.log_stride;
+  // The vector path stores 16-byte aligned and loads at any 4-byte alignment.
   const bool coaligned =
-      ((reinterpret_cast<uintptr_t>(dst_mine) ^ reinterpret_cast<uintptr_t>(src)) & 15u) == 0;
+      ((reinterpret_cast<uintptr_t>(dst_mine) ^ reinterpret_cast<uintptr_t>(src)) & 3u) == 0;
   if (!coaligned || n < 256) {
     for (int m = 0; m < as.size; ++m) {
       if (m == skip_idx) continue;
@@ -65,7 +66,7 @@ __device__ __forceinline__ void wg_copy_to_members(char *dst_mine, const char *s
     }
     return;
   }
-  const size_t head = (16u - (reinterpret_cast<uintptr_t>(src) & 15u)) & 15u;
+  const size_t head = stream_head(dst_mine, n);
   const size_t body = (n - head) & ~static_cast<size_t>(15);
   const size_t tail = n - head - body;
   for (size_t t = tid; edges && t < head + tail; t += nthr) {
@@ -148,7 +149,7 @@ __device__ __forceinline__ void wg_broadcast_bytes(int my_pe, void *dest, const 
   const char *root_src = translate(static_cast<const char *>(source), my_pe, as.pe_at(root_idx));
   const size_t pass_bytes = static_cast<size_t>(nthr) * 16u * kStreamUnroll;
   const bool coaligned =
-      ((reinterpret_cast<uintptr_t>(dest) ^ reinterpret_cast<uintptr_t>(root_src)) & 15u) == 0;
+      ((reinterpret_cast<uintptr_t>(dest) ^ reinterpret_cast<uintptr_t>(root_src)) & 3u) == 0;
   if (coaligned && nbytes >= 2 * parts * pass_bytes) {
     wg_copy_to_members(static_cast<char *>(dest), root_src, nbytes, as, my_pe, root_idx, tid, nthr,
                        part, parts, part == 0);

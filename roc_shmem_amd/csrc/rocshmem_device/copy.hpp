@@ -202,6 +202,22 @@ __device__ __forceinline__ void stream_copy_sized(char *d, const char *s, size_t
   }
 }
 
+// Bytes in front of the vector body of a copy of `n` bytes to `d`: up to the
+// next 16-byte boundary, for a message of some size up to the next 128-byte
+// boundary (every wave store then covers whole cache lines) and for a large
+// one up to the next 1 KiB boundary (the 1 KiB that the 64 lanes of a wave
+// store with one instruction then never straddles two).  Measured on MI355X,
+// 8 x 192 MiB put as 64 MiB messages: 4.98 TB/s with the body starting 16
+// bytes past a 128-byte boundary, 5.94 at a 128-byte boundary that is not a
+// 1 KiB boundary, 6.1 at a 1 KiB boundary; a 1 -> 7 broadcast of 64 MiB takes
+// 146 us from a 128-byte and 138 us from a 1 KiB boundary.
+constexpr size_t kStoreChunkBytes = 1024;
+__device__ __forceinline__ size_t stream_head(const char *d, size_t n) {
+  const uintptr_t at = reinterpret_cast<uintptr_t>(d);
+  const uintptr_t boundary = n >= 65536 ? kStoreChunkBytes : n >= 4096 ? 128u : 16u;
+  return (boundary - (at & (boundary - 1))) & (boundary - 1);
+}
+
 // memcpy(dst, src, n) by lanes tid = 0..nthr-1 of a group that passes the
 // same (dst, src, n) in every lane.
 __device__ __forceinline__ void group_copy_uniform(void *dst, const void *src, size_t n,
@@ -212,7 +228,7 @@ __device__ __forceinline__ void group_copy_uniform(void *dst, const void *src, s
     for (size_t i = tid; i < n; i += nthr) d[i] = s[i];
     return;
   }
-  const size_t head = (16u - (reinterpret_cast<uintptr_t>(d) & 15u)) & 15u;
+  const size_t head = stream_head(d, n);
   for (size_t i = tid; i < head; i += nthr) d[i] = s[i];
   d += head;
   s += head;
@@ -241,10 +257,11 @@ __device__ __forceinline__ void group_copy_dealt(void *dst, const void *src, siz
   char *d = static_cast<char *>(dst);
   const char *s = static_cast<const char *>(src);
   const size_t pass_bytes = static_cast<size_t>(nthr) * 16u * kStreamUnroll;
+  // The vector path stores 16-byte aligned and loads at any 4-byte alignment.
   const bool coaligned =
-      ((reinterpret_cast<uintptr_t>(d) ^ reinterpret_cast<uintptr_t>(s)) & 15u) == 0;
+      ((reinterpret_cast<uintptr_t>(d) ^ reinterpret_cast<uintptr_t>(s)) & 3u) == 0;
   if (coaligned && n >= 2 * parts * pass_bytes) {
-    const size_t head = (16u - (reinterpret_cast<uintptr_t>(d) & 15u)) & 15u;
+    const size_t head = stream_head(d, n);
     const size_t body = (n - head) & ~static_cast<size_t>(15);
     if (part == 0) {
       for (size_t i = tid; i < head; i += nthr) d[i] = s[i];
