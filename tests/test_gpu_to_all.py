@@ -114,11 +114,45 @@ def test_zero_elements_is_a_no_op():
 
 
 @pytest.mark.parametrize("shift", [1, 3])
-def test_unaligned_arrays_take_the_element_path(shift):
+def test_arrays_shifted_alike_off_the_vector_boundary(shift):
     with runtime(4):
         got, expect, _ = run_case(rs.INT, rs.XOR, 4, 1000, seed=77, elem_shift=shift)
         for p in range(4):
             assert np.array_equal(got[p], expect[p])  # includes the untouched leading guard
+
+
+@pytest.mark.parametrize("dtype,dst_shift,src_shift", [
+    (rs.INT, 1, 2), (rs.INT, 0, 3), (rs.LONG, 1, 0), (rs.LONGLONG, 3, 6),
+    (rs.SHORT, 2, 4),      # two-byte elements an even number apart: vector path
+    (rs.SHORT, 1, 2),      # an odd number apart: element by element
+    (rs.SHORT, 5, 0)])
+@pytest.mark.parametrize("n,wgs", [(37, 1), (3000, 2), (70001, 3)])
+def test_source_and_destination_shifted_differently(dtype, dst_shift, src_shift, n, wgs):
+    # sizes below 4 KiB, below 64 KiB and above: the vector body starts at the destination's next
+    # 16-byte, 128-byte and 1 KiB boundary; bytes around the destination stay as they were
+    n_pes = 4
+    npd = rs.NP_DTYPE[dtype]
+    es = np.dtype(npd).itemsize
+    total = n + 16
+    with runtime(n_pes):
+        src = rs.sym_array(total, npd)
+        dst = rs.sym_array(total, npd)
+        psync = rs.sym_array(wgs * rs.ROC_SHMEM_REDUCE_SYNC_SIZE, np.int64, fill=0)
+        heap = oracle.Heap(n_pes, 2 * total * es + 64)
+        for p in range(n_pes):
+            vals = random_values(dtype, total, 900 + p)
+            src.write(p, vals)
+            heap.view(p, 0, total, npd)[:] = vals
+            guard = np.full(total, 0x3C, np.uint8).repeat(es).view(npd)[:total]
+            dst.write(p, guard)
+            heap.view(p, total * es, total, npd)[:] = guard
+        rs.roc_shmem_to_all(dtype, rs.SUM, dst.addr + dst_shift * es, src.addr + src_shift * es, n, 0, 0,
+                            n_pes, None, psync, rs.Launch(wgs, 256))
+        rs.synchronize()
+        oracle.to_all(heap, dtype, rs.SUM, (total + dst_shift) * es, src_shift * es, n)
+        for p in range(n_pes):
+            assert np.array_equal(dst.read(p), heap.view(p, total * es, total, npd)), "PE %d" % p
+            assert not psync.read(p).any()
 
 
 def test_in_place():
