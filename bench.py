@@ -366,6 +366,44 @@ def bench_bcast_a2a(rs, n_pes, slice_bytes):
     return res
 
 
+def bench_alignment(rs, n_pes):
+    """Large put, broadcast and reduction with source and destination shifted off their natural
+    alignment: (source shift, destination shift) in bytes -> GB/s."""
+    out = {"put_64MiB_messages": {}, "broadcast_64MiB": {}, "float_sum_to_all_2^26": {}}
+    src = rs.sym_array(256 << 20, np.uint8, fill=1)
+    dst = rs.sym_array(256 << 20, np.uint8, fill=0)
+    world = rs.roc_shmem_team_world()
+    psync = rs.sym_array(TO_ALL_LAUNCH["wgs_per_pe"] * rs.ROC_SHMEM_REDUCE_SYNC_SIZE, np.int64, fill=0)
+    total, msg, n = 192 << 20, 64 << 20, (1 << 26) - 1024
+    for ss, ds in ((0, 0), (16, 16), (128, 128), (256, 256), (1024, 1024), (4, 4), (4, 8), (16, 32), (1, 0)):
+        key = "%d/%d" % (ss, ds)
+
+        def put():
+            rs.roc_shmem_rma(rs.PUT, rs.WG_SHARED, dst.addr + ds, src.addr + ss, msg, total // msg, msg, msg, 1,
+                             rs.Launch(**PUT_LAUNCH))
+
+        def bcast():
+            rs.roc_shmem_team_broadcast(1, world, dst.addr + ds, src.addr + ss, msg, 0, rs.Launch(8, 1024))
+
+        def reduce():
+            rs.roc_shmem_to_all(rs.FLOAT, rs.SUM, dst.addr + ds, src.addr + ss, n, 0, 0, n_pes, None, psync,
+                                rs.Launch(**TO_ALL_LAUNCH))
+
+        for name, fn, nbytes in (("put_64MiB_messages", put, 2.0 * n_pes * total),
+                                 ("broadcast_64MiB", bcast, float(n_pes) * msg),
+                                 ("float_sum_to_all_2^26", reduce, 2.0 * n_pes * n * 4)):
+            if name.startswith("float") and (ss % 4 or ds % 4):
+                continue
+            fn()
+            rs.synchronize()
+            out[name][key] = round(nbytes / (event_time_ms(rs, fn, 5) / 5) / 1e6, 1)
+    if rs.take_status():
+        raise RuntimeError("device status word raised")
+    for a in (psync, dst, src):
+        a.free()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -377,6 +415,8 @@ def main():
                          "plain wg putmem copy of known size (2 GiB read + 2 GiB written), nothing else")
     ap.add_argument("--small-ops", action="store_true",
                     help="for rocprofv3 --pmc: the 10 M-operation streams and the consumer pass, nothing else")
+    ap.add_argument("--alignment", action="store_true",
+                    help="large put / broadcast / reduction with shifted source and destination, nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: every PE slice lives in one GPU's HBM; this build measures one GPU only "
@@ -391,6 +431,12 @@ def main():
         out = bench_small_ops(rs, 16, 10_000_000, 1024, 256, 64 << 20, seed=4)
         rs.roc_shmem_finalize()
         print(json.dumps({"small_ops_16x64MiB_1024wg_x256": out}))
+        return
+    if args.alignment:
+        rs.roc_shmem_init(8, 1 << 30, 64, 1024)
+        out = bench_alignment(rs, 8)
+        rs.roc_shmem_finalize()
+        print(json.dumps({"GBps_by_source_shift/destination_shift_8pe": out}))
         return
     device = device_report() if not args.counter_pair else {}
     ceilings = hbm_ceilings() if not (args.counter_pair or args.quick) else {}
