@@ -85,6 +85,13 @@ typedef struct rsm_small_op {
   int64_t aux;
 } rsm_small_op_t;
 
+/* Host threads.  Entry points may be called from any host thread; the library
+ * runs one of them at a time (one recursive lock around the whole interface).
+ * Kernels they launch on different streams still run concurrently on the
+ * device; two launches that use the same contexts (the same (PE, workgroup
+ * index) pairs) at the same time share send queues and pSync slices and must
+ * not overlap. */
+
 /* Argument checks of the data-path entry points.  A symmetric operand must lie
  * inside a live allocation of rsm_malloc and the bytes the call touches
  * (elements x element size, team size x block, messages x stride, wgs_per_pe

@@ -48,6 +48,11 @@ bool resolve_launch(const rsm_launch_t *in, Launch *out) {
   return true;
 }
 
+std::recursive_mutex &abi_lock() {
+  static std::recursive_mutex mu;
+  return mu;
+}
+
 bool check_symmetric(const void *p, const char *what, bool allow_null) {
   using rocshmem::host::Runtime;
   Runtime *rt = Runtime::get();
@@ -110,6 +115,7 @@ namespace detail = rocshmem::detail;
 extern "C" {
 
 int rsm_init(int num_pes, size_t heap_bytes_per_pe, int num_blocks, unsigned sq_size) {
+  RSM_ENTRY;
   rsm::clear_error();
   Options o = Options::from_env();
   if (num_pes) o.num_pes = num_pes;
@@ -124,6 +130,7 @@ int rsm_init(int num_pes, size_t heap_bytes_per_pe, int num_blocks, unsigned sq_
 }
 
 int rsm_finalize(void) {
+  RSM_ENTRY;
   Runtime::destroy();
   rocshmem::ROC_SHMEM_TEAM_WORLD = nullptr;
   return 0;
@@ -132,6 +139,7 @@ int rsm_finalize(void) {
 int rsm_is_initialized(void) { return Runtime::get() ? 1 : 0; }
 
 const char *rsm_last_error(void) {
+  RSM_ENTRY;
   static thread_local std::string copy;
   std::lock_guard<std::mutex> lk(rsm::g_error_mu);
   copy = rsm::g_error;
@@ -144,6 +152,7 @@ size_t rsm_heap_size(void) { return Runtime::get() ? Runtime::get()->options().h
 size_t rsm_slice_stride(void) { return Runtime::get() ? Runtime::get()->slice_stride() : 0; }
 
 void *rsm_malloc(size_t bytes) {
+  RSM_ENTRY;
   Runtime *rt = Runtime::get();
   if (!rt) {
     rsm::fail("rsm_init has not been called");
@@ -158,6 +167,7 @@ void *rsm_malloc(size_t bytes) {
 }
 
 int rsm_free(void *ptr) {
+  RSM_ENTRY;
   RSM_NEED_RT(rt);
   (void)hipDeviceSynchronize();
   return rt->sym_free(ptr) ? 0 : rsm::fail("rsm_free: not an outstanding symmetric allocation");
@@ -166,11 +176,13 @@ int rsm_free(void *ptr) {
 size_t rsm_heap_bytes_in_use(void) { return Runtime::get() ? Runtime::get()->bytes_in_use() : 0; }
 
 void *rsm_ptr(const void *sym, int pe) {
+  RSM_ENTRY;
   Runtime *rt = Runtime::get();
   return rt ? rt->translate(sym, pe) : nullptr;
 }
 
 void *rsm_heap_base(int pe) {
+  RSM_ENTRY;
   Runtime *rt = Runtime::get();
   if (!rt || pe < 0 || pe >= rt->num_pes()) return nullptr;
   return rt->slice_base(pe);
@@ -179,16 +191,19 @@ void *rsm_heap_base(int pe) {
 int rsm_state_units(void) { return rocshmem::host::registered_state_units(); }
 
 int rsm_take_status(void) {
+  RSM_ENTRY;
   RSM_NEED_RT(rt);
   return static_cast<int>(rt->take_status());
 }
 
 uint64_t rsm_team_world(void) {
+  RSM_ENTRY;
   Runtime *rt = Runtime::get();
   return rt ? reinterpret_cast<uint64_t>(rt->team_world()) : 0;
 }
 
 int rsm_team_split_strided(uint64_t parent, int start, int stride, int size, uint64_t *new_team) {
+  RSM_ENTRY;
   RSM_NEED_RT(rt);
   if (!new_team) return rsm::fail("new_team is NULL");
   detail::Team *out = nullptr;
@@ -199,6 +214,7 @@ int rsm_team_split_strided(uint64_t parent, int start, int stride, int size, uin
 }
 
 int rsm_team_destroy(uint64_t team) {
+  RSM_ENTRY;
   RSM_NEED_RT(rt);
   (void)hipDeviceSynchronize();
   rt->team_destroy(reinterpret_cast<detail::Team *>(team));
@@ -206,10 +222,12 @@ int rsm_team_destroy(uint64_t team) {
 }
 
 int rsm_team_n_pes(uint64_t team) {
+  RSM_ENTRY;
   return rocshmem::roc_shmem_team_n_pes(reinterpret_cast<rocshmem::roc_shmem_team_t>(team));
 }
 
 int rsm_team_translate_pe(uint64_t src_team, int src_pe, uint64_t dst_team) {
+  RSM_ENTRY;
   if (!Runtime::get()) return -1;
   return rocshmem::roc_shmem_team_translate_pe(
       reinterpret_cast<rocshmem::roc_shmem_team_t>(src_team), src_pe,
@@ -217,22 +235,27 @@ int rsm_team_translate_pe(uint64_t src_team, int src_pe, uint64_t dst_team) {
 }
 
 int rsm_copy_to_device(void *dst, const void *host_src, size_t bytes) {
+  RSM_ENTRY;
   RSM_HIP(hipMemcpy(dst, host_src, bytes, hipMemcpyHostToDevice));
   return 0;
 }
 int rsm_copy_to_host(void *host_dst, const void *src, size_t bytes) {
+  RSM_ENTRY;
   RSM_HIP(hipMemcpy(host_dst, src, bytes, hipMemcpyDeviceToHost));
   return 0;
 }
 int rsm_fill(void *dst, int byte_value, size_t bytes) {
+  RSM_ENTRY;
   RSM_HIP(hipMemset(dst, byte_value, bytes));
   return 0;
 }
 int rsm_synchronize(void) {
+  RSM_ENTRY;
   RSM_HIP(hipDeviceSynchronize());
   return 0;
 }
 void *rsm_device_alloc(size_t bytes) {
+  RSM_ENTRY;
   void *p = nullptr;
   if (hipMalloc(&p, bytes) != hipSuccess) {
     rsm::fail("hipMalloc failed");
@@ -241,10 +264,12 @@ void *rsm_device_alloc(size_t bytes) {
   return p;
 }
 int rsm_device_free(void *ptr) {
+  RSM_ENTRY;
   RSM_HIP(hipFree(ptr));
   return 0;
 }
 void *rsm_stream_create(void) {
+  RSM_ENTRY;
   hipStream_t s = nullptr;
   if (hipStreamCreate(&s) != hipSuccess) {
     rsm::fail("hipStreamCreate failed");
@@ -253,10 +278,12 @@ void *rsm_stream_create(void) {
   return s;
 }
 int rsm_stream_destroy(void *stream) {
+  RSM_ENTRY;
   RSM_HIP(hipStreamDestroy(static_cast<hipStream_t>(stream)));
   return 0;
 }
 void *rsm_event_create(void) {
+  RSM_ENTRY;
   hipEvent_t e = nullptr;
   if (hipEventCreate(&e) != hipSuccess) {
     rsm::fail("hipEventCreate failed");
@@ -265,14 +292,17 @@ void *rsm_event_create(void) {
   return e;
 }
 int rsm_event_destroy(void *event) {
+  RSM_ENTRY;
   RSM_HIP(hipEventDestroy(static_cast<hipEvent_t>(event)));
   return 0;
 }
 int rsm_event_record(void *event, void *stream) {
+  RSM_ENTRY;
   RSM_HIP(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
   return 0;
 }
 int rsm_event_elapsed_ms(void *start, void *stop, float *ms) {
+  RSM_ENTRY;
   RSM_HIP(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
   RSM_HIP(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
   return 0;
@@ -283,12 +313,14 @@ int rsm_event_elapsed_ms(void *start, void *stop, float *ms) {
 // them can be recorded once and replayed as one submission.
 
 int rsm_capture_begin(void *stream) {
+  RSM_ENTRY;
   if (!stream) return rsm::fail("rsm_capture_begin: capture needs a stream of its own, not the default stream");
   RSM_HIP(hipStreamBeginCapture(static_cast<hipStream_t>(stream), hipStreamCaptureModeThreadLocal));
   return 0;
 }
 
 void *rsm_capture_end(void *stream) {
+  RSM_ENTRY;
   hipGraph_t graph = nullptr;
   hipError_t e = hipStreamEndCapture(static_cast<hipStream_t>(stream), &graph);
   if (e != hipSuccess || !graph) {
@@ -306,11 +338,13 @@ void *rsm_capture_end(void *stream) {
 }
 
 int rsm_graph_launch(void *graph, void *stream) {
+  RSM_ENTRY;
   RSM_HIP(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), static_cast<hipStream_t>(stream)));
   return 0;
 }
 
 int rsm_graph_destroy(void *graph) {
+  RSM_ENTRY;
   RSM_HIP(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)));
   return 0;
 }
@@ -322,6 +356,7 @@ static bool sq_args_ok(Runtime *rt, int pe, int block) {
 }
 
 int rsm_sq_reset(void) {
+  RSM_ENTRY;
   RSM_NEED_RT(rt);
   RSM_HIP(hipDeviceSynchronize());
   rt->reset_queues(nullptr);
@@ -330,6 +365,7 @@ int rsm_sq_reset(void) {
 }
 
 int rsm_sq_read(int pe, int block, unsigned index, uint64_t out_words[8]) {
+  RSM_ENTRY;
   RSM_NEED_RT(rt);
   if (!sq_args_ok(rt, pe, block) || index >= rt->options().sq_size)
     return rsm::fail("rsm_sq_read: arguments out of range");
@@ -340,6 +376,7 @@ int rsm_sq_read(int pe, int block, unsigned index, uint64_t out_words[8]) {
 }
 
 int rsm_sq_image(int pe, int block, void *host_out, size_t bytes) {
+  RSM_ENTRY;
   RSM_NEED_RT(rt);
   if (!sq_args_ok(rt, pe, block) || bytes > 64ull * rt->options().sq_size)
     return rsm::fail("rsm_sq_image: arguments out of range");
@@ -350,6 +387,7 @@ int rsm_sq_image(int pe, int block, void *host_out, size_t bytes) {
 
 int rsm_sq_state(int pe, int block, uint32_t *sq_counter, uint32_t *published,
                  uint32_t *atomic_counter, uint64_t mailbox[2]) {
+  RSM_ENTRY;
   RSM_NEED_RT(rt);
   if (!sq_args_ok(rt, pe, block)) return rsm::fail("rsm_sq_state: arguments out of range");
   RSM_HIP(hipDeviceSynchronize());
@@ -365,6 +403,7 @@ int rsm_sq_state(int pe, int block, uint32_t *sq_counter, uint32_t *published,
 
 int rsm_sq_constants(int pe, int block, uint32_t *ctrl_qp_sq, uint64_t *ctrl_sig, uint32_t *lkey,
                      uint32_t *atomic_lkey, uint64_t *atomic_ret_base, uint32_t *max_nwqe) {
+  RSM_ENTRY;
   RSM_NEED_RT(rt);
   if (!sq_args_ok(rt, pe, block)) return rsm::fail("rsm_sq_constants: arguments out of range");
   const detail::SqRing &r = rt->ctx_image(pe, block).ring;
@@ -378,6 +417,7 @@ int rsm_sq_constants(int pe, int block, uint32_t *ctrl_qp_sq, uint64_t *ctrl_sig
 }
 
 int rsm_sq_rkey(int dest_pe, uint32_t *rkey) {
+  RSM_ENTRY;
   RSM_NEED_RT(rt);
   if (dest_pe < 0 || dest_pe >= rt->num_pes() || !rkey)
     return rsm::fail("rsm_sq_rkey: arguments out of range");
@@ -388,18 +428,23 @@ int rsm_sq_rkey(int dest_pe, uint32_t *rkey) {
 // ---- host-logic hooks ------------------------------------------------------------
 
 void *rsm_host_alloc_create(size_t heap_bytes) {
+  RSM_ENTRY;
   return new rocshmem::host::Pow2Allocator(heap_bytes);
 }
 void rsm_host_alloc_destroy(void *allocator) {
+  RSM_ENTRY;
   delete static_cast<rocshmem::host::Pow2Allocator *>(allocator);
 }
 size_t rsm_host_alloc_alloc(void *allocator, size_t request) {
+  RSM_ENTRY;
   return static_cast<rocshmem::host::Pow2Allocator *>(allocator)->alloc(request);
 }
 int rsm_host_alloc_free(void *allocator, size_t offset) {
+  RSM_ENTRY;
   return static_cast<rocshmem::host::Pow2Allocator *>(allocator)->free(offset) ? 0 : -1;
 }
 size_t rsm_host_alloc_in_use(void *allocator) {
+  RSM_ENTRY;
   return static_cast<rocshmem::host::Pow2Allocator *>(allocator)->bytes_in_use();
 }
 

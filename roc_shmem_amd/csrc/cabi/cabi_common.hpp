@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <mutex>
 #include <string>
 
 #include "host/runtime.hpp"
@@ -26,6 +27,12 @@ struct Launch {
 bool resolve_launch(const rsm_launch_t *in, Launch *out);
 
 // True when `p` is a symmetric address in PE 0's slice (or NULL when allowed).
+// One lock for the whole C ABI: entry points may be called from any host thread, one runs at a
+// time (they share the allocator, the team table and the last-error text).  Recursive because
+// entry points call each other.
+std::recursive_mutex &abi_lock();
+#define RSM_ENTRY std::lock_guard<std::recursive_mutex> rsm_entry_guard_(rsm::abi_lock())
+
 bool check_symmetric(const void *p, const char *what, bool allow_null = false);
 // `bytes` starting at the symmetric address `p` stay inside the live symmetric allocation that
 // contains `p` (a kernel that ran past it would overwrite its neighbours or fault the device);

@@ -223,6 +223,7 @@ extern "C" {
 int rsm_broadcast(size_t elem_size, void *dest, const void *source, size_t nelem, int pe_root,
                   int pe_start, int log_pe_stride, int pe_size, long *pSync,
                   const rsm_launch_t *launch) {
+  RSM_ENTRY;
   rsm::Launch l;
   if (!rsm::resolve_launch(launch, &l)) return -1;
   host::Runtime *rt = host::Runtime::get();
@@ -241,6 +242,7 @@ int rsm_broadcast(size_t elem_size, void *dest, const void *source, size_t nelem
 
 int rsm_broadcast_team(size_t elem_size, uint64_t team, void *dest, const void *source,
                        size_t nelem, int pe_root, const rsm_launch_t *launch) {
+  RSM_ENTRY;
   rsm::Launch l;
   if (!rsm::resolve_launch(launch, &l)) return -1;
   host::Runtime *rt = host::Runtime::get();
@@ -258,15 +260,18 @@ int rsm_broadcast_team(size_t elem_size, uint64_t team, void *dest, const void *
 
 int rsm_alltoall(size_t elem_size, uint64_t team, void *dest, const void *source, size_t nelem,
                  const rsm_launch_t *launch) {
+  RSM_ENTRY;
   return run_exchange<false>(elem_size, team, dest, source, nelem, launch);
 }
 
 int rsm_fcollect(size_t elem_size, uint64_t team, void *dest, const void *source, size_t nelem,
                  const rsm_launch_t *launch) {
+  RSM_ENTRY;
   return run_exchange<true>(elem_size, team, dest, source, nelem, launch);
 }
 
 int rsm_barrier_all(int iterations, const rsm_launch_t *launch) {
+  RSM_ENTRY;
   rsm::Launch l;
   if (!rsm::resolve_launch(launch, &l)) return -1;
   if (l.wgs_per_pe > host::Runtime::get()->options().num_blocks)

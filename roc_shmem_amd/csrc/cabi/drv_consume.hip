@@ -35,6 +35,7 @@ bool ring_args_ok(Runtime *rt, int pe, int block) {
 extern "C" {
 
 int rsm_sq_consume(int pe, int block, void *target_arena, rsm_consume_totals_t *totals) {
+  RSM_ENTRY;
   Runtime *rt = Runtime::get();
   if (!rt) return rsm::fail("rsm_init has not been called");
   if ((pe != -1 && (pe < 0 || pe >= rt->num_pes())) ||
@@ -56,6 +57,7 @@ int rsm_sq_consume(int pe, int block, void *target_arena, rsm_consume_totals_t *
 }
 
 int rsm_sq_set_mode(int queue_mode) {
+  RSM_ENTRY;
   Runtime *rt = Runtime::get();
   if (!rt) return rsm::fail("rsm_init has not been called");
   if (!rt->set_sq_queue_mode(queue_mode != 0))
@@ -64,6 +66,7 @@ int rsm_sq_set_mode(int queue_mode) {
 }
 
 int rsm_sq_consumer_state(int pe, int block, uint32_t *consumed, uint32_t *cq_producer) {
+  RSM_ENTRY;
   Runtime *rt = Runtime::get();
   if (!rt) return rsm::fail("rsm_init has not been called");
   if (!ring_args_ok(rt, pe, block)) return rsm::fail("rsm_sq_consumer_state: arguments out of range");
@@ -76,6 +79,7 @@ int rsm_sq_consumer_state(int pe, int block, uint32_t *consumed, uint32_t *cq_pr
 }
 
 int rsm_cq_image(int pe, int block, void *host_out, size_t bytes) {
+  RSM_ENTRY;
   Runtime *rt = Runtime::get();
   if (!rt) return rsm::fail("rsm_init has not been called");
   if (!ring_args_ok(rt, pe, block) || bytes > 64ull * rt->options().sq_size)
@@ -86,6 +90,7 @@ int rsm_cq_image(int pe, int block, void *host_out, size_t bytes) {
 }
 
 int rsm_atomic_ret_image(int pe, int block, void *host_out, size_t bytes) {
+  RSM_ENTRY;
   Runtime *rt = Runtime::get();
   if (!rt) return rsm::fail("rsm_init has not been called");
   if (!ring_args_ok(rt, pe, block) || bytes > 8ull * detail::kAtomicRetSlots)
@@ -98,6 +103,7 @@ int rsm_atomic_ret_image(int pe, int block, void *host_out, size_t bytes) {
 }
 
 int rsm_arena(void **base, size_t *bytes, size_t *slice_stride) {
+  RSM_ENTRY;
   Runtime *rt = Runtime::get();
   if (!rt) return rsm::fail("rsm_init has not been called");
   if (base) *base = rt->arena();

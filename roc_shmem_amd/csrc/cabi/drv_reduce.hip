@@ -237,6 +237,7 @@ extern "C" {
 int rsm_to_all(int dtype, int op, void *dest, const void *source, size_t nreduce, int pe_start,
                int log_pe_stride, int pe_size, void *pWrk, long *pSync,
                const rsm_launch_t *launch) {
+  RSM_ENTRY;
   rsm::Launch l;
   if (!rsm::resolve_launch(launch, &l)) return -1;
   host::Runtime *rt = host::Runtime::get();
@@ -254,6 +255,7 @@ int rsm_to_all(int dtype, int op, void *dest, const void *source, size_t nreduce
 
 int rsm_to_all_team(int dtype, int op, uint64_t team, void *dest, const void *source,
                     size_t nreduce, const rsm_launch_t *launch) {
+  RSM_ENTRY;
   rsm::Launch l;
   if (!rsm::resolve_launch(launch, &l)) return -1;
   host::Runtime *rt = host::Runtime::get();

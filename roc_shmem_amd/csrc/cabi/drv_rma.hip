@@ -84,6 +84,7 @@ __global__ void __launch_bounds__(1024)
 extern "C" int rsm_rma(int kind, int granularity, void *dest, const void *source,
                        size_t msg_bytes, size_t n_msgs, size_t dst_stride, size_t src_stride,
                        int pe_shift, const rsm_launch_t *launch) {
+  RSM_ENTRY;
   rsm::Launch l;
   if (!rsm::resolve_launch(launch, &l)) return -1;
   if (kind < RSM_PUT || kind > RSM_GET_NBI) return rsm::fail("rma: unknown kind");

@@ -146,6 +146,7 @@ extern "C" {
 
 int rsm_small_ops(const rsm_small_op_t *ops, size_t n_ops, int64_t *fetched,
                   const rsm_launch_t *launch) {
+  RSM_ENTRY;
   rsm::Launch l;
   if (!rsm::resolve_launch(launch, &l)) return -1;
   if (!ops) return rsm::fail("small_ops: ops is NULL");
@@ -157,6 +158,7 @@ int rsm_small_ops(const rsm_small_op_t *ops, size_t n_ops, int64_t *fetched,
 
 int rsm_kat_fetch_incr(uint64_t lane_mask, int n_wgs, int wg_size, uint64_t *per_thread,
                        uint64_t *counter_out) {
+  RSM_ENTRY;
   if (n_wgs < 1 || wg_size < 64 || wg_size > 1024 || wg_size % 64)
     return rsm::fail("kat_fetch_incr: bad grid");
   const size_t n = static_cast<size_t>(n_wgs) * wg_size;
@@ -181,6 +183,7 @@ int rsm_kat_fetch_incr(uint64_t lane_mask, int n_wgs, int wg_size, uint64_t *per
 int rsm_kat_coalesce(uint64_t lane_mask, const int32_t *pe, const uint64_t *src,
                      const uint64_t *dst, const uint64_t *size, uint8_t *must_send,
                      uint64_t *out_size) {
+  RSM_ENTRY;
   char *buf = nullptr;
   const size_t bytes = 64 * (4 + 8 + 8 + 8 + 1 + 8) + 64;
   RSM_HIP(hipMalloc(reinterpret_cast<void **>(&buf), bytes));

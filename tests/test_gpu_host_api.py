@@ -75,3 +75,53 @@ def test_reference_functional_testers_restated():
     print(out.stdout[-1500:], flush=True)
     assert out.returncode == 0, tail
     assert "DEVICE_API_OK" in out.stdout, tail
+
+
+@pytest.mark.gpu
+def test_entry_points_called_from_several_host_threads():
+    """The C ABI serialises its entry points: threads that allocate, launch, read back and free at
+    the same time each get their own correct result (ctypes drops the interpreter lock during
+    the calls, so they do overlap)."""
+    import threading
+
+    import numpy as np
+
+    import roc_shmem_amd as rs
+
+    n_pes, n, rounds = 4, 2000, 25
+    rs.roc_shmem_init(n_pes, 64 << 20, 8, 1024)
+    in_use_at_start = rs.heap_bytes_in_use()
+    errors = []
+
+    def worker(tid):
+        try:
+            rng = np.random.default_rng(tid)
+            for r in range(rounds):
+                src = rs.sym_array(n, np.int64)
+                dst = rs.sym_array(n, np.int64, fill=0)
+                psync = rs.sym_array(rs.ROC_SHMEM_REDUCE_SYNC_SIZE, np.int64, fill=0)
+                host = [rng.integers(-1000, 1000, n, dtype=np.int64) + tid for _ in range(n_pes)]
+                for p in range(n_pes):
+                    src.write(p, host[p])
+                rs.roc_shmem_to_all(rs.LONG, rs.SUM, dst, src, n, 0, 0, n_pes, None, psync)
+                rs.synchronize()
+                want = np.sum(np.stack(host), axis=0, dtype=np.int64)
+                for p in range(n_pes):
+                    if not np.array_equal(dst.read(p), want):
+                        errors.append("thread %d round %d PE %d" % (tid, r, p))
+                for a in (psync, dst, src):
+                    a.free()
+        except Exception as e:  # noqa: BLE001 - reported by the main thread
+            errors.append("thread %d: %r" % (tid, e))
+
+    try:
+        threads = [threading.Thread(target=worker, args=(t,)) for t in range(6)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        assert not errors, errors[:5]
+        assert rs.take_status() == 0
+        assert rs.heap_bytes_in_use() == in_use_at_start
+    finally:
+        rs.roc_shmem_finalize()
