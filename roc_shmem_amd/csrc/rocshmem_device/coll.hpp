@@ -36,11 +36,62 @@ __device__ __forceinline__ void split_range(size_t n, int parts, int idx, size_t
   if (end > n) end = n;
 }
 
+// Vector body of wg_copy_to_members: passes first_pass, first_pass +
+// pass_step, ... of `body` bytes (a multiple of 16) from `src` to the `ndst`
+// destinations dst0 + m * member_step, m counting past `skip_at`.  `dst0` is
+// 16-byte aligned.  kBufferLoads: `src` is 4-byte aligned and read through a
+// buffer descriptor; otherwise it is read with per-lane unaligned vector loads.
+template <bool kBufferLoads>
+__device__ __forceinline__ void copy_passes_to_members(char *dst0, const char *src, size_t body,
+                                                       int64_t member_step, int ndst, int skip_at,
+                                                       uint32_t tid, uint32_t nthr,
+                                                       size_t first_pass, size_t pass_step) {
+  constexpr int U = kStreamUnroll;
+  constexpr int kNt = 2;
+  const uint32_t lane_off = tid * 16u;
+  const uint32_t access_bytes = nthr * 16u;
+  const uint32_t pass_bytes = access_bytes * U;
+  const size_t step_bytes = pass_step * pass_bytes;
+  for (size_t b = first_pass * pass_bytes; b < body; b += step_bytes) {
+    const size_t left = body - b;
+    const int valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
+    u32x4 v[U];
+    if constexpr (kBufferLoads) {
+      __amdgpu_buffer_rsrc_t rs = uniform_rsrc(src + b, valid);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        v[u] = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * access_bytes, kNt);
+    } else if (static_cast<uint32_t>(valid) == pass_bytes) {
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        v[u] = __builtin_nontemporal_load(
+            reinterpret_cast<const u32x4_a1 *>(src + b + u * access_bytes + lane_off));
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t off = u * access_bytes + lane_off;  // valid is a multiple of 16
+        v[u] = u32x4{0, 0, 0, 0};
+        if (off < static_cast<uint32_t>(valid))
+          v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_a1 *>(src + b + off));
+      }
+    }
+    // Destination i of the ndst that are written, without a branch around the
+    // skipped member: a conditional `continue` in this loop cost a sixth of
+    // the broadcast's bandwidth.
+    for (int i = 0; i < ndst; ++i) {
+      const int m = i + (i >= skip_at ? 1 : 0);
+      __amdgpu_buffer_rsrc_t rd = uniform_rsrc(dst0 + m * member_step + b, valid);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        __builtin_amdgcn_raw_buffer_store_b128(v[u], rd, lane_off, u * access_bytes, kNt);
+    }
+  }
+}
+
 // Copy `n` bytes from `src` into the same symmetric address `dst_mine` of
-// every member for which `skip_idx != member index`.  When source and
-// destinations are aligned alike modulo 4 every source vector is loaded
-// once and stored to each destination (raw-buffer addressing as in
-// stream_copy_uniform); otherwise each destination is copied on its own.
+// every member for which `skip_idx != member index`.  Every source vector is
+// loaded once and stored to each destination (raw-buffer addressing as in
+// stream_copy_uniform); payloads under 256 bytes are copied per destination.
 // Arguments are workgroup-uniform.
 //
 // `first_pass` / `pass_step` (vector path only; the caller checks alignment
@@ -56,10 +107,12 @@ __device__ __forceinline__ void wg_copy_to_members(char *dst_mine, const char *s
   const int64_t stride = static_cast<int64_t>(g_state.slice_stride);
   char *dst0 = dst_mine + (static_cast<int64_t>(as.pe_start) - my_pe) * stride;
   const int64_t member_step = stride << as.log_stride;
-  // The vector path stores 16-byte aligned and loads at any 4-byte alignment.
+  // The vector path stores 16-byte aligned; it loads through a buffer
+  // descriptor when the source then sits at a 4-byte boundary and with
+  // per-lane unaligned vector loads otherwise.
   const bool coaligned =
       ((reinterpret_cast<uintptr_t>(dst_mine) ^ reinterpret_cast<uintptr_t>(src)) & 3u) == 0;
-  if (!coaligned || n < 256) {
+  if (n < 256) {
     for (int m = 0; m < as.size; ++m) {
       if (m == skip_idx) continue;
       group_copy_uniform(dst0 + m * member_step, src, n, tid, nthr);
@@ -75,33 +128,16 @@ __device__ __forceinline__ void wg_copy_to_members(char *dst_mine, const char *s
     for (int m = 0; m < as.size; ++m)
       if (m != skip_idx) dst0[m * member_step + off] = b;
   }
-  constexpr int U = kStreamUnroll;
-  constexpr int kNt = 2;
   const bool skips = skip_idx >= 0 && skip_idx < as.size;
   const int ndst = as.size - (skips ? 1 : 0);
   const int skip_at = skips ? skip_idx : as.size;
-  const uint32_t lane_off = tid * 16u;
-  const uint32_t access_bytes = nthr * 16u;
-  const uint32_t pass_bytes = access_bytes * U;
-  const size_t step_bytes = pass_step * pass_bytes;
-  for (size_t b = first_pass * pass_bytes; b < body; b += step_bytes) {
-    const size_t left = body - b;
-    const int valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
-    __amdgpu_buffer_rsrc_t rs = uniform_rsrc(src + head + b, valid);
-    u32x4 v[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-      v[u] = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * access_bytes, kNt);
-    // Destination i of the ndst that are written, without a branch around the
-    // skipped member: a conditional `continue` in this loop cost a sixth of
-    // the broadcast's bandwidth.
-    for (int i = 0; i < ndst; ++i) {
-      const int m = i + (i >= skip_at ? 1 : 0);
-      __amdgpu_buffer_rsrc_t rd = uniform_rsrc(dst0 + m * member_step + head + b, valid);
-#pragma unroll
-      for (int u = 0; u < U; ++u)
-        __builtin_amdgcn_raw_buffer_store_b128(v[u], rd, lane_off, u * access_bytes, kNt);
-    }
+  // One loop per way of loading, so that neither carries the other's registers and branches.
+  if (coaligned) {
+    copy_passes_to_members<true>(dst0 + head, src + head, body, member_step, ndst, skip_at, tid, nthr,
+                                 first_pass, pass_step);
+  } else {
+    copy_passes_to_members<false>(dst0 + head, src + head, body, member_step, ndst, skip_at, tid, nthr,
+                                  first_pass, pass_step);
   }
 }
 
@@ -111,7 +147,7 @@ __device__ __forceinline__ void wg_copy_to_members(char *dst_mine, const char *s
 // is the root's ordinal within the active set.
 //
 // `shard` / `nshards`: several workgroups of every member share the call.  A
-// large, mutually aligned payload is dealt to them pass by pass (the
+// large payload is dealt to them pass by pass (the
 // workgroups running at one moment then write one compact window of every
 // destination: 1 -> 15 broadcast of 64 MiB on MI355X, 5.8 TB/s with 8
 // workgroups of 1024 lanes per PE against 5.6 TB/s with a contiguous range
@@ -148,9 +184,7 @@ __device__ __forceinline__ void wg_broadcast_bytes(int my_pe, void *dest, const 
 
   const char *root_src = translate(static_cast<const char *>(source), my_pe, as.pe_at(root_idx));
   const size_t pass_bytes = static_cast<size_t>(nthr) * 16u * kStreamUnroll;
-  const bool coaligned =
-      ((reinterpret_cast<uintptr_t>(dest) ^ reinterpret_cast<uintptr_t>(root_src)) & 3u) == 0;
-  if (coaligned && nbytes >= 2 * parts * pass_bytes) {
+  if (nbytes >= 2 * parts * pass_bytes) {
     wg_copy_to_members(static_cast<char *>(dest), root_src, nbytes, as, my_pe, root_idx, tid, nthr,
                        part, parts, part == 0);
   } else {

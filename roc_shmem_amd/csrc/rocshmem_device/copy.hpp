@@ -97,6 +97,43 @@ __device__ __forceinline__ void copy_vec_src_bytes(u32x4 *__restrict__ d,
   }
 }
 
+// dst 16-byte aligned, src at any byte offset, group-uniform arguments: the
+// hardware reads a 16-byte vector at any byte address (unaligned access is
+// enabled for global memory), so the pass structure of stream_copy_uniform
+// carries over with per-lane global loads in place of buffer loads.
+typedef u32x4 u32x4_a1 __attribute__((aligned(1)));
+template <bool kNt, int U>
+__device__ __forceinline__ void stream_copy_src_unaligned(char *d, const char *s, size_t nbytes,
+                                                          uint32_t tid, uint32_t nthr,
+                                                          size_t first_pass = 0,
+                                                          size_t pass_step = 1) {
+  const size_t access_bytes = static_cast<size_t>(nthr) * 16u;
+  const size_t pass_bytes = access_bytes * U;
+  const size_t mine = static_cast<size_t>(tid) * 16u;
+  // This group takes passes first_pass, first_pass + pass_step, ...; the last
+  // pass of the range may be partial.
+  for (size_t b = first_pass * pass_bytes; b < nbytes; b += pass_step * pass_bytes) {
+    if (b + pass_bytes <= nbytes) {
+      u32x4 v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const u32x4_a1 *p = reinterpret_cast<const u32x4_a1 *>(s + b + u * access_bytes + mine);
+        if constexpr (kNt) {
+          v[u] = __builtin_nontemporal_load(p);
+        } else {
+          v[u] = *p;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        store_vec<kNt>(v[u], reinterpret_cast<u32x4 *>(d + b + u * access_bytes + mine));
+    } else {
+      for (size_t at = b + mine; at < nbytes; at += access_bytes)
+        *reinterpret_cast<u32x4 *>(d + at) = *reinterpret_cast<const u32x4_a1 *>(s + at);
+    }
+  }
+}
+
 // memcpy(dst, src, n) executed cooperatively by lanes tid = 0..nthr-1, for
 // per-lane (possibly different in every lane) arguments: the thread-level
 // put/get path.  No barrier inside.
@@ -237,7 +274,11 @@ __device__ __forceinline__ void group_copy_uniform(void *dst, const void *src, s
   if ((reinterpret_cast<uintptr_t>(s) & 3u) == 0) {
     stream_copy_sized(d, s, body, tid, nthr);
   } else {
-    copy_vec_src_bytes(reinterpret_cast<u32x4 *>(d), s, body / 16, tid, nthr);
+    if (body >= kNonTemporalBytes) {
+      stream_copy_src_unaligned<true, kStreamUnroll>(d, s, body, tid, nthr);
+    } else {
+      stream_copy_src_unaligned<false, kCopyUnroll>(d, s, body, tid, nthr);
+    }
   }
   for (size_t i = body + tid; i < n; i += nthr) d[i] = s[i];
 }
@@ -260,14 +301,18 @@ __device__ __forceinline__ void group_copy_dealt(void *dst, const void *src, siz
   // The vector path stores 16-byte aligned and loads at any 4-byte alignment.
   const bool coaligned =
       ((reinterpret_cast<uintptr_t>(d) ^ reinterpret_cast<uintptr_t>(s)) & 3u) == 0;
-  if (coaligned && n >= 2 * parts * pass_bytes) {
+  if (n >= 2 * parts * pass_bytes) {
     const size_t head = stream_head(d, n);
     const size_t body = (n - head) & ~static_cast<size_t>(15);
     if (part == 0) {
       for (size_t i = tid; i < head; i += nthr) d[i] = s[i];
       for (size_t i = head + body + tid; i < n; i += nthr) d[i] = s[i];
     }
-    stream_copy_uniform<2 /* nt */, kStreamUnroll>(d + head, s + head, body, tid, nthr, part, parts);
+    if (coaligned) {
+      stream_copy_uniform<2 /* nt */, kStreamUnroll>(d + head, s + head, body, tid, nthr, part, parts);
+    } else {
+      stream_copy_src_unaligned<true, kStreamUnroll>(d + head, s + head, body, tid, nthr, part, parts);
+    }
   } else {
     size_t share = (n + parts - 1) / parts;
     share = (share + 255) / 256 * 256;

@@ -68,9 +68,10 @@ def test_broadcast_shrinking_and_strided_sets(pe_start, log_stride, pe_size, roo
 @pytest.mark.parametrize("wgs,wg_size,tile,shift", [(2, 256, 0, 4), (3, 128, 0, 0), (4, 512, 0, 4),
                                                     (2, 256, 100000, 4), (2, 256, 0, (4, 5))])
 def test_broadcast_large_payload_shared_by_several_workgroups(wgs, wg_size, tile, shift):
-    # tile 0: the PE's workgroups share one broadcast pass by pass (mutually aligned arrays, here
-    # 4 bytes past a 16-byte boundary) or range by range (arrays misaligned against each other);
-    # tile > 0: one standard call per tile.  3 MiB + 13 bytes, bytes around the payload untouched.
+    # tile 0: the PE's workgroups share one broadcast pass by pass, reading the source through a
+    # buffer descriptor (arrays aligned alike modulo 4, here 4 bytes past a 16-byte boundary) or
+    # with unaligned vector loads (arrays one byte apart); tile > 0: one standard call per tile.
+    # 3 MiB + 13 bytes, bytes around the payload untouched.
     n_pes, nbytes = 4, (3 << 20) + 13
     s_shift, d_shift = shift if isinstance(shift, tuple) else (shift, shift)
     with runtime(n_pes):
