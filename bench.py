@@ -260,6 +260,29 @@ def bench_small_ops(rs, n_pes, n_ops, wgs_total, wg_size, slice_bytes, seed):
         ms = event_time_ms(rs, step, 3) / 3
         res[name] = {"Mops_per_s": n_ops / ms / 1e3, "ms": ms}
         dev.free()
+    # Fetch-adds that collide: every op on one word, and on 16 words (one per PE).  Lanes of a wave
+    # that name the same word share one atomic.
+    for name, n_words in (("fetch_add_one_word", 1), ("fetch_add_16_words", 16)):
+        ops = np.zeros(n_ops, rs.SMALL_OP_DTYPE)
+        word = rng.integers(0, n_words, n_ops)
+        ops["kind"] = rs.OP_FADD64
+        ops["pe"] = word % n_pes
+        ops["offset"] = mem.offset + (words - 1) * 8
+        ops["value"] = rng.integers(1, 5, n_ops)
+        mem.fill(0)
+        dev = rs.device_array(ops)
+
+        def hot():
+            rs.roc_shmem_small_ops(dev, n_ops, None, launch)
+
+        hot()
+        rs.synchronize()
+        ms = event_time_ms(rs, hot, 3) / 3
+        total = sum(int(mem.read(p)[words - 1]) for p in range(min(n_pes, n_words)))
+        if total != 4 * int(ops["value"].sum()):
+            raise RuntimeError("%s: the words hold %d, expected %d" % (name, total, 4 * int(ops["value"].sum())))
+        res[name] = {"Mops_per_s": n_ops / ms / 1e3, "ms": ms}
+        dev.free()
     # Lane-contiguous 8-byte putmems: the coalescer merges each wave's 64 messages into one 512-byte
     # WQE (wf_coal_policy.cpp:57-172); every lane still moves its own 8 bytes.
     half = words // 2

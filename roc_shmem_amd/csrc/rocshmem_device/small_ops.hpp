@@ -177,10 +177,80 @@ __device__ __forceinline__ void amo_record(DeviceCtx *ctx, uint8_t opcode, T *re
   wave_post(ctx, true, rq);
 }
 
+__device__ __forceinline__ uint32_t first_lane_word(uint32_t v) { return first_lane_u32(v); }
+__device__ __forceinline__ uint64_t first_lane_word(uint64_t v) { return first_lane_u64(v); }
+__device__ __forceinline__ uint32_t lane_word(uint32_t v, int lane) {
+  return __builtin_amdgcn_readlane(v, lane);
+}
+__device__ __forceinline__ uint64_t lane_word(uint64_t v, int lane) {
+  const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(v), lane);
+  const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(v >> 32), lane);
+  return (static_cast<uint64_t>(hi) << 32) | lo;
+}
+
+// fetch_add on `remote` by every active lane.  Atomics on one word are
+// carried out one after the other where the word lives (12 ns each at agent
+// scope: 83 M/s however many lanes ask), so lanes of the wave that name the
+// same word add the sum of their operands with one atomic, and each gets what
+// it would have fetched had they gone in lane order: the word's previous value
+// plus the operands of the group's lanes below it.  Any serialisation is a
+// valid outcome of concurrent AMOs; this is one.
+//
+// Groups are looked for leader by leader (the lowest lane not yet served and
+// every lane with its address).  The search stops at the first leader without
+// a partner, so a wave whose lanes all name different words (the usual case,
+// uniformly random targets) pays one round of a dozen instructions; at most
+// kCombineRounds groups are formed.  Lanes left over issue their own atomic.
+constexpr int kCombineRounds = 16;
+template <typename T>
+__device__ __forceinline__ T wave_fetch_add(T *remote, T value) {
+  using W = typename AtomicWord<T>::type;
+  const uint64_t active = __ballot(1);
+  const uint64_t addr = reinterpret_cast<uint64_t>(remote);
+  const uint32_t me = lane_id();
+  W v;
+  __builtin_memcpy(&v, &value, sizeof(T));
+  W fetched = 0;
+  uint64_t todo = active;
+  for (int round = 0; round < kCombineRounds && todo; ++round) {
+    const int leader = __builtin_ctzll(todo);
+    const uint64_t group = __ballot(addr == lane_word(addr, leader)) & todo;
+    const uint32_t members = __popcll(group);
+    if (members == 1) break;
+    W below = 0, total = 0;
+    if ((__ballot(v == lane_word(v, leader)) & group) == group) {
+      // one operand for the whole group (increments, a common addend): closed form
+      below = static_cast<W>(rank_in_mask(group)) * v;
+      total = static_cast<W>(members) * lane_word(v, leader);
+    } else {
+      for (uint64_t g = group; g; g &= g - 1) {
+        const int lane = __builtin_ctzll(g);
+        if (me == static_cast<uint32_t>(lane)) below = total;
+        total += lane_word(v, lane);
+      }
+    }
+    W base = 0;
+    if (me == static_cast<uint32_t>(leader)) {
+      base = __hip_atomic_fetch_add(reinterpret_cast<W *>(remote), total, __ATOMIC_RELAXED,
+                                    __HIP_MEMORY_SCOPE_AGENT);
+    }
+    base = lane_word(base, leader);
+    if ((group >> me) & 1u) fetched = base + below;
+    todo &= ~group;
+  }
+  if ((todo >> me) & 1u) {
+    fetched = __hip_atomic_fetch_add(reinterpret_cast<W *>(remote), v, __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_AGENT);
+  }
+  T old;
+  __builtin_memcpy(&old, &fetched, sizeof(T));
+  return old;
+}
+
 template <typename T>
 __device__ __forceinline__ T amo_fetch_add(DeviceCtx *ctx, T *dest, T value, int pe) {
   T *remote = translate(dest, ctx->my_pe, pe);
-  const T old = __hip_atomic_fetch_add(remote, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const T old = wave_fetch_add(remote, value);
   amo_record<T>(ctx, kOpcodeAtomicFa, remote, value, T(0), pe);
   return old;
 }
@@ -188,7 +258,7 @@ __device__ __forceinline__ T amo_fetch_add(DeviceCtx *ctx, T *dest, T value, int
 template <typename T>
 __device__ __forceinline__ void amo_add(DeviceCtx *ctx, T *dest, T value, int pe) {
   T *remote = translate(dest, ctx->my_pe, pe);
-  (void)__hip_atomic_fetch_add(remote, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  (void)wave_fetch_add(remote, value);
   amo_record<T>(ctx, kOpcodeAtomicFa, remote, value, T(0), pe);
 }
 

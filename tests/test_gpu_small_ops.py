@@ -216,6 +216,62 @@ def test_amo_family_closed_forms():
         mem.free()
 
 
+def assert_serialisation(fetched, addends, initial, final, modulus):
+    """The fetched values are those of some order of the adds: sorted by what they fetched, each
+    op finds the word as the previous one left it (all addends are positive and the total stays
+    below the modulus... or wraps exactly once, which the sort key accounts for)."""
+    seen = [int(f) % modulus for f in fetched]
+    order = sorted(range(len(seen)), key=lambda i: (seen[i] - initial) % modulus)
+    value = initial % modulus
+    for i in order:
+        assert seen[i] == value, "op %d fetched %d, the word held %d" % (i, seen[i], value)
+        value = (value + int(addends[i])) % modulus
+    assert value == final % modulus
+
+
+@pytest.mark.parametrize("n_words,wg_size", [(1, 256), (3, 256), (16, 64), (40, 128)])
+def test_fetch_adds_that_collide_form_a_serialisation(n_words, wg_size):
+    # Lanes of a wave that name the same word share one atomic; every op must still fetch what
+    # some order of all the adds would have shown it, and the word must end at the total.
+    n_pes, wgs, words, n = 4, 2, 64, 6000
+    rng = np.random.default_rng(n_words)
+    with runtime(n_pes, num_blocks=2):
+        init = [np.full(words, 1000 + p, np.int64) for p in range(n_pes)]
+        ops = np.zeros(n, rs.SMALL_OP_DTYPE)
+        word = rng.integers(0, n_words, n)
+        ops["kind"] = rs.OP_FADD64
+        ops["pe"] = word % n_pes
+        ops["offset"] = (word // n_pes) * 8
+        ops["value"] = rng.integers(1, 1000, n)
+        same = rng.random(n) < 0.3
+        ops["value"][same] = 7                     # runs of equal addends take the closed-form path
+        mem, shifted, out, got = run_stream(ops, n_pes, wgs, wg_size, words * 8, init)
+        for w in range(n_words):
+            sel = np.nonzero(word == w)[0]
+            pe, slot = w % n_pes, w // n_pes
+            assert_serialisation(got[sel], ops["value"][sel], 1000 + pe, int(out[pe][slot]), 1 << 64)
+            assert int(out[pe][slot]) == 1000 + pe + int(ops["value"][sel].sum())
+        mem.free()
+
+
+def test_colliding_32_bit_fetch_adds_wrap():
+    n_pes, words, n = 2, 8, 3000
+    rng = np.random.default_rng(5)
+    with runtime(n_pes, num_blocks=2):
+        init = [np.zeros(words, np.int64) for _ in range(n_pes)]
+        init[1][0] = 0xFFFFF000                    # low word close to wrapping, high word zero
+        ops = np.zeros(n, rs.SMALL_OP_DTYPE)
+        ops["kind"], ops["pe"], ops["offset"] = rs.OP_FADD32, 1, 0
+        ops["value"] = rng.integers(1, 100, n)
+        mem, shifted, out, got = run_stream(ops, n_pes, 2, 256, words * 8, init)
+        total = int(ops["value"].sum())
+        low = int(out[1][0]) & 0xFFFFFFFF
+        assert low == (0xFFFFF000 + total) & 0xFFFFFFFF
+        assert int(out[1][0]) >> 32 == 0, "a 32-bit add reached the neighbouring word"
+        assert_serialisation(got & 0xFFFFFFFF, ops["value"], 0xFFFFF000, low, 1 << 32)
+        mem.free()
+
+
 def test_swap_set_cswap_fetch_and_bitwise():
     n_pes, words = 2, 32
     with runtime(n_pes, num_blocks=1):
