@@ -905,6 +905,77 @@ static void primitive_amo() {
   EXPECT(hipFree(ret_val) == hipSuccess, "hipFree");
 }
 
+// ---- many collectives inside one kernel (the shape of sos_tests/bcast_flood.cpp and
+// shmem_team_b2b_collectives.cpp, on the device): `rounds` reductions back to back on one pSync,
+// every PE changing its source between two of them; then as many broadcasts from a moving root.
+__global__ void BackToBackCollectives(int rounds, long *src, long *dst, long *pWrk, long *pSync, int n,
+                                      uint64_t *timer) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  const int np = roc_shmem_ctx_n_pes(ctx);
+  src = roc_shmemx_my_addr(src);
+  dst = roc_shmemx_my_addr(dst);
+  pWrk = roc_shmemx_my_addr(pWrk);
+  pSync = roc_shmemx_my_addr(pSync);
+  const uint64_t start = roc_shmem_timer();
+  for (int r = 0; r < rounds; ++r) {
+    roc_shmem_ctx_long_sum_wg_to_all(ctx, dst, src, n, 0, 0, np, pWrk, pSync);
+    // the reduction has returned on this PE, so every PE has read this source
+    for (int k = threadIdx.x; k < n; k += blockDim.x) src[k] += 1;
+  }
+  if (threadIdx.x == 0) timer[blockIdx.x] = roc_shmem_timer() - start;
+  for (int r = 0; r < rounds; ++r)
+    roc_shmem_ctx_long_wg_broadcast(ctx, src, dst, n, r % np, 0, 0, np, pSync);
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+static void back_to_back_collectives() {
+  current_case = "collectives back to back inside one kernel";
+  const int n = 4096, rounds = 100;
+  long *src = static_cast<long *>(roc_shmem_malloc(n * sizeof(long)));
+  long *dst = static_cast<long *>(roc_shmem_malloc(n * sizeof(long)));
+  long *pWrk = static_cast<long *>(roc_shmem_malloc(ROC_SHMEM_REDUCE_MIN_WRKDATA_SIZE * sizeof(long)));
+  long *pSync = static_cast<long *>(roc_shmem_malloc(ROC_SHMEM_REDUCE_SYNC_SIZE * sizeof(long)));
+  uint64_t *timer;
+  EXPECT(hipMalloc(&timer, npes * sizeof(uint64_t)) == hipSuccess, "hipMalloc");
+  std::vector<long> v(n);
+  for (int pe = 0; pe < npes; ++pe) {
+    for (int k = 0; k < n; ++k) v[k] = pe + k;
+    roc_shmem_putmem(src, v.data(), n * sizeof(long), pe);
+    fill(dst, n, -1L, pe);
+    fill(pSync, static_cast<int>(ROC_SHMEM_REDUCE_SYNC_SIZE), 0L, pe);
+  }
+  BackToBackCollectives<<<npes, 512>>>(rounds, src, dst, pWrk, pSync, n, timer);
+  finish_kernel("BackToBackCollectives");
+  // the last reduction saw src_p[k] = p + k + rounds - 1
+  for (int pe = 0; pe < npes; ++pe) {
+    std::vector<long> got = load(dst, n, pe);
+    for (int k = 0; k < n; ++k) {
+      const long want = static_cast<long>(npes) * (k + rounds - 1) + static_cast<long>(npes) * (npes - 1) / 2;
+      if (got[k] != want) {
+        EXPECT(false, "PE %d dst[%d] = %ld, expected %ld", pe, k, got[k], want);
+        break;
+      }
+    }
+    // every broadcast copied dst (the same everywhere) over src of all PEs but that round's root,
+    // and every PE has been a receiver by then
+    std::vector<long> s = load(src, n, pe);
+    EXPECT(s == got, "PE %d: src differs from dst after the broadcasts (src[7] = %ld)", pe, s[7]);
+    for (long x : load(pSync, static_cast<int>(ROC_SHMEM_REDUCE_SYNC_SIZE), pe)) EXPECT(x == 0, "pSync on PE %d", pe);
+  }
+  uint64_t ticks = 0;
+  EXPECT(hipMemcpy(&ticks, timer, sizeof(ticks), hipMemcpyDeviceToHost) == hipSuccess, "timer copy");
+  printf("  sum_to_all of %d longs inside one kernel: %.2f us per call (%d PEs, one workgroup each)\n", n,
+         ticks * 0.01 / rounds, npes);
+  EXPECT(hipFree(timer) == hipSuccess, "hipFree");
+  roc_shmem_free(pSync);
+  roc_shmem_free(pWrk);
+  roc_shmem_free(dst);
+  roc_shmem_free(src);
+}
+
 int main() {
   if (!getenv("ROC_SHMEM_NUM_PES")) setenv("ROC_SHMEM_NUM_PES", "4", 1);
   setenv("ROC_SHMEM_HEAP_SIZE", "67108864", 0);
@@ -920,7 +991,8 @@ int main() {
                {"swarm", swarm},               {"amo_testers", amo_testers},
                {"random_access", random_access},
                {"default_ctx", default_ctx},   {"primitive_mr", primitive_mr},
-               {"primitive_amo", primitive_amo}};
+               {"primitive_amo", primitive_amo},
+               {"back_to_back_collectives", back_to_back_collectives}};
   for (auto &c : cases) {
     const int before = failures;
     c.run();
