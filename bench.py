@@ -364,8 +364,9 @@ def bench_bcast_a2a(rs, n_pes, slice_bytes):
     res = {}
     src = rs.sym_array(slice_bytes, np.uint8, fill=3)
     dst = rs.sym_array(slice_bytes, np.uint8, fill=0)
-    launch = rs.Launch(16, 512)
-    bcast_launch = rs.Launch(8, 1024)
+    # best of a sweep over 8/16/32 workgroups per PE x 512/1024 threads for each
+    launch = rs.Launch(16, 1024)
+    bcast_launch = fcollect_launch = rs.Launch(8, 1024)
     nelem = slice_bytes // 4
 
     def bcast():
@@ -384,6 +385,17 @@ def bench_bcast_a2a(rs, n_pes, slice_bytes):
     rs.synchronize()
     ms = event_time_ms(rs, a2a, 5) / 5
     res["alltoall"] = {"GBps": 2.0 * n_pes * slice_bytes / ms / 1e6, "ms": ms}
+
+    def fcollect():
+        rs.roc_shmem_fcollect(4, world, dst, src, block, fcollect_launch)
+
+    fcollect()
+    rs.synchronize()
+    ms = event_time_ms(rs, fcollect, 5) / 5
+    # every member's block is read once and written into all n_pes dests
+    res["fcollect"] = {"GBps": float(n_pes + 1) * slice_bytes / ms / 1e6, "ms": ms}
+    if rs.take_status():
+        raise RuntimeError("device status word raised")
     src.free()
     dst.free()
     return res
@@ -438,6 +450,8 @@ def main():
                          "plain wg putmem copy of known size (2 GiB read + 2 GiB written), nothing else")
     ap.add_argument("--small-ops", action="store_true",
                     help="for rocprofv3 --pmc: the 10 M-operation streams and the consumer pass, nothing else")
+    ap.add_argument("--collectives", action="store_true",
+                    help="for rocprofv3: broadcast, alltoall and fcollect over 16 slices x 64 MiB, nothing else")
     ap.add_argument("--alignment", action="store_true",
                     help="large put / broadcast / reduction with shifted source and destination, nothing else")
     args = ap.parse_args()
@@ -454,6 +468,12 @@ def main():
         out = bench_small_ops(rs, 16, 10_000_000, 1024, 256, 64 << 20, seed=4)
         rs.roc_shmem_finalize()
         print(json.dumps({"small_ops_16x64MiB_1024wg_x256": out}))
+        return
+    if args.collectives:
+        rs.roc_shmem_init(16, 256 << 20, 64, 1024)
+        out = bench_bcast_a2a(rs, 16, 64 << 20)
+        rs.roc_shmem_finalize()
+        print(json.dumps({"collectives_16x64MiB": out}))
         return
     if args.alignment:
         rs.roc_shmem_init(8, 1 << 30, 64, 1024)
