@@ -29,6 +29,7 @@ def _load():
     lib.orc_dtype_size.restype = sz
     lib.orc_dtype_size.argtypes = [i32]
     lib.orc_to_all.argtypes = [i32, i32, vp, sz, sz, sz, sz, i32, i32, i32]
+    lib.orc_to_all_team.argtypes = [i32, i32, vp, sz, sz, sz, sz, i32, i32, i32]
     lib.orc_to_all_mt.argtypes = [i32, i32, vp, sz, sz, sz, sz, i32, i32, i32, i32]
     lib.orc_to_all_f64.argtypes = [i32, i32, vp, sz, sz, sz, i32, i32, i32, vp]
     lib.orc_abs_sum_f64.argtypes = [i32, vp, sz, sz, sz, i32, i32, i32, vp]
@@ -41,7 +42,9 @@ def _load():
         getattr(lib, name).argtypes = [vp, sz, sz, sz, sz, i32, i32]
     lib.orc_broadcast.restype = None
     lib.orc_broadcast.argtypes = [vp, sz, sz, sz, sz, i32, i32, i32, i32]
-    for name in ("orc_alltoall", "orc_fcollect"):
+    lib.orc_broadcast_team.restype = None
+    lib.orc_broadcast_team.argtypes = [vp, sz, sz, sz, sz, i32, i32, i32, i32]
+    for name in ("orc_alltoall", "orc_fcollect", "orc_alltoall_team", "orc_fcollect_team"):
         getattr(lib, name).restype = None
         getattr(lib, name).argtypes = [vp, sz, sz, sz, sz, i32, i32, i32]
     lib.orc_copy_mt.restype = None
@@ -116,9 +119,13 @@ class Heap:
 
 
 def to_all(heap, dtype, op, dest_off, src_off, n, pe_start=0, log_stride=0, pe_size=None,
-           threads=1):
+           threads=1, pe_stride=None):
+    """pe_stride: the team form, members pe_start + k * pe_stride (log_stride is then ignored)."""
     pe_size = heap.n_pes if pe_size is None else pe_size
-    if threads > 1:
+    if pe_stride is not None:
+        rc = _lib.orc_to_all_team(dtype, op, heap.ptr, heap.stride, dest_off, src_off, n, pe_start,
+                                  pe_stride, pe_size)
+    elif threads > 1:
         rc = _lib.orc_to_all_mt(dtype, op, heap.ptr, heap.stride, dest_off, src_off, n, pe_start,
                                 log_stride, pe_size, threads)
     else:
@@ -167,20 +174,35 @@ def get(heap, dest_off, src_off, nbytes, my_pe, from_pe):
     _lib.orc_get(heap.ptr, heap.stride, dest_off, src_off, nbytes, my_pe, from_pe)
 
 
-def broadcast(heap, dest_off, src_off, nbytes, root_idx, pe_start=0, log_stride=0, pe_size=None):
+def broadcast(heap, dest_off, src_off, nbytes, root_idx, pe_start=0, log_stride=0, pe_size=None,
+              pe_stride=None):
     pe_size = heap.n_pes if pe_size is None else pe_size
+    if pe_stride is not None:
+        _lib.orc_broadcast_team(heap.ptr, heap.stride, dest_off, src_off, nbytes, root_idx, pe_start,
+                                pe_stride, pe_size)
+        return
     _lib.orc_broadcast(heap.ptr, heap.stride, dest_off, src_off, nbytes, root_idx, pe_start,
                        log_stride, pe_size)
 
 
-def alltoall(heap, dest_off, src_off, block_bytes, pe_start=0, log_stride=0, pe_size=None):
+def alltoall(heap, dest_off, src_off, block_bytes, pe_start=0, log_stride=0, pe_size=None,
+             pe_stride=None):
     pe_size = heap.n_pes if pe_size is None else pe_size
+    if pe_stride is not None:
+        _lib.orc_alltoall_team(heap.ptr, heap.stride, dest_off, src_off, block_bytes, pe_start,
+                               pe_stride, pe_size)
+        return
     _lib.orc_alltoall(heap.ptr, heap.stride, dest_off, src_off, block_bytes, pe_start, log_stride,
                       pe_size)
 
 
-def fcollect(heap, dest_off, src_off, block_bytes, pe_start=0, log_stride=0, pe_size=None):
+def fcollect(heap, dest_off, src_off, block_bytes, pe_start=0, log_stride=0, pe_size=None,
+             pe_stride=None):
     pe_size = heap.n_pes if pe_size is None else pe_size
+    if pe_stride is not None:
+        _lib.orc_fcollect_team(heap.ptr, heap.stride, dest_off, src_off, block_bytes, pe_start,
+                               pe_stride, pe_size)
+        return
     _lib.orc_fcollect(heap.ptr, heap.stride, dest_off, src_off, block_bytes, pe_start, log_stride,
                       pe_size)
 

@@ -31,6 +31,9 @@ size_t orc_dtype_size(int dtype);
  * Returns 0, or -1 for an undefined (dtype, op) pair. */
 int orc_to_all(int dtype, int op, char *heap, size_t stride, size_t dest_off, size_t src_off,
                size_t n, int pe_start, int log_stride, int pe_size);
+/* Team form: members pe_start + k * pe_stride, any pe_stride >= 1. */
+int orc_to_all_team(int dtype, int op, char *heap, size_t stride, size_t dest_off, size_t src_off,
+                    size_t n, int pe_start, int pe_stride, int pe_size);
 /* Ground truth: the same reduction evaluated in long double on the exact
  * values of the inputs, returned as double.  out[n]. */
 int orc_to_all_f64(int dtype, int op, const char *heap, size_t stride, size_t src_off, size_t n,
@@ -56,6 +59,13 @@ void orc_alltoall(char *heap, size_t stride, size_t dest_off, size_t src_off, si
                   int pe_start, int log_stride, int pe_size);
 void orc_fcollect(char *heap, size_t stride, size_t dest_off, size_t src_off, size_t block_bytes,
                   int pe_start, int log_stride, int pe_size);
+/* Team forms of the three: members pe_start + k * pe_stride, any pe_stride >= 1. */
+void orc_broadcast_team(char *heap, size_t stride, size_t dest_off, size_t src_off, size_t nbytes,
+                        int root_idx, int pe_start, int pe_stride, int pe_size);
+void orc_alltoall_team(char *heap, size_t stride, size_t dest_off, size_t src_off,
+                       size_t block_bytes, int pe_start, int pe_stride, int pe_size);
+void orc_fcollect_team(char *heap, size_t stride, size_t dest_off, size_t src_off,
+                       size_t block_bytes, int pe_start, int pe_stride, int pe_size);
 /* memcpy spread over `threads` host threads (CPU baseline for put/get). */
 void orc_copy_mt(char *dst, const char *src, size_t nbytes, int threads);
 

@@ -49,7 +49,9 @@ uint16_t orc_float_to_bf16(float f) {
   return (uint16_t)(u >> 16);
 }
 
-static int member_pe(int k, int pe_start, int log_stride) { return pe_start + (k << log_stride); }
+/* Member k of the set {pe_start + k * pe_stride}.  The active-set calls pass 1 << logPE_stride; a
+ * team may have any stride (roc_shmem_team_split_strided, library/src/roc_shmem.cpp:236-250). */
+static int member_pe(int k, int pe_start, int pe_stride) { return pe_start + k * pe_stride; }
 
 /* Integer fold on an unsigned carrier of the element's width: two's-complement
  * wrap for sum and prod, signed comparison for max and min. */
@@ -134,16 +136,16 @@ static void combine_bf16(int op, uint16_t *restrict dst, const uint16_t *restric
  * a bounded scratch block so that dest == source (in place) and misaligned
  * offsets are handled the same way. */
 static void reduce_range(int dtype, int op, char *heap, size_t stride, size_t dest_off,
-                         size_t src_off, size_t e0, size_t e1, int pe_start, int log_stride,
+                         size_t src_off, size_t e0, size_t e1, int pe_start, int pe_stride,
                          int pe_size) {
   enum { BLOCK = 4096 };
   const size_t es = orc_dtype_size(dtype);
   union { int64_t i64[BLOCK]; double f64[BLOCK]; char bytes[BLOCK * 8]; } acc, in;
   for (size_t b = e0; b < e1; b += BLOCK) {
     const size_t n = (e1 - b < BLOCK) ? e1 - b : BLOCK;
-    memcpy(acc.bytes, heap + (size_t)member_pe(0, pe_start, log_stride) * stride + src_off + b * es, n * es);
+    memcpy(acc.bytes, heap + (size_t)member_pe(0, pe_start, pe_stride) * stride + src_off + b * es, n * es);
     for (int k = 1; k < pe_size; ++k) {
-      memcpy(in.bytes, heap + (size_t)member_pe(k, pe_start, log_stride) * stride + src_off + b * es, n * es);
+      memcpy(in.bytes, heap + (size_t)member_pe(k, pe_start, pe_stride) * stride + src_off + b * es, n * es);
       switch (dtype) {
         case ORC_SHORT: combine_i16(op, (int16_t *)acc.bytes, (const int16_t *)in.bytes, n); break;
         case ORC_INT: combine_i32(op, (int32_t *)acc.bytes, (const int32_t *)in.bytes, n); break;
@@ -154,14 +156,23 @@ static void reduce_range(int dtype, int op, char *heap, size_t stride, size_t de
       }
     }
     for (int m = 0; m < pe_size; ++m)
-      memcpy(heap + (size_t)member_pe(m, pe_start, log_stride) * stride + dest_off + b * es, acc.bytes, n * es);
+      memcpy(heap + (size_t)member_pe(m, pe_start, pe_stride) * stride + dest_off + b * es, acc.bytes, n * es);
   }
 }
 
 int orc_to_all(int dtype, int op, char *heap, size_t stride, size_t dest_off, size_t src_off,
                size_t n, int pe_start, int log_stride, int pe_size) {
   if (!op_defined(dtype, op)) return -1;
-  reduce_range(dtype, op, heap, stride, dest_off, src_off, 0, n, pe_start, log_stride, pe_size);
+  reduce_range(dtype, op, heap, stride, dest_off, src_off, 0, n, pe_start, 1 << log_stride, pe_size);
+  return 0;
+}
+
+/* The team form (GPUIBContext::to_all(team, ...), context_ib_tmpl_device.hpp:238-260): the members
+ * are the team's, pe_start + k * pe_stride in world ranks. */
+int orc_to_all_team(int dtype, int op, char *heap, size_t stride, size_t dest_off, size_t src_off,
+                    size_t n, int pe_start, int pe_stride, int pe_size) {
+  if (!op_defined(dtype, op) || pe_stride < 1) return -1;
+  reduce_range(dtype, op, heap, stride, dest_off, src_off, 0, n, pe_start, pe_stride, pe_size);
   return 0;
 }
 
@@ -182,9 +193,9 @@ int orc_to_all_f64(int dtype, int op, const char *heap, size_t stride, size_t sr
   const size_t es = orc_dtype_size(dtype);
   if (!es) return -1;
   for (size_t i = 0; i < n; ++i) {
-    long double acc = load_ld(dtype, heap + (size_t)member_pe(0, pe_start, log_stride) * stride + src_off + i * es);
+    long double acc = load_ld(dtype, heap + (size_t)member_pe(0, pe_start, 1 << log_stride) * stride + src_off + i * es);
     for (int k = 1; k < pe_size; ++k) {
-      long double x = load_ld(dtype, heap + (size_t)member_pe(k, pe_start, log_stride) * stride + src_off + i * es);
+      long double x = load_ld(dtype, heap + (size_t)member_pe(k, pe_start, 1 << log_stride) * stride + src_off + i * es);
       switch (op) {
         case ORC_SUM: acc += x; break;
         case ORC_PROD: acc *= x; break;
@@ -204,7 +215,7 @@ int orc_abs_sum_f64(int dtype, const char *heap, size_t stride, size_t src_off, 
   for (size_t i = 0; i < n; ++i) {
     long double acc = 0;
     for (int k = 0; k < pe_size; ++k)
-      acc += fabsl(load_ld(dtype, heap + (size_t)member_pe(k, pe_start, log_stride) * stride + src_off + i * es));
+      acc += fabsl(load_ld(dtype, heap + (size_t)member_pe(k, pe_start, 1 << log_stride) * stride + src_off + i * es));
     out[i] = (double)acc;
   }
   return 0;
@@ -220,7 +231,7 @@ struct mt_job {
 static void *mt_worker(void *arg) {
   struct mt_job *j = (struct mt_job *)arg;
   reduce_range(j->dtype, j->op, j->heap, j->stride, j->dest_off, j->src_off, j->e0, j->e1,
-               j->pe_start, j->log_stride, j->pe_size);
+               j->pe_start, 1 << j->log_stride, j->pe_size);
   return NULL;
 }
 

@@ -25,7 +25,9 @@
 
 #include "oracle.h"
 
-static int member_pe(int k, int pe_start, int log_stride) { return pe_start + (k << log_stride); }
+/* Member k of the set {pe_start + k * pe_stride}: 1 << logPE_stride for an active set, any stride
+ * for a team (roc_shmem_team_split_strided, library/src/roc_shmem.cpp:236-250). */
+static int member_pe(int k, int pe_start, int pe_stride) { return pe_start + k * pe_stride; }
 
 void orc_put(char *heap, size_t stride, size_t dest_off, size_t src_off, size_t nbytes,
              int src_pe, int dest_pe) {
@@ -41,33 +43,49 @@ void orc_get(char *heap, size_t stride, size_t dest_off, size_t src_off, size_t 
           nbytes);
 }
 
-void orc_broadcast(char *heap, size_t stride, size_t dest_off, size_t src_off, size_t nbytes,
-                   int root_idx, int pe_start, int log_stride, int pe_size) {
+void orc_broadcast_team(char *heap, size_t stride, size_t dest_off, size_t src_off, size_t nbytes,
+                   int root_idx, int pe_start, int pe_stride, int pe_size) {
   if (!nbytes) return;
-  const char *src = heap + (size_t)member_pe(root_idx, pe_start, log_stride) * stride + src_off;
+  const char *src = heap + (size_t)member_pe(root_idx, pe_start, pe_stride) * stride + src_off;
   for (int m = 0; m < pe_size; ++m) {
     if (m == root_idx) continue;
-    memmove(heap + (size_t)member_pe(m, pe_start, log_stride) * stride + dest_off, src, nbytes);
+    memmove(heap + (size_t)member_pe(m, pe_start, pe_stride) * stride + dest_off, src, nbytes);
   }
+}
+
+void orc_alltoall_team(char *heap, size_t stride, size_t dest_off, size_t src_off, size_t block_bytes,
+                  int pe_start, int pe_stride, int pe_size) {
+  if (!block_bytes) return;
+  for (int i = 0; i < pe_size; ++i)
+    for (int j = 0; j < pe_size; ++j)
+      memmove(heap + (size_t)member_pe(j, pe_start, pe_stride) * stride + dest_off + (size_t)i * block_bytes,
+              heap + (size_t)member_pe(i, pe_start, pe_stride) * stride + src_off + (size_t)j * block_bytes,
+              block_bytes);
+}
+
+void orc_fcollect_team(char *heap, size_t stride, size_t dest_off, size_t src_off, size_t block_bytes,
+                  int pe_start, int pe_stride, int pe_size) {
+  if (!block_bytes) return;
+  for (int i = 0; i < pe_size; ++i)
+    for (int j = 0; j < pe_size; ++j)
+      memmove(heap + (size_t)member_pe(j, pe_start, pe_stride) * stride + dest_off + (size_t)i * block_bytes,
+              heap + (size_t)member_pe(i, pe_start, pe_stride) * stride + src_off, block_bytes);
+}
+
+/* Active-set forms: the members are pe_start + (k << log_stride). */
+void orc_broadcast(char *heap, size_t stride, size_t dest_off, size_t src_off, size_t nbytes,
+                   int root_idx, int pe_start, int log_stride, int pe_size) {
+  orc_broadcast_team(heap, stride, dest_off, src_off, nbytes, root_idx, pe_start, 1 << log_stride, pe_size);
 }
 
 void orc_alltoall(char *heap, size_t stride, size_t dest_off, size_t src_off, size_t block_bytes,
                   int pe_start, int log_stride, int pe_size) {
-  if (!block_bytes) return;
-  for (int i = 0; i < pe_size; ++i)
-    for (int j = 0; j < pe_size; ++j)
-      memmove(heap + (size_t)member_pe(j, pe_start, log_stride) * stride + dest_off + (size_t)i * block_bytes,
-              heap + (size_t)member_pe(i, pe_start, log_stride) * stride + src_off + (size_t)j * block_bytes,
-              block_bytes);
+  orc_alltoall_team(heap, stride, dest_off, src_off, block_bytes, pe_start, 1 << log_stride, pe_size);
 }
 
 void orc_fcollect(char *heap, size_t stride, size_t dest_off, size_t src_off, size_t block_bytes,
                   int pe_start, int log_stride, int pe_size) {
-  if (!block_bytes) return;
-  for (int i = 0; i < pe_size; ++i)
-    for (int j = 0; j < pe_size; ++j)
-      memmove(heap + (size_t)member_pe(j, pe_start, log_stride) * stride + dest_off + (size_t)i * block_bytes,
-              heap + (size_t)member_pe(i, pe_start, log_stride) * stride + src_off, block_bytes);
+  orc_fcollect_team(heap, stride, dest_off, src_off, block_bytes, pe_start, 1 << log_stride, pe_size);
 }
 
 struct copy_job { char *dst; const char *src; size_t n; };

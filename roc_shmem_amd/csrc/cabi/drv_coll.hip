@@ -65,7 +65,8 @@ __device__ __forceinline__ bool in_set(int me, int pe_start, int stride, int pe_
 template <typename T, bool kTeam, bool kShard>
 __global__ void __launch_bounds__(1024)
     broadcast_kernel(roc_shmem_team_t team, T *dest0, const T *source0, size_t n, size_t tile,
-                     int pe_root, int pe_start, int log_stride, int pe_size, long *pSync0) {
+                     int pe_root, int pe_start, int log_stride, int pe_stride, int pe_size,
+                     long *pSync0) {
   __shared__ roc_shmem_ctx_t ctx;
   roc_shmem_wg_init();
   roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
@@ -73,7 +74,7 @@ __global__ void __launch_bounds__(1024)
   const int npes = roc_shmem_ctx_n_pes(ctx);
   const size_t w = blockIdx.x / npes;
   const size_t nw = gridDim.x / npes;
-  if (in_set(me, pe_start, 1 << log_stride, pe_size)) {
+  if (in_set(me, pe_start, pe_stride, pe_size)) {
     T *dest = roc_shmemx_my_addr(dest0);
     const T *source = roc_shmemx_my_addr(source0);
     long *pSync = kTeam ? nullptr : roc_shmemx_my_addr(pSync0) + w * ROC_SHMEM_BCAST_SYNC_SIZE;
@@ -139,7 +140,7 @@ struct BcastArgs {
   void *dest;
   const void *source;
   size_t n, tile;
-  int root, pe_start, log_stride, pe_size;
+  int root, pe_start, log_stride, pe_stride, pe_size;  // log_stride: active-set form only
   long *pSync;
 };
 
@@ -147,7 +148,8 @@ template <typename T, bool kTeam, bool kShard>
 void launch_bcast_form(const rsm::Launch &l, const BcastArgs &a) {
   hipLaunchKernelGGL((broadcast_kernel<T, kTeam, kShard>), dim3(l.grid), dim3(l.wg_size), 0,
                      l.stream, a.team, static_cast<T *>(a.dest), static_cast<const T *>(a.source),
-                     a.n, a.tile, a.root, a.pe_start, a.log_stride, a.pe_size, a.pSync);
+                     a.n, a.tile, a.root, a.pe_start, a.log_stride, a.pe_stride, a.pe_size,
+                     a.pSync);
 }
 
 template <typename T>
@@ -235,8 +237,8 @@ int rsm_broadcast(size_t elem_size, void *dest, const void *source, size_t nelem
       pe_start + ((pe_size - 1) << log_pe_stride) >= rt->num_pes() || pe_root < 0 ||
       pe_root >= pe_size)
     return rsm::fail("broadcast: active set or root out of range");
-  BcastArgs a{nullptr, dest, source, nelem, l.tile, pe_root, pe_start, log_pe_stride, pe_size,
-              pSync};
+  BcastArgs a{nullptr, dest, source, nelem, l.tile, pe_root, pe_start, log_pe_stride,
+              1 << log_pe_stride, pe_size, pSync};
   return run_bcast(elem_size, l, a);
 }
 
@@ -254,7 +256,7 @@ int rsm_broadcast_team(size_t elem_size, uint64_t team, void *dest, const void *
   const detail::TeamInfo &ti = rec->image.wrt_world;
   if (pe_root < 0 || pe_root >= ti.size) return rsm::fail("broadcast_team: root out of range");
   BcastArgs a{reinterpret_cast<roc_shmem_team_t>(team), dest, source, nelem, l.tile, pe_root,
-              ti.pe_start, ti.log_stride, ti.size, nullptr};
+              ti.pe_start, 0, ti.stride, ti.size, nullptr};
   return run_bcast(elem_size, l, a);
 }
 

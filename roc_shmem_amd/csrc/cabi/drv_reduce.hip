@@ -265,7 +265,7 @@ int rsm_to_all_team(int dtype, int op, uint64_t team, void *dest, const void *so
   if (l.wgs_per_pe > rt->options().num_blocks)
     return rsm::fail("to_all_team: wgs_per_pe exceeds the contexts per PE (team pSync slices)");
   const detail::TeamInfo &ti = rec->image.wrt_world;
-  ReduceArgs a{dest, source, nreduce, l.tile, ti.pe_start, ti.log_stride, ti.size, nullptr,
+  ReduceArgs a{dest, source, nreduce, l.tile, ti.pe_start, 0, ti.size, nullptr,
                nullptr, reinterpret_cast<roc_shmem_team_t>(team), ti.stride};
   return run(dtype, op, l, a);
 }

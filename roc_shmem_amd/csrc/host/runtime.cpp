@@ -372,9 +372,10 @@ int Runtime::team_split(detail::Team *parent, int start, int stride, int size,
   int stride_world = stride * pi.stride;
   int end_world = start_world + stride_world * (size - 1);
   if (end_world >= opt_.num_pes) return -1;
-  if (stride_world & (stride_world - 1)) return -1;  // collectives address members by log2 stride
+  // Any stride makes a team, as in the reference; log_stride is its log2 rounded down
+  // (library/src/team.cpp:68), exact for the powers of two the active-set calls can name.
   int log_stride = 0;
-  while ((1 << log_stride) < stride_world) ++log_stride;
+  while ((2 << log_stride) <= stride_world) ++log_stride;
   // teams_ holds the world team too; the reference counts user teams only
   // (num_user_teams >= max_num_teams - 1 aborts, roc_shmem.cpp:224-228).
   if (static_cast<int>(teams_.size()) - 1 >= kMaxTeams - 1) {

@@ -418,8 +418,8 @@ __device__ __forceinline__ void to_all_active_set(roc_shmem_ctx_t ctx, T *dest, 
                                                   size_t nreduce, int pe_start, int log_stride,
                                                   int pe_size, long *psync, int shard = 0,
                                                   int nshards = 1) {
-  wg_all_reduce<T, Op>(ctx_of(ctx)->my_pe, dest, source, nreduce, pe_start, log_stride, pe_size,
-                       psync, shard, nshards);
+  wg_all_reduce<T, Op>(ctx_of(ctx)->my_pe, dest, source, nreduce, pe_start, 1 << log_stride,
+                       pe_size, psync, shard, nshards);
 }
 // reference: GPUIBContext::to_all(team, ...), context_ib_tmpl_device.hpp:238-260
 template <typename T, ROC_SHMEM_OP Op>
@@ -429,7 +429,7 @@ __device__ __forceinline__ void to_all_team(roc_shmem_ctx_t ctx, roc_shmem_team_
   const DeviceCtx *c = ctx_of(ctx);
   const Team *t = team_of(team);
   wg_all_reduce<T, Op>(c->my_pe, dest, source, nreduce, t->wrt_world.pe_start,
-                       t->wrt_world.log_stride, t->wrt_world.size,
+                       t->wrt_world.stride, t->wrt_world.size,
                        team_psync(c, t->reduce_psync_off), shard, nshards);
 }
 }  // namespace detail
@@ -507,7 +507,7 @@ ROCSHMEM_REDUCTION(__hip_bfloat16, bf16, min, ROC_SHMEM_MIN)
     if (nelem <= 0) return;                                                                    \
     detail::wg_broadcast_bytes(detail::ctx_of(ctx)->my_pe, dest, source,                       \
                                static_cast<size_t>(nelem) * sizeof(T), pe_root, pe_start,      \
-                               log_pe_stride, pe_size, p_sync);                                \
+                               1 << log_pe_stride, pe_size, p_sync);                           \
   }                                                                                            \
   __device__ inline void roc_shmem_ctx_##TNAME##_wg_broadcast(                                 \
       roc_shmem_ctx_t ctx, roc_shmem_team_t team, T *dest, const T *source, int nelem,         \
@@ -516,7 +516,7 @@ ROCSHMEM_REDUCTION(__hip_bfloat16, bf16, min, ROC_SHMEM_MIN)
     const detail::DeviceCtx *c = detail::ctx_of(ctx);                                          \
     const detail::Team *t = detail::team_of(team);                                             \
     detail::wg_broadcast_bytes(c->my_pe, dest, source, static_cast<size_t>(nelem) * sizeof(T), \
-                               pe_root, t->wrt_world.pe_start, t->wrt_world.log_stride,        \
+                               pe_root, t->wrt_world.pe_start, t->wrt_world.stride,            \
                                t->wrt_world.size, detail::team_psync(c, t->bcast_psync_off));  \
   }                                                                                            \
   /* extension: `nshards` workgroups of every member share one broadcast (same */              \
@@ -525,7 +525,7 @@ ROCSHMEM_REDUCTION(__hip_bfloat16, bf16, min, ROC_SHMEM_MIN)
       roc_shmem_ctx_t ctx, T *dest, const T *source, size_t nelem, int pe_root, int pe_start,  \
       int log_pe_stride, int pe_size, long *p_sync, int shard, int nshards) {                  \
     detail::wg_broadcast_bytes(detail::ctx_of(ctx)->my_pe, dest, source, nelem * sizeof(T),    \
-                               pe_root, pe_start, log_pe_stride, pe_size, p_sync, shard,       \
+                               pe_root, pe_start, 1 << log_pe_stride, pe_size, p_sync, shard,  \
                                nshards);                                                       \
   }                                                                                            \
   __device__ inline void roc_shmemx_ctx_##TNAME##_wg_broadcast_shard(                          \
@@ -534,7 +534,7 @@ ROCSHMEM_REDUCTION(__hip_bfloat16, bf16, min, ROC_SHMEM_MIN)
     const detail::DeviceCtx *c = detail::ctx_of(ctx);                                          \
     const detail::Team *t = detail::team_of(team);                                             \
     detail::wg_broadcast_bytes(c->my_pe, dest, source, nelem * sizeof(T), pe_root,             \
-                               t->wrt_world.pe_start, t->wrt_world.log_stride,                 \
+                               t->wrt_world.pe_start, t->wrt_world.stride,                     \
                                t->wrt_world.size, detail::team_psync(c, t->bcast_psync_off),   \
                                shard, nshards);                                                \
   }                                                                                            \
@@ -546,7 +546,7 @@ ROCSHMEM_REDUCTION(__hip_bfloat16, bf16, min, ROC_SHMEM_MIN)
     const detail::DeviceCtx *c = detail::ctx_of(ctx);                                          \
     const detail::Team *t = detail::team_of(team);                                             \
     detail::wg_alltoall_bytes(c->my_pe, dest, source, static_cast<size_t>(nelem) * sizeof(T),  \
-                              shard, nshards, t->wrt_world.pe_start, t->wrt_world.log_stride,  \
+                              shard, nshards, t->wrt_world.pe_start, t->wrt_world.stride,      \
                               t->wrt_world.size, detail::team_psync(c, t->alltoall_psync_off)); \
   }                                                                                            \
   __device__ inline void roc_shmem_ctx_##TNAME##_wg_alltoall(                                  \
@@ -560,7 +560,7 @@ ROCSHMEM_REDUCTION(__hip_bfloat16, bf16, min, ROC_SHMEM_MIN)
     const detail::DeviceCtx *c = detail::ctx_of(ctx);                                          \
     const detail::Team *t = detail::team_of(team);                                             \
     detail::wg_fcollect_bytes(c->my_pe, dest, source, static_cast<size_t>(nelem) * sizeof(T),  \
-                              shard, nshards, t->wrt_world.pe_start, t->wrt_world.log_stride,  \
+                              shard, nshards, t->wrt_world.pe_start, t->wrt_world.stride,      \
                               t->wrt_world.size, detail::team_psync(c, t->alltoall_psync_off)); \
   }                                                                                            \
   __device__ inline void roc_shmem_ctx_##TNAME##_wg_fcollect(                                  \
@@ -577,7 +577,7 @@ ROCSHMEM_STANDARD_TYPES(ROCSHMEM_COLLECTIVES)
 __device__ inline void roc_shmem_ctx_wg_team_sync(roc_shmem_ctx_t ctx, roc_shmem_team_t team) {
   const detail::DeviceCtx *c = detail::ctx_of(ctx);
   const detail::Team *t = detail::team_of(team);
-  detail::wg_sync_members(c->my_pe, t->wrt_world.pe_start, t->wrt_world.log_stride,
+  detail::wg_sync_members(c->my_pe, t->wrt_world.pe_start, t->wrt_world.stride,
                           t->wrt_world.size, detail::team_psync(c, t->barrier_psync_off));
 }
 __device__ inline void roc_shmem_wg_team_sync(roc_shmem_team_t team) {
@@ -586,7 +586,7 @@ __device__ inline void roc_shmem_wg_team_sync(roc_shmem_team_t team) {
 __device__ inline void roc_shmem_ctx_wg_sync_all(roc_shmem_ctx_t ctx) {
   const detail::DeviceCtx *c = detail::ctx_of(ctx);
   const detail::Team *t = detail::g_state.team_world;
-  detail::wg_sync_members(c->my_pe, 0, 0, c->num_pes,
+  detail::wg_sync_members(c->my_pe, 0, 1, c->num_pes,
                           detail::team_psync(c, t->barrier_psync_off));
 }
 __device__ inline void roc_shmem_wg_sync_all() { roc_shmem_ctx_wg_sync_all(ROC_SHMEM_CTX_DEFAULT); }

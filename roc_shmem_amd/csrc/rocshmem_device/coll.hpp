@@ -106,7 +106,7 @@ __device__ __forceinline__ void wg_copy_to_members(char *dst_mine, const char *s
   if (n == 0) return;
   const int64_t stride = static_cast<int64_t>(g_state.slice_stride);
   char *dst0 = dst_mine + (static_cast<int64_t>(as.pe_start) - my_pe) * stride;
-  const int64_t member_step = stride << as.log_stride;
+  const int64_t member_step = stride * as.pe_stride;
   // The vector path stores 16-byte aligned; it loads through a buffer
   // descriptor when the source then sits at a 4-byte boundary and with
   // per-lane unaligned vector loads otherwise.
@@ -154,7 +154,7 @@ __device__ __forceinline__ void wg_copy_to_members(char *dst_mine, const char *s
 // per workgroup); anything else is cut into contiguous ranges.
 __device__ __forceinline__ void wg_broadcast_bytes(int my_pe, void *dest, const void *source,
                                                    size_t nbytes, int root_idx, int pe_start,
-                                                   int log_stride, int pe_size, long *psync,
+                                                   int pe_stride, int pe_size, long *psync,
                                                    int shard = 0, int nshards = 1) {
   my_pe = uniform(my_pe);
   shard = uniform(shard);
@@ -164,7 +164,7 @@ __device__ __forceinline__ void wg_broadcast_bytes(int my_pe, void *dest, const 
   nbytes = uniform(nbytes);
   root_idx = uniform(root_idx);
   pe_start = uniform(pe_start);
-  log_stride = uniform(log_stride);
+  pe_stride = uniform(pe_stride);
   pe_size = uniform(pe_size);
   psync = uniform(psync);
   if (nbytes == 0) return;
@@ -173,14 +173,14 @@ __device__ __forceinline__ void wg_broadcast_bytes(int my_pe, void *dest, const 
     status_raise(kStatusBadArgument);
     return;
   }
-  const ActiveSet as{pe_start, log_stride, pe_size};
-  const int my_idx = (my_pe - pe_start) >> log_stride;
+  const ActiveSet as{pe_start, pe_stride, pe_size};
+  const int my_idx = member_index(my_pe - pe_start, pe_stride);
   const uint32_t tid = flat_thread_id();
   const uint32_t nthr = flat_block_size();
   const size_t parts = static_cast<size_t>(pe_size) * nshards;
   const size_t part = static_cast<size_t>(shard) * pe_size + my_idx;
 
-  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, log_stride, pe_size);
+  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, pe_stride, pe_size);
 
   const char *root_src = translate(static_cast<const char *>(source), my_pe, as.pe_at(root_idx));
   const size_t pass_bytes = static_cast<size_t>(nthr) * 16u * kStreamUnroll;
@@ -194,7 +194,7 @@ __device__ __forceinline__ void wg_broadcast_bytes(int my_pe, void *dest, const 
                        tid, nthr);
   }
 
-  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, log_stride, pe_size);
+  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size);
 }
 
 // Alltoall block exchange: member i's block j goes to member j's block i,
@@ -205,7 +205,7 @@ __device__ __forceinline__ void wg_broadcast_bytes(int my_pe, void *dest, const 
 // measured slower here: 5.9 against 6.1 TB/s for 16 x 16 blocks of 4 MiB).
 __device__ __forceinline__ void wg_alltoall_bytes(int my_pe, void *dest, const void *source,
                                                   size_t block_bytes, int shard, int nshards,
-                                                  int pe_start, int log_stride, int pe_size,
+                                                  int pe_start, int pe_stride, int pe_size,
                                                   long *psync) {
   my_pe = uniform(my_pe);
   dest = uniform(dest);
@@ -214,7 +214,7 @@ __device__ __forceinline__ void wg_alltoall_bytes(int my_pe, void *dest, const v
   shard = uniform(shard);
   nshards = uniform(nshards);
   pe_start = uniform(pe_start);
-  log_stride = uniform(log_stride);
+  pe_stride = uniform(pe_stride);
   pe_size = uniform(pe_size);
   psync = uniform(psync);
   if (block_bytes == 0) return;
@@ -222,12 +222,12 @@ __device__ __forceinline__ void wg_alltoall_bytes(int my_pe, void *dest, const v
     status_raise(kStatusBadArgument);
     return;
   }
-  const ActiveSet as{pe_start, log_stride, pe_size};
-  const int my_idx = (my_pe - pe_start) >> log_stride;
+  const ActiveSet as{pe_start, pe_stride, pe_size};
+  const int my_idx = member_index(my_pe - pe_start, pe_stride);
   const uint32_t tid = flat_thread_id();
   const uint32_t nthr = flat_block_size();
 
-  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, log_stride, pe_size);
+  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, pe_stride, pe_size);
 
   char *dst_mine = static_cast<char *>(dest) + static_cast<size_t>(my_idx) * block_bytes;
   const char *src = static_cast<const char *>(source);
@@ -241,14 +241,14 @@ __device__ __forceinline__ void wg_alltoall_bytes(int my_pe, void *dest, const v
                        src + static_cast<size_t>(j) * block_bytes + b, e - b, tid, nthr);
   }
 
-  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, log_stride, pe_size);
+  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size);
 }
 
 // Fcollect: member i's `block_bytes` land in block i of every member's dest
 // (reference: fcollect_broadcast, context_ib_tmpl_device.hpp:845-876).
 __device__ __forceinline__ void wg_fcollect_bytes(int my_pe, void *dest, const void *source,
                                                   size_t block_bytes, int shard, int nshards,
-                                                  int pe_start, int log_stride, int pe_size,
+                                                  int pe_start, int pe_stride, int pe_size,
                                                   long *psync) {
   my_pe = uniform(my_pe);
   dest = uniform(dest);
@@ -257,7 +257,7 @@ __device__ __forceinline__ void wg_fcollect_bytes(int my_pe, void *dest, const v
   shard = uniform(shard);
   nshards = uniform(nshards);
   pe_start = uniform(pe_start);
-  log_stride = uniform(log_stride);
+  pe_stride = uniform(pe_stride);
   pe_size = uniform(pe_size);
   psync = uniform(psync);
   if (block_bytes == 0) return;
@@ -265,12 +265,12 @@ __device__ __forceinline__ void wg_fcollect_bytes(int my_pe, void *dest, const v
     status_raise(kStatusBadArgument);
     return;
   }
-  const ActiveSet as{pe_start, log_stride, pe_size};
-  const int my_idx = (my_pe - pe_start) >> log_stride;
+  const ActiveSet as{pe_start, pe_stride, pe_size};
+  const int my_idx = member_index(my_pe - pe_start, pe_stride);
   const uint32_t tid = flat_thread_id();
   const uint32_t nthr = flat_block_size();
 
-  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, log_stride, pe_size);
+  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, pe_stride, pe_size);
 
   // The member's own block goes to block my_idx of everybody; the member's
   // workgroups take one contiguous range of it each (dealing a 4 MiB block
@@ -281,25 +281,25 @@ __device__ __forceinline__ void wg_fcollect_bytes(int my_pe, void *dest, const v
   split_range(block_bytes, nshards, shard, 256, b, e);
   wg_copy_to_members(dst_mine + b, src + b, e - b, as, my_pe, -1, tid, nthr);
 
-  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, log_stride, pe_size);
+  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size);
 }
 
 // Barrier among the member workgroups (reference: internal_sync,
 // context_ib_device_coll.cpp:67-89).
-__device__ __forceinline__ void wg_sync_members(int my_pe, int pe_start, int log_stride,
+__device__ __forceinline__ void wg_sync_members(int my_pe, int pe_start, int pe_stride,
                                                 int pe_size, long *psync) {
   my_pe = uniform(my_pe);
   pe_start = uniform(pe_start);
-  log_stride = uniform(log_stride);
+  pe_stride = uniform(pe_stride);
   pe_size = uniform(pe_size);
   psync = uniform(psync);
   if (pe_size > kMaxPes || pe_size <= 0) {
     status_raise(kStatusBadArgument);
     return;
   }
-  const int my_idx = (my_pe - pe_start) >> log_stride;
-  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, log_stride, pe_size);
-  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, log_stride, pe_size);
+  const int my_idx = member_index(my_pe - pe_start, pe_stride);
+  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, pe_stride, pe_size);
+  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size);
 }
 
 }  // namespace detail

@@ -131,12 +131,21 @@ struct VecOf {
 constexpr int kReduceUnroll = 8;   // vectors per lane per pass
 constexpr int kReducePeChunk = 1;  // members whose loads are issued together
 
+// Members of a collective: world PEs pe_start + k * pe_stride, k < size.  The
+// active-set calls name powers of two (1 << logPE_stride); a team may have any
+// stride (roc_shmem_team_split_strided, library/src/roc_shmem.cpp:236-250).
 struct ActiveSet {
   int pe_start;
-  int log_stride;
+  int pe_stride;
   int size;
-  __device__ __forceinline__ int pe_at(int k) const { return pe_start + (k << log_stride); }
+  __device__ __forceinline__ int pe_at(int k) const { return pe_start + k * pe_stride; }
 };
+
+// Ordinal of the PE `rel` places after pe_start in a set of stride pe_stride.
+__device__ __forceinline__ int member_index(int rel, int pe_stride) {
+  if ((pe_stride & (pe_stride - 1)) == 0) return rel >> __builtin_ctz(pe_stride);
+  return rel / pe_stride;
+}
 
 // Reduce vectors [v_begin, v_end) of the symmetric arrays `src`/`dst` (given
 // as this PE's addresses, both 16-byte aligned) over all members and write
@@ -173,7 +182,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
                (static_cast<int64_t>(as.pe_start) - my_pe) * stride;
   char *dst0 =
       reinterpret_cast<char *>(dst) + (static_cast<int64_t>(as.pe_start) - my_pe) * stride;
-  const int64_t member_step = stride << as.log_stride;
+  const int64_t member_step = stride * as.pe_stride;
 
   const uint32_t lane_off = tid * 16u;
   const uint32_t access_bytes = nthr * 16u;       // bytes one instruction of the workgroup sweeps
@@ -251,7 +260,7 @@ __device__ __forceinline__ void reduce_elements(T *dst, const T *src, size_t e_b
                      (static_cast<int64_t>(as.pe_start) - my_pe) * stride;
   char *dst0 =
       reinterpret_cast<char *>(dst) + (static_cast<int64_t>(as.pe_start) - my_pe) * stride;
-  const int64_t member_step = stride << as.log_stride;
+  const int64_t member_step = stride * as.pe_stride;
   for (size_t i = e_begin + tid; i < e_end; i += nthr) {
     Acc acc = to_acc<T, Acc>(reinterpret_cast<const Elem *>(src0)[i]);
     for (int k = 1; k < as.size; ++k) {
@@ -273,7 +282,7 @@ __device__ __forceinline__ void reduce_elements(T *dst, const T *src, size_t e_b
 // overwritten by the same lanes.
 template <typename T, ROC_SHMEM_OP Op>
 __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *source, size_t nreduce,
-                                              int pe_start, int log_stride, int pe_size,
+                                              int pe_start, int pe_stride, int pe_size,
                                               long *psync, int shard = 0, int nshards = 1) {
   // Workgroup-collective: every lane holds the same arguments.
   my_pe = uniform(my_pe);
@@ -281,7 +290,7 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
   source = uniform(source);
   nreduce = uniform(nreduce);
   pe_start = uniform(pe_start);
-  log_stride = uniform(log_stride);
+  pe_stride = uniform(pe_stride);
   pe_size = uniform(pe_size);
   psync = uniform(psync);
   shard = uniform(shard);
@@ -291,8 +300,8 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
     status_raise(kStatusBadArgument);
     return;
   }
-  const ActiveSet as{pe_start, log_stride, pe_size};
-  const int my_idx = (my_pe - pe_start) >> log_stride;
+  const ActiveSet as{pe_start, pe_stride, pe_size};
+  const int my_idx = member_index(my_pe - pe_start, pe_stride);
   const uint32_t tid = flat_thread_id();
   const uint32_t nthr = flat_block_size();
   const size_t n = nreduce;
@@ -301,7 +310,7 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
   const size_t parts = static_cast<size_t>(pe_size) * nshards;
   const size_t part = static_cast<size_t>(shard) * pe_size + my_idx;
 
-  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, log_stride, pe_size);
+  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, pe_stride, pe_size);
 
   constexpr size_t E = VecOf<T>::kElems;
   // The vector path stores 16-byte aligned and loads at any 4-byte alignment,
@@ -366,7 +375,7 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
     reduce_elements<T, Op>(dest, source, e0, e1, as, my_pe, tid, nthr);
   }
 
-  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, log_stride, pe_size);
+  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size);
 }
 
 }  // namespace detail

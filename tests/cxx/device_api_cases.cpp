@@ -429,6 +429,71 @@ static void sync_and_barrier() {
   roc_shmem_free(slot);
 }
 
+// A team of stride 3 (world PEs 0 and 3; shmem_team_translate.cpp:46-47 splits the world this way):
+// team_sync with a hand-off between the two members in every round, then a sum reduction over the
+// team inside the same kernel.  PEs 1 and 2 run the kernel too and must be left alone.
+__global__ void StridedTeamTest(int loop, long *slot, int *dst, const int *src, int n,
+                                roc_shmem_team_t team, roc_shmem_team_t world, int *errors) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  const int me = roc_shmem_ctx_my_pe(ctx);
+  const int rank = roc_shmem_team_translate_pe(world, me, team);
+  if (rank >= 0) {
+    slot = roc_shmemx_my_addr(slot);
+    const int other = roc_shmem_team_translate_pe(team, 1 - rank, world);
+    for (int i = 1; i <= loop; i++) {
+      if (threadIdx.x == 0) {
+        roc_shmem_ctx_long_p(ctx, slot, 1000L * me + i, other);
+        roc_shmem_ctx_quiet(ctx);
+      }
+      roc_shmem_ctx_wg_team_sync(ctx, team);
+      if (threadIdx.x == 0 && roc_shmem_ctx_long_g(ctx, slot, me) != 1000L * other + i) atomicAdd(errors, 1);
+      roc_shmem_ctx_wg_team_sync(ctx, team);
+    }
+    roc_shmem_ctx_int_sum_wg_to_all(ctx, team, roc_shmemx_my_addr(dst), roc_shmemx_my_addr(src), n);
+  }
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+static void strided_team() {
+  current_case = "team of stride 3";
+  if (npes < 4) return;
+  const int n = 3000, loop = 40;
+  long *slot = static_cast<long *>(roc_shmem_malloc(sizeof(long)));
+  int *src = static_cast<int *>(roc_shmem_malloc(n * sizeof(int)));
+  int *dst = static_cast<int *>(roc_shmem_malloc(n * sizeof(int)));
+  int *errors = nullptr;
+  (void)hipMalloc(reinterpret_cast<void **>(&errors), sizeof(int));
+  (void)hipMemset(errors, 0, sizeof(int));
+  roc_shmem_team_t team = ROC_SHMEM_TEAM_INVALID;
+  const int ret = roc_shmem_team_split_strided(ROC_SHMEM_TEAM_WORLD, 0, 3, 2, nullptr, 0, &team);
+  EXPECT(ret == 0 && team != ROC_SHMEM_TEAM_INVALID, "split {0, 3} returned %d", ret);
+  if (team != ROC_SHMEM_TEAM_INVALID) {
+    for (int pe = 0; pe < npes; ++pe) {
+      fill(slot, 1, -1L, pe);
+      fill(src, n, 100 * (pe + 1), pe);
+      fill(dst, n, -5, pe);
+    }
+    StridedTeamTest<<<npes, 256>>>(loop, slot, dst, src, n, team, ROC_SHMEM_TEAM_WORLD, errors);
+    finish_kernel("StridedTeamTest");
+    int bad = -1;
+    (void)hipMemcpy(&bad, errors, sizeof(int), hipMemcpyDeviceToHost);
+    EXPECT(bad == 0, "%d hand-offs seen too early or too late", bad);
+    for (int pe = 0; pe < npes; ++pe) {
+      std::vector<int> got = load(dst, n, pe);
+      const int want = (pe == 0 || pe == 3) ? 100 * 1 + 100 * 4 : -5;
+      for (int i = 0; i < n; ++i) EXPECT(got[i] == want, "PE %d [%d] = %d, expected %d", pe, i, got[i], want);
+    }
+    roc_shmem_team_destroy(team);
+  }
+  (void)hipFree(errors);
+  roc_shmem_free(dst);
+  roc_shmem_free(src);
+  roc_shmem_free(slot);
+}
+
 // ---- swarm_tester.cpp:31-58: every thread of PE 0's workgroup gets its own chunk from PE 1 -------
 __global__ void GetSwarmTest(int loop, char *s_buf, char *r_buf, int size) {
   __shared__ roc_shmem_ctx_t ctx;
@@ -988,6 +1053,7 @@ int main() {
                {"narrow_ping_pong", narrow_ping_pong},
                {"shmem_ptr", shmem_ptr},       {"team_ctx_infra", team_ctx_infra},
                {"team_ctx_primitive", team_ctx_primitive}, {"sync_and_barrier", sync_and_barrier},
+               {"strided_team", strided_team},
                {"swarm", swarm},               {"amo_testers", amo_testers},
                {"random_access", random_access},
                {"default_ctx", default_ctx},   {"primitive_mr", primitive_mr},

@@ -795,6 +795,107 @@ static void team_reuse_teams() {
   roc_shmem_team_destroy(old_team);
 }
 
+// clients/sos_tests/shmem_team_translate.cpp:40-93: teams of every second and every third PE; a PE
+// is in team_2s iff me % 2 == 0 and in team_3s iff me % 3 == 0, and its rank translates from one
+// team to the other iff it is in both.  Beyond the reference's checks: the ranks themselves, and a
+// sum reduction and a broadcast over the team of stride 3.
+static void team_translate() {
+  current_case = "shmem_team_translate.cpp";
+  roc_shmem_team_t team_2s, team_3s;
+  int ret = roc_shmem_team_split_strided(ROC_SHMEM_TEAM_WORLD, 0, 2, (npes - 1) / 2 + 1, nullptr, 0, &team_2s);
+  EXPECT(ret == 0 && team_2s != ROC_SHMEM_TEAM_INVALID, "split of stride 2 returned %d", ret);
+  ret = roc_shmem_team_split_strided(ROC_SHMEM_TEAM_WORLD, 0, 3, (npes - 1) / 3 + 1, nullptr, 0, &team_3s);
+  EXPECT(ret == 0 && team_3s != ROC_SHMEM_TEAM_INVALID, "split of stride 3 returned %d", ret);
+  if (team_2s == ROC_SHMEM_TEAM_INVALID || team_3s == ROC_SHMEM_TEAM_INVALID) return;
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    const int t_pe_3 = roc_shmem_team_my_pe(team_3s), t_pe_2 = roc_shmem_team_my_pe(team_2s);
+    const int t_pe_3_to_2 = roc_shmem_team_translate_pe(team_3s, t_pe_3, team_2s);
+    const int t_pe_2_to_3 = roc_shmem_team_translate_pe(team_2s, t_pe_2, team_3s);
+    const bool in2 = me % 2 == 0, in3 = me % 3 == 0;
+    EXPECT((t_pe_2 != -1) == in2 && (t_pe_3 != -1) == in3 && (t_pe_2_to_3 != -1) == (in2 && in3) &&
+               (t_pe_3_to_2 != -1) == (in2 && in3),
+           "PE %d: t_pe_2=%d t_pe_3=%d t_pe_3_to_2=%d t_pe_2_to_3=%d", me, t_pe_2, t_pe_3, t_pe_3_to_2,
+           t_pe_2_to_3);
+    if (in2) EXPECT(t_pe_2 == me / 2, "PE %d is member %d of team_2s", me, t_pe_2);
+    if (in3) EXPECT(t_pe_3 == me / 3, "PE %d is member %d of team_3s", me, t_pe_3);
+    if (in2 && in3)
+      EXPECT(t_pe_3_to_2 == me / 2 && t_pe_2_to_3 == me / 3, "PE %d translates to %d and %d", me,
+             t_pe_3_to_2, t_pe_2_to_3);
+  }
+  roc_shmemx_set_pe(0);
+  const int N = 1000, members = (npes - 1) / 3 + 1;
+  Sym<int> src(N), dst(N);
+  for (int me = 0; me < npes; ++me) {
+    std::vector<int> v(N);
+    for (int i = 0; i < N; ++i) v[i] = (me + 1) * 1000 + i;
+    src.store(me, v);
+    dst.fill(me, -7);
+  }
+  roc_shmem_ctx_int_sum_to_all(ROC_SHMEM_CTX_DEFAULT, team_3s, dst.ptr, src.ptr, N);
+  for (int me = 0; me < npes; ++me) {
+    std::vector<int> got = dst.load(me);
+    for (int i = 0; i < N; ++i) {
+      int want = -7;
+      if (me % 3 == 0) {
+        want = 0;
+        for (int k = 0; k < members; ++k) want += (3 * k + 1) * 1000 + i;
+      }
+      EXPECT(got[i] == want, "sum over team_3s: PE %d [%d] = %d, expected %d", me, i, got[i], want);
+    }
+    dst.fill(me, -7);
+  }
+  // root = last member of the team
+  roc_shmem_ctx_int_broadcast(ROC_SHMEM_CTX_DEFAULT, team_3s, dst.ptr, src.ptr, N, members - 1);
+  for (int me = 0; me < npes; ++me) {
+    std::vector<int> got = dst.load(me);
+    const int root_world = 3 * (members - 1);
+    for (int i = 0; i < N; ++i) {
+      const int want = (me % 3 == 0 && me != root_world) ? (root_world + 1) * 1000 + i : -7;
+      EXPECT(got[i] == want, "broadcast over team_3s: PE %d [%d] = %d, expected %d", me, i, got[i], want);
+    }
+  }
+  roc_shmem_team_destroy(team_3s);
+  roc_shmem_team_destroy(team_2s);
+}
+
+// clients/sos_tests/barrier.cpp:92-103: thirty barrier_all calls in a row.
+static void barrier_loop() {
+  current_case = "barrier.cpp";
+  for (int j = 0; j < 30; ++j) roc_shmem_barrier_all();
+  EXPECT(roc_shmemx_take_status() == 0, "status word raised by thirty barriers");
+}
+
+// clients/sos_tests/shmem_test.cpp:38-75: every PE puts mype + 1 into wait_vars[mype] of every PE;
+// each PE then polls the array with roc_shmem_long_test(!= 0) until it has seen npes messages,
+// checks wait_vars[who] == who + 1 and clears the entry.
+static void shmem_test_any() {
+  current_case = "shmem_test.cpp";
+  Sym<long> wait_vars(npes);
+  for (int me = 0; me < npes; ++me) wait_vars.fill(me, 0);
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    for (int i = 0; i < npes; ++i) roc_shmem_long_p(&wait_vars.ptr[me], me + 1, i);
+  }
+  for (int me = 0; me < npes; ++me) {
+    roc_shmemx_set_pe(me);
+    int nrecv = 0, idx = 0, polls = 0;
+    while (nrecv < npes && polls < 100 * npes) {
+      ++polls;
+      if (!roc_shmem_long_test(&wait_vars.ptr[idx], ROC_SHMEM_CMP_NE, 0)) {
+        idx = (idx + 1) % npes;
+        continue;
+      }
+      const long got = roc_shmem_long_g(&wait_vars.ptr[idx], me);
+      EXPECT(got == idx + 1, "PE %d: wait_vars[%d] = %ld, expected %d", me, idx, got, idx + 1);
+      roc_shmem_long_p(&wait_vars.ptr[idx], 0, me);
+      ++nrecv;
+    }
+    EXPECT(nrecv == npes, "PE %d saw %d of %d messages", me, nrecv, npes);
+  }
+  roc_shmemx_set_pe(0);
+}
+
 int main() {
   if (!getenv("ROC_SHMEM_NUM_PES")) setenv("ROC_SHMEM_NUM_PES", "6", 1);
   setenv("ROC_SHMEM_HEAP_SIZE", "134217728", 0);
@@ -824,7 +925,10 @@ int main() {
                {"pi", pi},
                {"many_ctx", many_ctx},
                {"team_b2b_collectives", team_b2b_collectives},
-               {"team_reuse_teams", team_reuse_teams}};
+               {"team_reuse_teams", team_reuse_teams},
+               {"team_translate", team_translate},
+               {"barrier", barrier_loop},
+               {"shmem_test", shmem_test_any}};
   for (auto &c : cases) {
     const int before = failures;
     c.run();
