@@ -15,7 +15,11 @@
  * shmem_team_reduce.cpp:88-101; clients/functional_tests/tester.cpp:149-164;
  * a brute-force scalar fold on small random inputs; and, for floating
  * point, agreement of the in-type fold with the long-double ground truth on
- * exactly representable inputs.
+ * exactly representable inputs.  The team form with a stride that is not a
+ * power of two has no test in the reference (its collectives address members
+ * by a truncated log2 of the stride, library/src/team.cpp:68); it is pinned by
+ * brute-force folds over the members and by agreement with the active-set form
+ * for strides that are powers of two (tests/test_oracle_team_strides.py).
  */
 #include <math.h>
 #include <pthread.h>

@@ -18,7 +18,10 @@
  * clients/sos_tests/put1.cpp, bigput.cpp:202-263 (Source[i] = i+1),
  * tester.cpp:236-271 and sos_tests/broadcast_active_set.cpp:84-128 (root's dest
  * keeps its old value), tester.cpp:310-334 ((src_pe << 16) + dst_pe pattern),
- * tester.cpp:336-355 (fcollect value = source rank).
+ * tester.cpp:336-355 (fcollect value = source rank).  The team forms with a
+ * stride that is not a power of two have no test in the reference; they are
+ * pinned by moving the blocks by hand in numpy and by agreement with the
+ * active-set forms for powers of two (tests/test_oracle_team_strides.py).
  */
 #include <pthread.h>
 #include <string.h>
