@@ -231,6 +231,36 @@ def bench_putmem(rs, steps, n_pes, msg_bytes_list):
     return res
 
 
+def bench_granularities(rs, steps, n_pes):
+    """putmem / getmem issued per wave and per thread (every wave or lane moves its own message to
+    or from the next PE): GB/s counted as 2*m bytes per message, and messages per second."""
+    total = 256 << 20
+    src = rs.sym_array(total, np.uint8, fill=7)
+    dst = rs.sym_array(total, np.uint8, fill=0)
+    res = {}
+    shapes = [(rs.WAVE, "wave", m) for m in (256, 4096, 65536, 1 << 20)] + \
+             [(rs.THREAD, "thread", m) for m in (8, 256, 4096)]
+    launch = rs.Launch(64, 256)
+    for gran, name, m in shapes:
+        stride = max(m, 256)
+        n_msgs = min(total // stride, 1 << 16)
+        for kind, kname in ((rs.PUT, "putmem"), (rs.GET, "getmem")):
+            def step():
+                rs.roc_shmem_rma(kind, gran, dst, src, m, n_msgs, stride, stride, 1, launch)
+
+            step()
+            rs.synchronize()
+            ms = event_time_ms(rs, step, steps) / steps
+            res["%s_%s_%d" % (kname, name, m)] = {
+                "GBps": round(2.0 * n_pes * m * n_msgs / ms / 1e6, 1), "ms": round(ms, 4),
+                "calls_per_pe": n_msgs, "Mmsgs_per_s": round(n_pes * n_msgs / ms / 1e3, 1)}
+    if rs.take_status():
+        raise RuntimeError("device status word raised")
+    src.free()
+    dst.free()
+    return res
+
+
 def bench_small_ops(rs, n_pes, n_ops, wgs_total, wg_size, slice_bytes, seed):
     """10 M 8-byte puts (unique targets, lower half) and int64 fetch-adds (upper half)."""
     rng = np.random.default_rng(seed)
@@ -450,6 +480,8 @@ def main():
                          "plain wg putmem copy of known size (2 GiB read + 2 GiB written), nothing else")
     ap.add_argument("--small-ops", action="store_true",
                     help="for rocprofv3 --pmc: the 10 M-operation streams and the consumer pass, nothing else")
+    ap.add_argument("--granularities", action="store_true",
+                    help="putmem / getmem per wave and per thread, nothing else")
     ap.add_argument("--collectives", action="store_true",
                     help="for rocprofv3: broadcast, alltoall and fcollect over 16 slices x 64 MiB, nothing else")
     ap.add_argument("--alignment", action="store_true",
@@ -468,6 +500,12 @@ def main():
         out = bench_small_ops(rs, 16, 10_000_000, 1024, 256, 64 << 20, seed=4)
         rs.roc_shmem_finalize()
         print(json.dumps({"small_ops_16x64MiB_1024wg_x256": out}))
+        return
+    if args.granularities:
+        rs.roc_shmem_init(8, 1 << 30, 64, 1024)
+        out = bench_granularities(rs, 5, 8)
+        rs.roc_shmem_finalize()
+        print(json.dumps({"putmem_getmem_per_wave_and_thread_8pe": out}))
         return
     if args.collectives:
         rs.roc_shmem_init(16, 256 << 20, 64, 1024)
@@ -500,6 +538,7 @@ def main():
         extra["to_all_bf16_sum_8x2^26"] = {k: v for k, v in bench_to_all(
             rs, oracle, max(args.steps // 2, 3), 2, rs.BF16, n_pes, n, seed=3).items() if k != "cpu"}
         extra["putmem_wg_8pe"] = bench_putmem(rs, 5, n_pes, [8, 4096, 65536, 1 << 20, 64 << 20])
+        extra["putmem_getmem_per_wave_and_thread_8pe"] = bench_granularities(rs, 5, n_pes)
     rs.roc_shmem_finalize()
 
     if not args.quick:
