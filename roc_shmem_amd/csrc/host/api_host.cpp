@@ -225,19 +225,40 @@ void *remote_of(host::Runtime *rt, const void *sym, int pe, const char *fn) {
   }
   return p;
 }
-// Launch shape of host-initiated collectives: one workgroup per CU, spread over
-// as many contexts as the library has pSync slices for.
-rsm_launch_t collective_launch(host::Runtime *rt, size_t bytes) {
+// Launch shape of host-initiated collectives, from sweeps over 4, 8 and 16 PEs and 256 KiB to
+// 256 MiB per PE: one workgroup below 512 KiB (launch and barriers dominate), 16 small ones up
+// to 8 MiB, and for what streams a workgroup of 1024 lanes per CU for reductions (which read as
+// much as they write) or per second CU for a broadcast (which almost only writes).  Never more
+// workgroups per PE than the library has contexts (pSync slices) for.  `members` PEs take part;
+// the grid has workgroups for every PE, and those of the others return at once.
+rsm_launch_t collective_launch(host::Runtime *rt, size_t bytes, bool broadcast, int members) {
   rsm_launch_t l;
-  int per_pe = 256 / rt->num_pes();
-  if (per_pe < 1) per_pe = 1;
+  const int pes = members < 1 ? 1 : members;
+  int per_pe, wg_size;
+  if (bytes < (512u << 10)) {
+    per_pe = 1, wg_size = 512;
+  } else if (bytes < (8u << 20)) {
+    per_pe = 16, wg_size = 512;
+  } else if (broadcast) {
+    per_pe = 128 / pes, wg_size = 1024;
+  } else {
+    per_pe = 256 / pes, wg_size = bytes < (32u << 20) ? 512 : 1024;
+  }
+  if (per_pe * rt->num_pes() > 2048) per_pe = 2048 / rt->num_pes();
   if (per_pe > rt->options().num_blocks) per_pe = rt->options().num_blocks;
-  if (bytes < (1u << 20)) per_pe = 1;
+  if (per_pe < 1) per_pe = 1;
   l.wgs_per_pe = per_pe;
-  l.wg_size = 512;
+  l.wg_size = wg_size;
   l.tile = 0;
   l.stream = nullptr;
   return l;
+}
+size_t reduce_elem_size(int dtype) {
+  switch (dtype) {
+    case RSM_SHORT: case RSM_BF16: return 2;
+    case RSM_INT: case RSM_FLOAT: return 4;
+    default: return 8;
+  }
 }
 }  // namespace
 
@@ -330,7 +351,8 @@ void to_all(int dtype, int op, void *dest, const void *source, int nreduce, int 
   HOST_LOCKED;
   if (nreduce <= 0) return;
   host::Runtime *rt = runtime_or_die("roc_shmem_to_all");
-  rsm_launch_t l = collective_launch(rt, static_cast<size_t>(nreduce) * 4);
+  rsm_launch_t l = collective_launch(rt, static_cast<size_t>(nreduce) * reduce_elem_size(dtype),
+                                     false, pe_size);
   if (rsm_to_all(dtype, op, remote_of(rt, dest, 0, "roc_shmem_to_all"),
                  remote_of(rt, source, 0, "roc_shmem_to_all"), static_cast<size_t>(nreduce),
                  pe_start, log_pe_stride, pe_size, nullptr, host_psync(rt), &l))
@@ -342,7 +364,8 @@ void to_all_team(int dtype, int op, roc_shmem_team_t team, void *dest, const voi
                  int nreduce) {
   if (nreduce <= 0 || team == ROC_SHMEM_TEAM_INVALID) return;
   host::Runtime *rt = runtime_or_die("roc_shmem_to_all");
-  rsm_launch_t l = collective_launch(rt, static_cast<size_t>(nreduce) * 4);
+  rsm_launch_t l = collective_launch(rt, static_cast<size_t>(nreduce) * reduce_elem_size(dtype),
+                                     false, roc_shmem_team_n_pes(team));
   if (rsm_to_all_team(dtype, op, reinterpret_cast<uint64_t>(team),
                       remote_of(rt, dest, 0, "roc_shmem_to_all"),
                       remote_of(rt, source, 0, "roc_shmem_to_all"),
@@ -356,7 +379,7 @@ void broadcast(size_t elem_size, void *dest, const void *source, int nelem, int 
   HOST_LOCKED;
   if (nelem <= 0) return;
   host::Runtime *rt = runtime_or_die("roc_shmem_broadcast");
-  rsm_launch_t l = collective_launch(rt, static_cast<size_t>(nelem) * elem_size);
+  rsm_launch_t l = collective_launch(rt, static_cast<size_t>(nelem) * elem_size, true, pe_size);
   if (rsm_broadcast(elem_size, remote_of(rt, dest, 0, "roc_shmem_broadcast"),
                     remote_of(rt, source, 0, "roc_shmem_broadcast"), static_cast<size_t>(nelem),
                     pe_root, pe_start, log_pe_stride, pe_size, host_psync(rt), &l))
@@ -368,7 +391,8 @@ void broadcast_team(size_t elem_size, roc_shmem_team_t team, void *dest, const v
                     int nelem, int pe_root) {
   if (nelem <= 0 || team == ROC_SHMEM_TEAM_INVALID) return;
   host::Runtime *rt = runtime_or_die("roc_shmem_broadcast");
-  rsm_launch_t l = collective_launch(rt, static_cast<size_t>(nelem) * elem_size);
+  rsm_launch_t l = collective_launch(rt, static_cast<size_t>(nelem) * elem_size, true,
+                                     roc_shmem_team_n_pes(team));
   if (rsm_broadcast_team(elem_size, reinterpret_cast<uint64_t>(team),
                          remote_of(rt, dest, 0, "roc_shmem_broadcast"),
                          remote_of(rt, source, 0, "roc_shmem_broadcast"),
