@@ -132,10 +132,61 @@ def exchange_case(d, case):
     return what
 
 
+def team_case(d, case):
+    """One collective over a team of any stride (roc_shmem_team_split_strided takes any)."""
+    pe_stride = d.between(1, 8)
+    pe_size = d.between(1, (N_PES - 1) // pe_stride + 2)
+    pe_start = d.between(0, N_PES - (pe_size - 1) * pe_stride)
+    which = d.pick(["to_all", "broadcast", "alltoall", "fcollect"])
+    wgs, wg_size = d.pick([1, 2, 4]), d.pick([64, 256, 1024])
+    what = "team (%d,%d,%d) %s wgs=%d wg=%d" % (pe_start, pe_stride, pe_size, which, wgs, wg_size)
+    rc, team = rs.roc_shmem_team_split_strided(rs.roc_shmem_team_world(), pe_start, pe_stride, pe_size)
+    assert rc == 0 and team, what + ": split refused"
+    kw = dict(pe_size=pe_size, pe_stride=pe_stride)
+    try:
+        if which == "to_all":
+            dtype, op = d.pick(to_all.INT_TYPES), d.pick(to_all.INT_OPS)
+            es = np.dtype(rs.NP_DTYPE[dtype]).itemsize
+            n = d.size((1, 300), (300, 20000), (20000, 200000))
+            tile = d.pick([0, 0, d.between(max(1, n // 100), max(2, n))])
+            what += " dtype=%d op=%d n=%d tile=%d" % (dtype, op, n, tile)
+            src, dst, heap = coll.setup(N_PES, n * es, n * es + 32, seed=case)
+            rs.roc_shmem_team_to_all(dtype, op, team, dst, src, n, rs.Launch(wgs, wg_size, tile))
+            rs.synchronize()
+            oracle.to_all(heap, dtype, op, n * es, 0, n, pe_start, **kw)
+            coll.compare(N_PES, dst, heap, n * es, n * es + 32)
+        elif which == "broadcast":
+            nbytes = d.size((1, 300), (300, 70000), (70000, 2 << 20))
+            root = d.between(0, pe_size)
+            what += " n=%d root=%d" % (nbytes, root)
+            src, dst, heap = coll.setup(N_PES, nbytes, nbytes + 32, seed=case)
+            rs.roc_shmem_team_broadcast(1, team, dst, src, nbytes, root, rs.Launch(wgs, wg_size))
+            rs.synchronize()
+            oracle.broadcast(heap, nbytes, 0, nbytes, root, pe_start, **kw)
+            coll.compare(N_PES, dst, heap, nbytes, nbytes + 32)
+        else:
+            elem_size, nelem = d.pick([1, 2, 4, 8]), d.size((1, 100), (100, 30000))
+            block = elem_size * nelem
+            what += " elem=%d nelem=%d" % (elem_size, nelem)
+            src_bytes = block * pe_size if which == "alltoall" else block
+            src, dst, heap = coll.setup(N_PES, src_bytes, block * pe_size + 32, seed=case)
+            call = rs.roc_shmem_alltoall if which == "alltoall" else rs.roc_shmem_fcollect
+            call(elem_size, team, dst, src, nelem, rs.Launch(wgs, wg_size))
+            rs.synchronize()
+            getattr(oracle, which)(heap, src_bytes, 0, block, pe_start, **kw)
+            coll.compare(N_PES, dst, heap, src_bytes, block * pe_size + 32)
+    except AssertionError as e:
+        raise AssertionError("%s: %s" % (what, e))
+    src.free()
+    dst.free()
+    rs.roc_shmem_team_destroy(team)
+    return what
+
+
 @pytest.mark.parametrize("seed,ncases", [(101, 120), (202, 120)])
 def test_random_shapes_match_the_oracle(seed, ncases):
     d = Draw(seed)
-    makers = [reduction_case, reduction_case, rma_case, broadcast_case, exchange_case]
+    makers = [reduction_case, reduction_case, rma_case, broadcast_case, exchange_case, team_case]
     # the allocator never merges freed blocks, so the library is brought up afresh every 30 cases
     for first in range(0, ncases, 30):
         with runtime(N_PES, heap_size=256 << 20):
