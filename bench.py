@@ -351,6 +351,45 @@ def bench_small_ops(rs, n_pes, n_ops, wgs_total, wg_size, slice_bytes, seed):
     return res
 
 
+def bench_amo_kinds(rs, n_pes, n_ops, wgs_total, wg_size, slice_bytes, seed):
+    """One stream of n_ops operations per kind, uniformly random (PE, word) targets: M ops/s."""
+    rng = np.random.default_rng(seed)
+    words = slice_bytes // 8
+    mem = rs.sym_array(words, np.int64, fill=0)
+    ops = np.zeros(n_ops, rs.SMALL_OP_DTYPE)
+    ops["pe"] = rng.integers(0, n_pes, n_ops)
+    ops["offset"] = mem.offset + rng.integers(0, words // 2, n_ops) * 8
+    ops["value"] = rng.integers(1, 1000, n_ops)
+    launch = rs.Launch(wgs_total // n_pes, wg_size)
+    res = {}
+    kinds = [("p64", rs.OP_P64), ("p32", rs.OP_P32), ("fetch_add64", rs.OP_FADD64), ("fetch_add32", rs.OP_FADD32),
+             ("add64", rs.OP_ADD64), ("fetch_inc64", rs.OP_FINC64), ("inc64", rs.OP_INC64),
+             ("compare_swap64", rs.OP_CSWAP64), ("fetch64", rs.OP_FETCH64), ("set64", rs.OP_SET64),
+             ("swap64", rs.OP_SWAP64), ("fetch_and64", rs.OP_FAND64), ("fetch_or64", rs.OP_FOR64),
+             ("fetch_xor64", rs.OP_FXOR64), ("getmem8_nbi", rs.OP_GETMEM), ("putmem8_nbi", rs.OP_PUTMEM)]
+    for name, kind in kinds:
+        ops["kind"] = kind
+        if kind in (rs.OP_GETMEM, rs.OP_PUTMEM):
+            # `value` names the local buffer: a word of the upper half, one per operation
+            ops["value"] = mem.offset + (words // 2 + np.arange(n_ops) % (words // 2)) * 8
+            ops["aux"] = 8
+        dev = rs.device_array(ops)
+
+        def step():
+            rs.roc_shmem_small_ops(dev, n_ops, None, launch)
+
+        step()
+        rs.synchronize()
+        ms = event_time_ms(rs, step, 3) / 3
+        res[name] = {"Mops_per_s": round(n_ops / ms / 1e3, 1), "ms": round(ms, 4)}
+        dev.free()
+    status = rs.take_status()
+    if status:
+        raise RuntimeError("device status word raised: %d" % status)
+    mem.free()
+    return res
+
+
 def bench_small_collectives(rs, n_pes, n, calls):
     """A launch-bound sequence: `calls` int64 sum_to_all of `n` elements back to back, issued call by
     call and as one recorded graph.  Microseconds per collective."""
@@ -482,6 +521,8 @@ def main():
                     help="for rocprofv3 --pmc: the 10 M-operation streams and the consumer pass, nothing else")
     ap.add_argument("--granularities", action="store_true",
                     help="putmem / getmem per wave and per thread, nothing else")
+    ap.add_argument("--amo-kinds", action="store_true",
+                    help="10 M operations of every small-operation kind, random targets, nothing else")
     ap.add_argument("--collectives", action="store_true",
                     help="for rocprofv3: broadcast, alltoall and fcollect over 16 slices x 64 MiB, nothing else")
     ap.add_argument("--alignment", action="store_true",
@@ -500,6 +541,12 @@ def main():
         out = bench_small_ops(rs, 16, 10_000_000, 1024, 256, 64 << 20, seed=4)
         rs.roc_shmem_finalize()
         print(json.dumps({"small_ops_16x64MiB_1024wg_x256": out}))
+        return
+    if args.amo_kinds:
+        rs.roc_shmem_init(16, 256 << 20, 64, 1024)
+        out = bench_amo_kinds(rs, 16, 10_000_000, 1024, 256, 64 << 20, seed=5)
+        rs.roc_shmem_finalize()
+        print(json.dumps({"small_op_kinds_16x64MiB_1024wg_x256": out}))
         return
     if args.granularities:
         rs.roc_shmem_init(8, 1 << 30, 64, 1024)
