@@ -225,24 +225,31 @@ void *remote_of(host::Runtime *rt, const void *sym, int pe, const char *fn) {
   }
   return p;
 }
-// Launch shape of host-initiated collectives, from sweeps over 4, 8 and 16 PEs and 256 KiB to
-// 256 MiB per PE: one workgroup below 512 KiB (launch and barriers dominate), 16 small ones up
-// to 8 MiB, and for what streams a workgroup of 1024 lanes per CU for reductions (which read as
-// much as they write) or per second CU for a broadcast (which almost only writes).  Never more
-// workgroups per PE than the library has contexts (pSync slices) for.  `members` PEs take part;
-// the grid has workgroups for every PE, and those of the others return at once.
+// Launch shape of host-initiated collectives, from sweeps over 4, 8 and 16 PEs and 64 KiB to
+// 256 MiB per PE.  Reductions read as much as they write and every workgroup walks all members:
+// about 64 KiB of each member's array per workgroup, at least 4 workgroups from 128 KiB up, at
+// most one per CU, 1024 lanes once the arrays stream (32 MiB).  A broadcast almost only writes:
+// one workgroup below 512 KiB, 16 up to 8 MiB, then one of 1024 lanes per second CU.  Never
+// more workgroups per PE than the library has contexts (pSync slices) for.  `members` PEs take
+// part; the grid has workgroups for every PE, and those of the others return at once.
 rsm_launch_t collective_launch(host::Runtime *rt, size_t bytes, bool broadcast, int members) {
   rsm_launch_t l;
   const int pes = members < 1 ? 1 : members;
   int per_pe, wg_size;
-  if (bytes < (512u << 10)) {
-    per_pe = 1, wg_size = 512;
-  } else if (bytes < (8u << 20)) {
-    per_pe = 16, wg_size = 512;
-  } else if (broadcast) {
-    per_pe = 128 / pes, wg_size = 1024;
+  if (broadcast) {
+    if (bytes < (512u << 10)) {
+      per_pe = 1, wg_size = 512;
+    } else if (bytes < (8u << 20)) {
+      per_pe = 16, wg_size = 512;
+    } else {
+      per_pe = 128 / pes, wg_size = 1024;
+    }
   } else {
-    per_pe = 256 / pes, wg_size = bytes < (32u << 20) ? 512 : 1024;
+    const size_t want = bytes / (static_cast<size_t>(65536) * pes);
+    per_pe = 1;
+    while (static_cast<size_t>(per_pe) * 2 <= want && per_pe * 2 * pes <= 256) per_pe *= 2;
+    if (per_pe < 4 && bytes >= (128u << 10)) per_pe = 4;
+    wg_size = bytes < (32u << 20) ? 512 : 1024;
   }
   if (per_pe * rt->num_pes() > 2048) per_pe = 2048 / rt->num_pes();
   if (per_pe > rt->options().num_blocks) per_pe = rt->options().num_blocks;
