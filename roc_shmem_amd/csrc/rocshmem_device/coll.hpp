@@ -285,7 +285,8 @@ __device__ __forceinline__ void wg_fcollect_bytes(int my_pe, void *dest, const v
 }
 
 // Barrier among the member workgroups (reference: internal_sync,
-// context_ib_device_coll.cpp:67-89).
+// context_ib_device_coll.cpp:67-89).  `psync` is a slice of the team's barrier
+// pool, which only this routine uses.
 __device__ __forceinline__ void wg_sync_members(int my_pe, int pe_start, int pe_stride,
                                                 int pe_size, long *psync) {
   my_pe = uniform(my_pe);
@@ -298,8 +299,7 @@ __device__ __forceinline__ void wg_sync_members(int my_pe, int pe_start, int pe_
     return;
   }
   const int my_idx = member_index(my_pe - pe_start, pe_stride);
-  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, pe_stride, pe_size);
-  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size);
+  wg_epoch_barrier(psync, my_pe, my_idx, pe_start, pe_stride, pe_size);
 }
 
 }  // namespace detail
