@@ -191,7 +191,15 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
 
   // This workgroup takes passes first_pass, first_pass + pass_step, ... of the range.
   const size_t step_bytes = pass_step * pass_bytes;
-  for (size_t b = v_begin * 16 + first_pass * pass_bytes; b < byte_end; b += step_bytes) {
+  const size_t byte_begin = v_begin * 16 + first_pass * pass_bytes;
+  // A short first pass is the only one, and a wave whose every lane lies past
+  // its end has nothing to do in it.  Its accesses would be clipped, but a
+  // clipped access still costs its issue slots: a 4 KiB reduction by one
+  // workgroup of 1024 lanes took 10.4 us against 7.1 us by one of 256, now 8.0.
+  if (byte_begin < byte_end && byte_end - byte_begin < pass_bytes &&
+      uniform((tid & ~63u) * 16u) >= byte_end - byte_begin)
+    return;
+  for (size_t b = byte_begin; b < byte_end; b += step_bytes) {
     const size_t left = byte_end - b;
     const int valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
     Acc acc[U][E];
