@@ -152,8 +152,8 @@ __device__ __forceinline__ void wg_flag_barrier(long *psync, int set, int my_pe,
 // can only satisfy, never spoil, the wait of one still in call e, and nothing
 // has to be cleared between calls.  Every member must call it the same number
 // of times on a slice, which a collective guarantees; the host zeroes the pool
-// when the team is made.  Two flag barriers in a row take 1.7-2.2 us for 4
-// PEs, this one call half of that.
+// when the team is made.  Two flag barriers in a row took 1.7-2.4 us for 4
+// PEs (the figure differs from card to card), this one call 1.1-1.5 us.
 constexpr int kEpochSlot = kSyncSlots - 1;   // kMaxPes arrival slots fit below it
 
 __device__ __forceinline__ void wg_epoch_barrier(long *psync, int my_pe, int my_idx,
