@@ -162,10 +162,10 @@ __device__ __forceinline__ void wg_epoch_barrier(long *psync, int my_pe, int my_
   const uint32_t tid = flat_thread_id();
   const uint32_t nthr = flat_block_size();
   unsigned long long *own = reinterpret_cast<unsigned long long *>(psync);
+  unsigned long long epoch = 0;
   if (tid < static_cast<uint32_t>(n_pes)) {
     fence_release_agent();
-    const unsigned long long epoch =
-        __hip_atomic_load(own + kEpochSlot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+    epoch = __hip_atomic_load(own + kEpochSlot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
     for (uint32_t t = tid; t < static_cast<uint32_t>(n_pes); t += nthr) {
       int peer = pe_start + static_cast<int>(t) * pe_stride;
       unsigned long long *slot =
@@ -180,11 +180,8 @@ __device__ __forceinline__ void wg_epoch_barrier(long *psync, int my_pe, int my_
   // Behind the workgroup barrier every lane that reads the count has read it,
   // so lane 0 may advance it; the next call starts with a workgroup barrier,
   // behind which all lanes see the new count.
-  if (tid == 0) {
-    const unsigned long long done =
-        __hip_atomic_load(own + kEpochSlot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
-    __hip_atomic_store(own + kEpochSlot, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
+  if (tid == 0)
+    __hip_atomic_store(own + kEpochSlot, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace detail
