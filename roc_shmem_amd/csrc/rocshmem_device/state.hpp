@@ -111,8 +111,10 @@ struct DeviceState {
 // program built against other headers than the library it loads would index
 // ctx_table with the wrong stride and follow wild pointers, so every unit hands
 // its fingerprint to the library, which refuses to initialise on a mismatch.
-// Bump kStateRevision when a layout changes without changing a size.
-constexpr uint32_t kStateRevision = 2;
+// Bump kStateRevision when a layout changes without changing a size, or when
+// units must agree on how they use shared memory (3: the barrier pool holds
+// call counts, not flags that are reset).
+constexpr uint32_t kStateRevision = 3;
 constexpr uint32_t kStateLayout =
     (kStateRevision * 0x01000193u) ^
     static_cast<uint32_t>(sizeof(DeviceState) | (sizeof(DeviceCtx) << 8) | (sizeof(Team) << 16) |
