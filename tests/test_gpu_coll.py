@@ -203,3 +203,33 @@ def test_barrier_all_many_rounds():
         rs.roc_shmem_wg_barrier_all(200, rs.Launch(4, 64))
         rs.synchronize()
         assert rs.take_status() == 0
+
+
+def test_barriers_keep_count_across_launches_of_different_shapes():
+    # sync_all / barrier_all count their calls per context block in the team's barrier pool and
+    # never reset a slot: launches with other numbers of workgroups and rounds, with collectives on
+    # the world team and on a sub-team in between, must leave every block's count in step on all PEs
+    # (a count out of step ends in a wait that gives up and raises the status word).
+    import time
+    n_pes = 8
+    with runtime(n_pes, num_blocks=16):
+        world = rs.roc_shmem_team_world()
+        rc, evens = rs.roc_shmem_team_split_strided(world, 0, 2, 4)
+        assert rc == 0
+        src, dst, heap = setup(n_pes, 4096, 4096, seed=3)
+        t0 = time.perf_counter()
+        for rounds, wgs, wg_size in ((3, 1, 64), (2, 3, 256), (5, 2, 1024), (1, 16, 64), (4, 1, 512), (7, 16, 128)):
+            rs.roc_shmem_wg_barrier_all(rounds, rs.Launch(wgs, wg_size))
+            rs.roc_shmem_team_broadcast(1, evens, dst, src, 4096, 1, rs.Launch(2, 128))
+            rs.roc_shmem_team_to_all(rs.INT, rs.SUM, world, dst, src, 1024, rs.Launch(wgs, wg_size))
+        rs.synchronize()
+        assert rs.take_status() == 0
+        assert time.perf_counter() - t0 < 1.0, "a barrier waited for its time limit"
+        rs.roc_shmem_team_destroy(evens)
+        # a new team gets a cleared pool, wherever the allocator puts it
+        rc, again = rs.roc_shmem_team_split_strided(world, 1, 2, 4)
+        assert rc == 0
+        rs.roc_shmem_team_broadcast(1, again, dst, src, 4096, 0, rs.Launch(1, 64))
+        rs.synchronize()
+        assert rs.take_status() == 0
+        rs.roc_shmem_team_destroy(again)
