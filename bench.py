@@ -390,6 +390,32 @@ def bench_amo_kinds(rs, n_pes, n_ops, wgs_total, wg_size, slice_bytes, seed):
     return res
 
 
+def bench_small_latencies(rs, n_pes):
+    """Fixed cost of a collective: 4 KiB per PE, one workgroup of 256 lanes per PE, back-to-back
+    launches, microseconds per call."""
+    src = rs.sym_array(1 << 16, np.uint8, fill=1)
+    dst = rs.sym_array(1 << 16, np.uint8, fill=0)
+    psync = rs.sym_array(rs.ROC_SHMEM_REDUCE_SYNC_SIZE, np.int64, fill=0)
+    world = rs.roc_shmem_team_world()
+    launch, nbytes, out = rs.Launch(1, 256), 4096, {}
+    calls = {
+        "int_sum_to_all": lambda: rs.roc_shmem_to_all(rs.INT, rs.SUM, dst, src, nbytes // 4, 0, 0, n_pes, None,
+                                                      psync, launch),
+        "broadcast": lambda: rs.roc_shmem_team_broadcast(1, world, dst, src, nbytes, 0, launch),
+        "alltoall": lambda: rs.roc_shmem_alltoall(1, world, dst, src, nbytes // n_pes, launch),
+        "fcollect": lambda: rs.roc_shmem_fcollect(1, world, dst, src, nbytes // n_pes, launch),
+    }
+    for name, fn in calls.items():
+        fn()
+        rs.synchronize()
+        out[name + "_us"] = round(event_time_ms(rs, fn, 50) / 50 * 1e3, 2)
+    if rs.take_status():
+        raise RuntimeError("device status word raised")
+    for a in (psync, dst, src):
+        a.free()
+    return out
+
+
 def bench_small_collectives(rs, n_pes, n, calls):
     """A launch-bound sequence: `calls` int64 sum_to_all of `n` elements back to back, issued call by
     call and as one recorded graph.  Microseconds per collective."""
@@ -586,6 +612,7 @@ def main():
             rs, oracle, max(args.steps // 2, 3), 2, rs.BF16, n_pes, n, seed=3).items() if k != "cpu"}
         extra["putmem_wg_8pe"] = bench_putmem(rs, 5, n_pes, [8, 4096, 65536, 1 << 20, 64 << 20])
         extra["putmem_getmem_per_wave_and_thread_8pe"] = bench_granularities(rs, 5, n_pes)
+        extra["collectives_4KiB_8pe_one_wg_of_256"] = bench_small_latencies(rs, n_pes)
     rs.roc_shmem_finalize()
 
     if not args.quick:
