@@ -243,10 +243,11 @@ def bench_granularities(rs, steps, n_pes):
     res = {}
     shapes = [(rs.WAVE, "wave", m) for m in (256, 4096, 65536, 1 << 20)] + \
              [(rs.THREAD, "thread", m) for m in (8, 256, 4096)]
-    launch = rs.Launch(64, 256)
     for gran, name, m in shapes:
         stride = max(m, 256)
         n_msgs = min(total // stride, 1 << 16)
+        # short per-wave messages are bound by load latency: sixteen waves per workgroup
+        launch = rs.Launch(64, 1024) if gran == rs.WAVE and m <= 1024 else rs.Launch(64, 256)
         for kind, kname in ((rs.PUT, "putmem"), (rs.GET, "getmem")):
             def step():
                 rs.roc_shmem_rma(kind, gran, dst, src, m, n_msgs, stride, stride, 1, launch)
