@@ -75,6 +75,73 @@ __device__ __forceinline__ uint64_t heap_offset(uint64_t addr, uint64_t size, in
 // Retire everything ring `ctx` has published.  Called by all 64 lanes of one
 // wave.  `target` is the arena operations are executed against (nullptr: check
 // and complete only).
+// What one 64-byte entry says, and whether it is well formed.  `c` is the
+// entry's running number in its ring; w0..w7 are its eight 64-bit words.
+struct DecodedEntry {
+  bool ok, is_atomic, is_write, is_read, inl, wants_completion;
+  uint32_t head, opcode, size;
+  uint64_t laddr, roff;
+};
+
+__device__ __forceinline__ DecodedEntry decode_entry(const SqRing &ring, uint32_t c,
+                                                     uint64_t ret_lo, uint64_t ret_hi, uint64_t w0,
+                                                     uint64_t w1, uint64_t w2, uint64_t w3,
+                                                     uint64_t w4, uint64_t w5, uint64_t w6,
+                                                     uint64_t w7) {
+  const uint32_t head = static_cast<uint32_t>(w0);            // bytes 0..3
+  const uint32_t opcode = head >> 24;
+  const uint32_t index = __builtin_bswap16(static_cast<uint16_t>(head >> 8));
+  const uint32_t qpn_ds = static_cast<uint32_t>(w0 >> 32);    // bytes 4..7
+  const uint32_t ds = qpn_ds >> 24;
+  const uint32_t fm_ce_se = static_cast<uint32_t>(w1 >> 24) & 0xffu;  // byte 11
+  const uint64_t raddr = __builtin_bswap64(w2);
+  const uint32_t rkey = static_cast<uint32_t>(w3);
+
+  const bool is_atomic = opcode == kOpcodeAtomicFa || opcode == kOpcodeAtomicCs;
+  const bool is_write = opcode == kOpcodeRdmaWrite;
+  const bool is_read = opcode == kOpcodeRdmaRead;
+  bool ok = (head & 0xffu) == 0 && index == (c & 0xffffu) &&
+            (qpn_ds & 0xffffffu) == ring.ctrl_qp_sq && (is_atomic || is_write || is_read) &&
+            ds == (is_atomic ? 4u : 3u);
+
+  uint32_t size = 0;
+  bool inl = false;
+  uint64_t laddr = 0;
+  if (is_atomic) {
+    size = 8;
+    ok = ok && (raddr & 7u) == 0 && __builtin_bswap32(static_cast<uint32_t>(w6)) == 8u &&
+         static_cast<uint32_t>(w6 >> 32) == ring.atomic_lkey;
+    laddr = __builtin_bswap64(w7);
+    ok = ok && (laddr & 7u) == 0 && laddr >= ret_lo && laddr < ret_hi;
+  } else {
+    const uint32_t count = __builtin_bswap32(static_cast<uint32_t>(w4));
+    inl = (count & 0x80000000u) != 0;
+    size = inl ? (count & 0x3ffu) : count;
+    if (inl) {
+      ok = ok && is_write && size <= 12u;   // what fits the third segment
+    } else {
+      ok = ok && static_cast<uint32_t>(w4 >> 32) == ring.lkey;
+      laddr = __builtin_bswap64(w5);
+    }
+  }
+  int dest_pe = 0;
+  const uint64_t roff = ok ? heap_offset(raddr, size, &dest_pe) : ~0ull;
+  ok = ok && roff != ~0ull && rkey == ring.rkey_by_pe[dest_pe];
+  DecodedEntry d;
+  d.ok = ok;
+  d.is_atomic = is_atomic;
+  d.is_write = is_write;
+  d.is_read = is_read;
+  d.inl = inl;
+  d.wants_completion = fm_ce_se == kCqUpdate;
+  d.head = head;
+  d.opcode = opcode;
+  d.size = size;
+  d.laddr = laddr;
+  d.roff = roff;
+  return d;
+}
+
 __device__ __forceinline__ void consume_ring(const DeviceCtx *ctx, char *target,
                                              ConsumeTotals *totals) {
   const SqRing &ring = ctx->ring;
@@ -95,6 +162,57 @@ __device__ __forceinline__ void consume_ring(const DeviceCtx *ctx, char *target,
     c = published - ring.max_nwqe;
   }
 
+  if (target == nullptr) {
+    // Check and complete only: nothing takes effect, so the order of the entries
+    // does not matter and every lane takes one of its own, 64 per round (one
+    // entry at a time, a pass over 1 Mi entries in 1024 rings took 1.45 ms).
+    typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+    const uint32_t todo = published - c;
+    unsigned long long lane_bytes = 0;
+    for (uint32_t done = 0; done < todo; done += 64) {
+      const uint32_t ci = c + done + lane;
+      const bool active = done + lane < todo;
+      uint64_t w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (active) {
+        const u64x2 *slot = reinterpret_cast<const u64x2 *>(ring.sq + 8ull * (ci & mask));
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const u64x2 v = slot[q];
+          w[2 * q] = v.x;
+          w[2 * q + 1] = v.y;
+        }
+      }
+      const DecodedEntry d =
+          decode_entry(ring, ci, ret_lo, ret_hi, w[0], w[1], w[2], w[3], w[4], w[5], w[6], w[7]);
+      const bool good = active && d.ok;
+      t.retired += __popcll(__ballot(active));
+      t.rejected += __popcll(__ballot(active && !d.ok));
+      t.atomics += __popcll(__ballot(good && d.is_atomic));
+      t.writes += __popcll(__ballot(good && !d.is_atomic && d.is_write));
+      t.reads += __popcll(__ballot(good && !d.is_atomic && !d.is_write));
+      if (good) lane_bytes += d.size;
+      const bool wants = active && d.wants_completion;
+      const uint64_t wanting = __ballot(wants);
+      if (wants) {
+        const uint32_t number = cq_producer + rank_in_mask(wanting);
+        u64x2 *cqe = reinterpret_cast<u64x2 *>(ring.cq + 8ull * (number & (ring.cq_size - 1)));
+        const uint64_t owner = (number >> ring.cq_log_size) & 1u;
+        const uint64_t last = (static_cast<uint64_t>(ring.ctrl_qp_sq & 0xffffffu) << 8) |
+                              (static_cast<uint64_t>((d.head >> 8) & 0xffffu) << 32) | (owner << 56);
+        cqe[0] = u64x2{0, 0};
+        cqe[1] = u64x2{0, 0};
+        cqe[2] = u64x2{0, 0};
+        cqe[3] = u64x2{0, last};
+      }
+      cq_producer += __popcll(wanting);
+      t.completions += __popcll(wanting);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) lane_bytes += __shfl_xor(lane_bytes, off);
+    t.bytes = lane_bytes;
+    c = published;
+  }
+
   for (; c != published; ++c) {
     // Eight lanes fetch the entry, everybody gets the words.
     const uint64_t *slot = ring.sq + 8ull * (c & mask);
@@ -104,45 +222,10 @@ __device__ __forceinline__ void consume_ring(const DeviceCtx *ctx, char *target,
                    w6 = lane_u64(mine, 6), w7 = lane_u64(mine, 7);
     ++t.retired;
 
-    const uint32_t head = static_cast<uint32_t>(w0);            // bytes 0..3
-    const uint32_t opcode = head >> 24;
-    const uint32_t index = __builtin_bswap16(static_cast<uint16_t>(head >> 8));
-    const uint32_t qpn_ds = static_cast<uint32_t>(w0 >> 32);    // bytes 4..7
-    const uint32_t ds = qpn_ds >> 24;
-    const uint32_t fm_ce_se = static_cast<uint32_t>(w1 >> 24) & 0xffu;  // byte 11
-    const uint64_t raddr = __builtin_bswap64(w2);
-    const uint32_t rkey = static_cast<uint32_t>(w3);
-
-    const bool is_atomic = opcode == kOpcodeAtomicFa || opcode == kOpcodeAtomicCs;
-    const bool is_write = opcode == kOpcodeRdmaWrite;
-    const bool is_read = opcode == kOpcodeRdmaRead;
-    bool ok = (head & 0xffu) == 0 && index == (c & 0xffffu) &&
-              (qpn_ds & 0xffffffu) == ring.ctrl_qp_sq && (is_atomic || is_write || is_read) &&
-              ds == (is_atomic ? 4u : 3u);
-
-    uint32_t size = 0;
-    bool inl = false;
-    uint64_t laddr = 0;
-    if (is_atomic) {
-      size = 8;
-      ok = ok && (raddr & 7u) == 0 && __builtin_bswap32(static_cast<uint32_t>(w6)) == 8u &&
-           static_cast<uint32_t>(w6 >> 32) == ring.atomic_lkey;
-      laddr = __builtin_bswap64(w7);
-      ok = ok && (laddr & 7u) == 0 && laddr >= ret_lo && laddr < ret_hi;
-    } else {
-      const uint32_t count = __builtin_bswap32(static_cast<uint32_t>(w4));
-      inl = (count & 0x80000000u) != 0;
-      size = inl ? (count & 0x3ffu) : count;
-      if (inl) {
-        ok = ok && is_write && size <= 12u;   // what fits the third segment
-      } else {
-        ok = ok && static_cast<uint32_t>(w4 >> 32) == ring.lkey;
-        laddr = __builtin_bswap64(w5);
-      }
-    }
-    int dest_pe = 0;
-    const uint64_t roff = ok ? heap_offset(raddr, size, &dest_pe) : ~0ull;
-    ok = ok && roff != ~0ull && rkey == ring.rkey_by_pe[dest_pe];
+    const DecodedEntry d = decode_entry(ring, c, ret_lo, ret_hi, w0, w1, w2, w3, w4, w5, w6, w7);
+    const bool ok = d.ok, is_atomic = d.is_atomic, is_write = d.is_write, inl = d.inl;
+    const uint32_t head = d.head, opcode = d.opcode, size = d.size;
+    const uint64_t laddr = d.laddr, roff = d.roff;
 
     if (!ok) {
       ++t.rejected;
@@ -197,7 +280,7 @@ __device__ __forceinline__ void consume_ring(const DeviceCtx *ctx, char *target,
       }
     }
 
-    if (fm_ce_se == kCqUpdate) {
+    if (d.wants_completion) {
       uint64_t *cqe = ring.cq + 8ull * (cq_producer & (ring.cq_size - 1));
       if (lane < 8) {
         uint64_t word = 0;
