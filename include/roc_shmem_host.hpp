@@ -190,8 +190,9 @@ inline T from_bits(uint64_t b) {
 // host_templates.hpp:426-487 (an atomic fetch of the calling PE's own copy of the word, compared
 // on the host; wait_until repeats it until the comparison holds); declared for the 13 standard
 // types at library/include/roc_shmem.hpp:1152-1163,1973-2019.  The calling PE is the host's
-// current PE.  Where the reference would spin for ever, the wait gives up after
-// ROC_SHMEM_WAIT_LIMIT_S seconds, prints a message and exits like the library's other fatal errors.
+// current PE.  The reference spins for ever; so does this wait with ROC_SHMEM_WAIT_LIMIT_S=0.
+// With a positive limit (the default is 2 s) it gives up after that many seconds, prints a
+// message and exits like the library's other fatal errors.
 namespace hostx {
 template <typename T>
 inline T own_value(const T *ptr) {
@@ -216,7 +217,8 @@ inline void wait_until(const T *ptr, roc_shmem_cmps cmp, T val) {
   const auto start = std::chrono::steady_clock::now();
   const double limit = wait_limit_seconds();
   while (!compare(cmp, own_value(ptr), val)) {
-    if (std::chrono::duration<double>(std::chrono::steady_clock::now() - start).count() > limit) {
+    if (limit > 0 &&
+        std::chrono::duration<double>(std::chrono::steady_clock::now() - start).count() > limit) {
       fprintf(stderr, "rocshmem: roc_shmem_wait_until: condition not met after %.1f s\n", limit);
       exit(EXIT_FAILURE);
     }

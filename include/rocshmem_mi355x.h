@@ -300,6 +300,11 @@ void rsm_host_alloc_destroy(void *allocator);
 size_t rsm_host_alloc_alloc(void *allocator, size_t request);
 int rsm_host_alloc_free(void *allocator, size_t offset);
 size_t rsm_host_alloc_in_use(void *allocator);
+/* The range check rsm_to_all and rsm_broadcast apply to an active set before they launch
+ * (members pe_start + k * 2^log_pe_stride, k < pe_size, must all be PEs below num_pes;
+ * reference: the PE_start / logPE_stride / PE_size triple of roc_shmem.hpp:837-847).
+ * 1 when the set is acceptable, 0 otherwise. */
+int rsm_host_active_set_in_range(int pe_start, int log_pe_stride, int pe_size, int num_pes);
 
 #ifdef __cplusplus
 }

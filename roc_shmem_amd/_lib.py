@@ -80,6 +80,7 @@ SIGNATURES = {
     "rsm_host_alloc_alloc": (sz, [vp, sz]),
     "rsm_host_alloc_free": (i32, [vp, sz]),
     "rsm_host_alloc_in_use": (sz, [vp]),
+    "rsm_host_active_set_in_range": (i32, [i32, i32, i32, i32]),
 }
 
 _lib = None

@@ -89,6 +89,15 @@ bool check_extent(const void *p, size_t bytes, const char *what) {
   return true;
 }
 
+bool active_set_in_range(int pe_start, int log_pe_stride, int pe_size, int num_pes) {
+  if (num_pes < 1 || pe_start < 0 || pe_start >= num_pes || log_pe_stride < 0 ||
+      log_pe_stride > 30 || pe_size < 1 || pe_size > rocshmem::detail::kMaxPes)
+    return false;
+  if (pe_size == 1) return true;
+  const int64_t last = pe_start + (static_cast<int64_t>(pe_size - 1) << log_pe_stride);
+  return last < num_pes;
+}
+
 int after_launch(const char *what) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(std::string(what) + ": " + hipGetErrorString(e));
@@ -426,6 +435,10 @@ int rsm_sq_rkey(int dest_pe, uint32_t *rkey) {
 }
 
 // ---- host-logic hooks ------------------------------------------------------------
+
+int rsm_host_active_set_in_range(int pe_start, int log_pe_stride, int pe_size, int num_pes) {
+  return rsm::active_set_in_range(pe_start, log_pe_stride, pe_size, num_pes) ? 1 : 0;
+}
 
 void *rsm_host_alloc_create(size_t heap_bytes) {
   RSM_ENTRY;

@@ -39,6 +39,12 @@ bool check_symmetric(const void *p, const char *what, bool allow_null = false);
 // true for addresses outside the arena, which cannot be judged here.
 bool check_extent(const void *p, size_t bytes, const char *what);
 
+// Members pe_start + k * 2^log_pe_stride, k < pe_size, of an active set all exist among
+// `num_pes` PEs and the set has at most kMaxPes members.  Pure host arithmetic in 64 bits:
+// a 32-bit shift by a large log_pe_stride wraps and would let a set through whose members
+// lie far outside the arena.
+bool active_set_in_range(int pe_start, int log_pe_stride, int pe_size, int num_pes);
+
 // hipGetLastError() after a launch, folded into the error convention.
 int after_launch(const char *what);
 

@@ -232,9 +232,7 @@ int rsm_broadcast(size_t elem_size, void *dest, const void *source, size_t nelem
   if (!rsm::check_symmetric(dest, "dest") || !rsm::check_symmetric(source, "source") ||
       !rsm::check_symmetric(pSync, "pSync"))
     return -1;
-  if (pe_start < 0 || log_pe_stride < 0 || log_pe_stride > 30 || pe_size < 1 ||
-      pe_size > detail::kMaxPes ||
-      pe_start + ((pe_size - 1) << log_pe_stride) >= rt->num_pes() || pe_root < 0 ||
+  if (!rsm::active_set_in_range(pe_start, log_pe_stride, pe_size, rt->num_pes()) || pe_root < 0 ||
       pe_root >= pe_size)
     return rsm::fail("broadcast: active set or root out of range");
   BcastArgs a{nullptr, dest, source, nelem, l.tile, pe_root, pe_start, log_pe_stride,

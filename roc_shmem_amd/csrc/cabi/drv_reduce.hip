@@ -244,9 +244,7 @@ int rsm_to_all(int dtype, int op, void *dest, const void *source, size_t nreduce
   if (!rsm::check_symmetric(dest, "dest") || !rsm::check_symmetric(source, "source") ||
       !rsm::check_symmetric(pSync, "pSync") || !rsm::check_symmetric(pWrk, "pWrk", true))
     return -1;
-  if (pe_start < 0 || log_pe_stride < 0 || log_pe_stride > 30 || pe_size < 1 ||
-      pe_size > detail::kMaxPes ||
-      pe_start + ((pe_size - 1) << log_pe_stride) >= rt->num_pes())
+  if (!rsm::active_set_in_range(pe_start, log_pe_stride, pe_size, rt->num_pes()))
     return rsm::fail("to_all: active set out of range");
   ReduceArgs a{dest, source, nreduce, l.tile, pe_start, log_pe_stride, pe_size, pWrk, pSync,
                nullptr, 1 << log_pe_stride};

@@ -260,6 +260,23 @@ rsm_launch_t collective_launch(host::Runtime *rt, size_t bytes, bool broadcast, 
   l.stream = nullptr;
   return l;
 }
+// A host-initiated collective returns only when its kernel has finished, and a kernel whose flag
+// waits gave up has produced incomplete results: fail like the library's other fatal errors
+// rather than hand them back with a normal return (take_status also puts the barrier pools
+// back in order, which matters to a caller that catches the exit in a test harness only).
+void finish_collective(host::Runtime *rt, const char *what) {
+  check_hip(hipDeviceSynchronize(), what);
+  const uint32_t status = rt->take_status();
+  if (status != 0) {
+    fprintf(stderr,
+            "rocshmem: %s: the device raised status %u (%s); the results are incomplete\n", what,
+            status,
+            status == detail::kStatusWaitTimeout
+                ? "a flag wait gave up after ROC_SHMEM_WAIT_LIMIT_S seconds"
+                : "an argument was refused on the device");
+    exit(EXIT_FAILURE);
+  }
+}
 size_t reduce_elem_size(int dtype) {
   switch (dtype) {
     case RSM_SHORT: case RSM_BF16: return 2;
@@ -364,7 +381,7 @@ void to_all(int dtype, int op, void *dest, const void *source, int nreduce, int 
                  remote_of(rt, source, 0, "roc_shmem_to_all"), static_cast<size_t>(nreduce),
                  pe_start, log_pe_stride, pe_size, nullptr, host_psync(rt), &l))
     die("roc_shmem_to_all");
-  check_hip(hipDeviceSynchronize(), "roc_shmem_to_all");
+  finish_collective(rt, "roc_shmem_to_all");
 }
 
 void to_all_team(int dtype, int op, roc_shmem_team_t team, void *dest, const void *source,
@@ -378,7 +395,7 @@ void to_all_team(int dtype, int op, roc_shmem_team_t team, void *dest, const voi
                       remote_of(rt, source, 0, "roc_shmem_to_all"),
                       static_cast<size_t>(nreduce), &l))
     die("roc_shmem_to_all");
-  check_hip(hipDeviceSynchronize(), "roc_shmem_to_all");
+  finish_collective(rt, "roc_shmem_to_all");
 }
 
 void broadcast(size_t elem_size, void *dest, const void *source, int nelem, int pe_root,
@@ -391,7 +408,7 @@ void broadcast(size_t elem_size, void *dest, const void *source, int nelem, int 
                     remote_of(rt, source, 0, "roc_shmem_broadcast"), static_cast<size_t>(nelem),
                     pe_root, pe_start, log_pe_stride, pe_size, host_psync(rt), &l))
     die("roc_shmem_broadcast");
-  check_hip(hipDeviceSynchronize(), "roc_shmem_broadcast");
+  finish_collective(rt, "roc_shmem_broadcast");
 }
 
 void broadcast_team(size_t elem_size, roc_shmem_team_t team, void *dest, const void *source,
@@ -405,7 +422,7 @@ void broadcast_team(size_t elem_size, roc_shmem_team_t team, void *dest, const v
                          remote_of(rt, source, 0, "roc_shmem_broadcast"),
                          static_cast<size_t>(nelem), pe_root, &l))
     die("roc_shmem_broadcast");
-  check_hip(hipDeviceSynchronize(), "roc_shmem_broadcast");
+  finish_collective(rt, "roc_shmem_broadcast");
 }
 
 }  // namespace hostx

@@ -104,8 +104,9 @@ Options Options::from_env() {
   if (env_u64("ROC_SHMEM_SQ_SIZE", &v)) o.sq_size = static_cast<uint32_t>(v);
   if (env_u64("ROC_SHMEM_SLICE_PAD", &v)) o.slice_pad = static_cast<size_t>(v);
   if (const char *s = getenv("ROC_SHMEM_WAIT_LIMIT_S")) {
-    double d = atof(s);
-    if (d > 0) o.wait_limit_s = d;
+    char *end = nullptr;
+    double d = strtod(s, &end);
+    if (end != s && d >= 0) o.wait_limit_s = d;   // 0: waits never give up
   }
   if (const char *s = getenv("ROC_SHMEM_SQ_MODE")) o.sq_queue_mode = strcmp(s, "queue") == 0;
   if (env_u64("ROC_SHMEM_HEAP_HOST_VISIBLE", &v)) o.heap_host_visible = v != 0;
@@ -255,7 +256,10 @@ std::string Runtime::init(const Options &opt) {
   state_.base_heap = base_heap_dev_;
   state_.team_world = world_->device;
   state_.status = status_dev_;
-  state_.wait_limit_ticks = static_cast<uint64_t>(opt_.wait_limit_s * 100e6);  // 100 MHz clock
+  // 100 MHz clock; a limit of 0 means "never give up" (the reference's behaviour)
+  state_.wait_limit_ticks = opt_.wait_limit_s > 0 && opt_.wait_limit_s < 1e9
+                                ? static_cast<uint64_t>(opt_.wait_limit_s * 100e6)
+                                : ~0ull;
   state_.sq_queue_mode = opt_.sq_queue_mode ? 1u : 0u;
   state_.pad_ = 0;
   reset_queues(nullptr);
@@ -441,8 +445,27 @@ uint32_t Runtime::take_status() {
   uint32_t v = 0;
   (void)hipDeviceSynchronize();
   (void)hipMemcpy(&v, status_dev_, sizeof(v), hipMemcpyDeviceToHost);
-  if (v) (void)hipMemset(status_dev_, 0, sizeof(v));
+  if (v) {
+    // A wait that gave up leaves synchronisation state behind that later calls would trip
+    // over: flags that were set and never consumed, and barrier call counts that differ
+    // between the members that got through and those that did not.  Nothing is running
+    // (the device was synchronised above), so put every library-owned pool back to zero.
+    reset_sync_pools();
+    (void)hipMemset(status_dev_, 0, sizeof(v));
+  }
   return v;
+}
+
+void Runtime::reset_sync_pools() {
+  const size_t pool_bytes = static_cast<size_t>(opt_.num_blocks) * detail::kSyncSlots * sizeof(long);
+  for (const auto &kv : teams_)
+    for (int p = 0; p < opt_.num_pes; ++p)
+      (void)hipMemset(slice_base(p) + kv.second.pool_offset, 0, 4 * pool_bytes);
+  if (host_psync_) {
+    const size_t off = reinterpret_cast<char *>(host_psync_) - slice_base(0);
+    for (int p = 0; p < opt_.num_pes; ++p) (void)hipMemset(slice_base(p) + off, 0, pool_bytes);
+  }
+  (void)hipDeviceSynchronize();
 }
 
 // ---------------------------------------------------------------------------

@@ -53,7 +53,7 @@ struct Options {
   int num_blocks = 64;             // ROC_SHMEM_NUM_BLOCKS, contexts per PE
   uint32_t sq_size = 1024;         // ROC_SHMEM_SQ_SIZE (reference: connection.hpp:225)
   size_t slice_pad = 0;            // ROC_SHMEM_SLICE_PAD, extra bytes between slices
-  double wait_limit_s = 2.0;       // ROC_SHMEM_WAIT_LIMIT_S, bound of a device flag wait
+  double wait_limit_s = 2.0;       // ROC_SHMEM_WAIT_LIMIT_S, bound of a flag wait; 0 = no limit
   bool sq_queue_mode = false;      // ROC_SHMEM_SQ_MODE=queue: slots are freed by the consumer pass
   // ROC_SHMEM_HEAP_HOST_VISIBLE (default 1): the arena is fine-grained device memory, which host
   // code can dereference like the reference's heap (hipExtMallocWithFlags, heap_type.hpp:50) and
@@ -124,8 +124,11 @@ class Runtime {
   }
   size_t arena_bytes() const { return stride_ * static_cast<size_t>(opt_.num_pes); }
 
-  // Reads and clears the sticky device status word.
+  // Reads and clears the sticky device status word.  When it was raised, the team pSync pools
+  // and the host collectives' pSync are zeroed in every PE slice (reset_sync_pools), so that
+  // the collectives and barriers that follow start from a consistent state.
   uint32_t take_status();
+  void reset_sync_pools();
 
   // pSync slices (num_blocks x 256 longs, zeroed, in every PE's heap) that the
   // host-initiated active-set collectives use; allocated on first use,

@@ -89,3 +89,31 @@ int main() { roc_shmem_init(); void *p = roc_shmem_malloc(64); roc_shmem_free(p)
            "-c", str(src), "-o", str(tmp_path / "user_kernel.o")]
     r = subprocess.run(cmd, capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-3000:]
+
+
+def test_active_set_range_check_is_done_in_64_bits():
+    # The check rsm_to_all / rsm_broadcast apply before they launch.  A 32-bit
+    # (pe_size - 1) << log_pe_stride wraps for large strides (4 << 30 == 0, 2 << 30 == INT_MIN)
+    # and would accept sets whose members lie far outside the arena.  No launch here.
+    from roc_shmem_amd import _lib
+    ok = _lib.load().rsm_host_active_set_in_range
+    assert ok(0, 0, 8, 8) == 1
+    assert ok(0, 0, 9, 8) == 0
+    assert ok(1, 1, 4, 8) == 1          # 1, 3, 5, 7
+    assert ok(1, 1, 5, 8) == 0          # ... 9
+    assert ok(0, 2, 2, 8) == 1          # 0, 4
+    assert ok(0, 3, 2, 8) == 0          # 0, 8
+    assert ok(0, 6, 2, 128) == 1 and ok(0, 7, 2, 128) == 0
+    assert ok(5, 0, 1, 8) == 1 and ok(8, 0, 1, 8) == 0 and ok(-1, 0, 1, 8) == 0
+    for pe_size in (2, 3, 5, 128):
+        for log in (29, 30, 31, 32, 40):
+            assert ok(0, log, pe_size, 128) == 0, (pe_size, log)
+    assert ok(0, 30, 1, 8) == 1 and ok(0, 31, 1, 8) == 0   # one member: any representable stride
+    assert ok(0, -1, 2, 8) == 0 and ok(0, 0, 0, 8) == 0 and ok(0, 0, 129, 128) == 0
+    # brute force against exact integers
+    for num_pes in (1, 2, 7, 8, 128):
+        for start in range(0, num_pes + 1):
+            for log in range(0, 9):
+                for size in (1, 2, 3, 4, 8, 16, 127, 128):
+                    want = int(start < num_pes and start + (size - 1) * (1 << log) < num_pes)
+                    assert ok(start, log, size, num_pes) == want, (start, log, size, num_pes)

@@ -233,3 +233,42 @@ def test_barriers_keep_count_across_launches_of_different_shapes():
         rs.synchronize()
         assert rs.take_status() == 0
         rs.roc_shmem_team_destroy(again)
+
+
+def test_barrier_pool_is_put_back_in_order_after_a_wait_that_gave_up():
+    # sync_all / barrier_all keep a count of calls per context block in the team's barrier pool.
+    # If a wait gives up, the counts of the members that got through and of those that did not
+    # differ from then on.  The condition is forced from the host: PE 1's count for block 0 is
+    # set ahead of everybody else's, so PE 1 announces a call number the others never reach and
+    # its wait gives up after the (tiny) limit; every kernel exits normally.  Reading the status
+    # word must report the timeout once and zero the pools, after which barriers work again.
+    import os
+    import time
+    os.environ["ROC_SHMEM_WAIT_LIMIT_S"] = "0.02"
+    try:
+        rs.roc_shmem_init(4, 4 << 20, 2, 64)
+    finally:
+        del os.environ["ROC_SHMEM_WAIT_LIMIT_S"]
+    try:
+        rs.roc_shmem_wg_barrier_all(3, rs.Launch(2, 64))
+        rs.synchronize()
+        assert rs.take_status() == 0
+        # device Team object: TeamInfo (4 ints), valid, pad, then the barrier pool's heap offset
+        team = rs.read_device(rs.roc_shmem_team_world(), 32)
+        pool_off = int(np.frombuffer(team, dtype=np.uint64)[3])
+        epoch_slot = 255                                     # last long of a 256-long slice
+        count_at = rs.heap_base(1) + pool_off + epoch_slot * 8
+        assert int(np.frombuffer(rs.read_device(count_at, 8), dtype=np.uint64)[0]) == 3
+        rs.write_device(count_at, np.array([10], dtype=np.uint64))
+        rs.roc_shmem_wg_barrier_all(1, rs.Launch(1, 64))
+        rs.synchronize()
+        assert rs.take_status() == 1, "the skewed barrier must time out and say so"
+        assert int(np.frombuffer(rs.read_device(count_at, 8), dtype=np.uint64)[0]) == 0, \
+            "reading a raised status word zeroes the barrier pools"
+        t0 = time.perf_counter()
+        rs.roc_shmem_wg_barrier_all(5, rs.Launch(2, 64))
+        rs.synchronize()
+        assert rs.take_status() == 0
+        assert time.perf_counter() - t0 < 0.5, "a barrier waited for its time limit after the reset"
+    finally:
+        rs.roc_shmem_finalize()
