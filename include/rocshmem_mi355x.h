@@ -180,6 +180,18 @@ int rsm_graph_destroy(void *graph);
 int rsm_to_all(int dtype, int op, void *dest, const void *source, size_t nreduce, int pe_start,
                int log_pe_stride, int pe_size, void *pWrk, long *pSync,
                const rsm_launch_t *launch);
+/* rsm_to_all for callers that cannot allocate device memory (code recorded into a HIP
+ * graph, serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference, whose active-set reductions always take the caller's pSync.  Same result
+ * as rsm_to_all with launch->tile == 0 (the sharded form); the synchronisation flags live
+ * in an array of the library's own (4 MiB of device memory per GPU, held until the process
+ * ends) instead of a caller-allocated pSync, and the call allocates and frees nothing.
+ * Limit: num_pes * launch->wgs_per_pe <= 2048 workgroups and launch->tile == 0, otherwise the
+ * call fails with a message and launches nothing.  All calls on one GPU share the array:
+ * calls that overlap in time on one GPU (different streams, different host threads) race;
+ * calls that follow each other on one stream are safe. */
+int rsm_to_all_noalloc(int dtype, int op, void *dest, const void *source, size_t nreduce,
+                       int pe_start, int log_pe_stride, int pe_size, const rsm_launch_t *launch);
 /* Team form (roc_shmem.hpp:848-851; context_ib_tmpl_device.hpp:238-260). */
 int rsm_to_all_team(int dtype, int op, uint64_t team, void *dest, const void *source,
                     size_t nreduce, const rsm_launch_t *launch);

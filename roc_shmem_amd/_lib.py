@@ -52,6 +52,7 @@ SIGNATURES = {
     "rsm_graph_launch": (i32, [vp, vp]),
     "rsm_graph_destroy": (i32, [vp]),
     "rsm_to_all": (i32, [i32, i32, vp, vp, sz, i32, i32, i32, vp, vp, LP]),
+    "rsm_to_all_noalloc": (i32, [i32, i32, vp, vp, sz, i32, i32, i32, LP]),
     "rsm_to_all_team": (i32, [i32, i32, u64, vp, vp, sz, LP]),
     "rsm_rma": (i32, [i32, i32, vp, vp, sz, sz, sz, sz, i32, LP]),
     "rsm_broadcast": (i32, [sz, vp, vp, sz, i32, i32, i32, i32, vp, LP]),

@@ -16,7 +16,8 @@ __all__ = [
     "roc_shmem_init", "roc_shmem_finalize", "roc_shmem_n_pes", "roc_shmem_malloc",
     "roc_shmem_free", "roc_shmem_ptr", "roc_shmem_team_world", "roc_shmem_team_split_strided",
     "roc_shmem_team_destroy", "roc_shmem_team_n_pes", "roc_shmem_team_translate_pe",
-    "roc_shmem_barrier_all", "roc_shmem_to_all", "roc_shmem_team_to_all", "roc_shmem_rma",
+    "roc_shmem_barrier_all", "roc_shmem_to_all", "roc_shmem_to_all_noalloc", "roc_shmem_team_to_all",
+    "roc_shmem_rma",
     "roc_shmem_broadcast", "roc_shmem_team_broadcast", "roc_shmem_alltoall",
     "roc_shmem_fcollect", "roc_shmem_wg_barrier_all", "roc_shmem_small_ops",
     "sq_reset", "sq_read", "sq_image", "sq_state", "sq_constants", "sq_rkey",
@@ -299,6 +300,14 @@ def roc_shmem_to_all(dtype, op, dest, source, nreduce, PE_start, logPE_stride, P
     _check(L.load().rsm_to_all(dtype, op, _addr(dest), _addr(source), nreduce, PE_start,
                                logPE_stride, PE_size, _addr(pWrk) if pWrk is not None else None,
                                _addr(pSync), _launch(launch)))
+
+
+def roc_shmem_to_all_noalloc(dtype, op, dest, source, nreduce, PE_start, logPE_stride, PE_size,
+                             launch=None):
+    """The sharded form of roc_shmem_to_all without a caller-allocated pSync: the flags live in
+    an array of the library's own and the call allocates nothing (rsm_to_all_noalloc)."""
+    _check(L.load().rsm_to_all_noalloc(dtype, op, _addr(dest), _addr(source), nreduce, PE_start,
+                                       logPE_stride, PE_size, _launch(launch)))
 
 
 def roc_shmem_team_to_all(dtype, op, team, dest, source, nreduce, launch=None):

@@ -133,6 +133,10 @@ int rsm_init(int num_pes, size_t heap_bytes_per_pe, int num_blocks, unsigned sq_
   if (sq_size) o.sq_size = sq_size;
   std::string err = Runtime::create(o);
   if (!err.empty()) return rsm::fail(err);
+  if (!rsm::noalloc_flags()) {
+    Runtime::destroy();
+    return -1;
+  }
   rocshmem::ROC_SHMEM_TEAM_WORLD =
       reinterpret_cast<rocshmem::roc_shmem_team_t>(Runtime::get()->team_world());
   return 0;

@@ -45,6 +45,11 @@ bool check_extent(const void *p, size_t bytes, const char *what);
 // lie far outside the arena.
 bool active_set_in_range(int pe_start, int log_pe_stride, int pe_size, int num_pes);
 
+// Device address, on the current device, of the flag array that rsm_to_all_noalloc uses
+// (defined beside the array in drv_reduce.hip); looked up on a device's first call, which
+// rsm_init makes.  nullptr, with the error set, when the runtime cannot resolve it.
+long *noalloc_flags();
+
 // hipGetLastError() after a launch, folded into the error convention.
 int after_launch(const char *what);
 

@@ -63,10 +63,30 @@ RSM_TO_ALL(__hip_bfloat16, bf16, sum, ROC_SHMEM_SUM)
 RSM_TO_ALL(__hip_bfloat16, bf16, max, ROC_SHMEM_MAX)
 RSM_TO_ALL(__hip_bfloat16, bf16, min, ROC_SHMEM_MIN)
 
-// kShard: the PE's workgroups share one reduction (sharded extension); otherwise one standard
-// call per tile, tiles dealt round-robin to the PE's workgroups.  Two kernels rather than a
-// branch: with both forms inlined into one kernel the compiler ran out of scalar registers.
-template <typename T, ROC_SHMEM_OP Op, bool kShard>
+// Flag scratch of rsm_to_all_noalloc: room for kNoAllocMaxWgs workgroups' flag
+// slices (ROC_SHMEM_REDUCE_SYNC_SIZE longs each, 4 MiB in all), laid out PE-major
+// ([pe][workgroup][256]) so that two PEs' copies of a workgroup's slice are a fixed
+// number of bytes apart, as the copies of a symmetric pSync are.  Every device that
+// loads the library holds its own copy until the process ends.  In host code this
+// name is a stand-in, not a device address: host code uses the address that
+// hipGetSymbolAddress returned (noalloc_flags()).
+constexpr unsigned kNoAllocMaxWgs = 2048;
+static __device__ __align__(256) long g_noalloc_flags[kNoAllocMaxWgs * ROC_SHMEM_REDUCE_SYNC_SIZE];
+
+__global__ void __launch_bounds__(256) clear_flags_kernel(long *flags, size_t n) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) flags[i] = ROC_SHMEM_SYNC_VALUE;
+}
+
+// Forms of the reduction kernel.  kTiled: one standard call per tile, tiles dealt
+// round-robin to the PE's workgroups.  kSharded: the PE's workgroups share one reduction
+// (sharded extension), pSync is the caller's symmetric array.  kShardedStaticFlags: the
+// same with the flags in the library's own array (`pSync0` is its device address).  Separate
+// kernels rather than branches: with more than one form inlined into one kernel the compiler
+// ran out of scalar registers.
+enum ToAllForm { kTiled = 0, kSharded = 1, kShardedStaticFlags = 2 };
+
+template <typename T, ROC_SHMEM_OP Op, int kForm>
 __global__ void __launch_bounds__(1024)
     to_all_kernel(T *dest0, const T *source0, size_t n, size_t tile, int pe_start, int log_stride,
                   int pe_size, T *pWrk0, long *pSync0) {
@@ -83,16 +103,23 @@ __global__ void __launch_bounds__(1024)
   if (member) {
     T *dest = roc_shmemx_my_addr(dest0);
     const T *source = roc_shmemx_my_addr(source0);
-    T *pWrk = roc_shmemx_my_addr(pWrk0);
-    long *pSync = roc_shmemx_my_addr(pSync0) + w * ROC_SHMEM_REDUCE_SYNC_SIZE;
-    if constexpr (kShard) {
-      ToAll<T, Op>::active_set_shard(ctx, dest, source, n, pe_start, log_stride, pe_size, pWrk,
-                                     pSync, static_cast<int>(w), static_cast<int>(nw));
+    if constexpr (kForm == kShardedStaticFlags) {
+      long *flags = pSync0 + (static_cast<size_t>(me) * nw + w) * ROC_SHMEM_REDUCE_SYNC_SIZE;
+      const int64_t pe_step = static_cast<int64_t>(nw) * ROC_SHMEM_REDUCE_SYNC_SIZE * sizeof(long);
+      detail::wg_all_reduce<T, Op>(me, dest, source, n, pe_start, 1 << log_stride, pe_size, flags,
+                                   static_cast<int>(w), static_cast<int>(nw), pe_step);
     } else {
-      for (size_t off = w * tile; off < n; off += nw * tile) {
-        size_t cnt = n - off < tile ? n - off : tile;
-        ToAll<T, Op>::active_set(ctx, dest + off, source + off, static_cast<int>(cnt), pe_start,
-                                 log_stride, pe_size, pWrk, pSync);
+      T *pWrk = roc_shmemx_my_addr(pWrk0);
+      long *pSync = roc_shmemx_my_addr(pSync0) + w * ROC_SHMEM_REDUCE_SYNC_SIZE;
+      if constexpr (kForm == kSharded) {
+        ToAll<T, Op>::active_set_shard(ctx, dest, source, n, pe_start, log_stride, pe_size, pWrk,
+                                       pSync, static_cast<int>(w), static_cast<int>(nw));
+      } else {
+        for (size_t off = w * tile; off < n; off += nw * tile) {
+          size_t cnt = n - off < tile ? n - off : tile;
+          ToAll<T, Op>::active_set(ctx, dest + off, source + off, static_cast<int>(cnt), pe_start,
+                                   log_stride, pe_size, pWrk, pSync);
+        }
       }
     }
   }
@@ -140,28 +167,31 @@ struct ReduceArgs {
   long *pSync;
   roc_shmem_team_t team;
   int stride;
+  bool static_flags;   // pSync is the device address of the library's own flag array
 };
 
+template <typename T, ROC_SHMEM_OP Op, int kForm>
+void launch_active_set(const rsm::Launch &l, const ReduceArgs &a) {
+  hipLaunchKernelGGL((to_all_kernel<T, Op, kForm>), dim3(l.grid), dim3(l.wg_size), 0, l.stream,
+                     static_cast<T *>(a.dest), static_cast<const T *>(a.source), a.n, a.tile,
+                     a.pe_start, a.log_stride, a.pe_size, static_cast<T *>(a.pWrk), a.pSync);
+}
+
 template <typename T, ROC_SHMEM_OP Op, bool kShard>
-void launch_form(const rsm::Launch &l, const ReduceArgs &a) {
-  if (a.team) {
-    hipLaunchKernelGGL((to_all_team_kernel<T, Op, kShard>), dim3(l.grid), dim3(l.wg_size), 0,
-                       l.stream, a.team, static_cast<T *>(a.dest),
-                       static_cast<const T *>(a.source), a.n, a.tile, a.pe_start, a.stride,
-                       a.pe_size);
-  } else {
-    hipLaunchKernelGGL((to_all_kernel<T, Op, kShard>), dim3(l.grid), dim3(l.wg_size), 0, l.stream,
-                       static_cast<T *>(a.dest), static_cast<const T *>(a.source), a.n, a.tile,
-                       a.pe_start, a.log_stride, a.pe_size, static_cast<T *>(a.pWrk), a.pSync);
-  }
+void launch_team(const rsm::Launch &l, const ReduceArgs &a) {
+  hipLaunchKernelGGL((to_all_team_kernel<T, Op, kShard>), dim3(l.grid), dim3(l.wg_size), 0,
+                     l.stream, a.team, static_cast<T *>(a.dest), static_cast<const T *>(a.source),
+                     a.n, a.tile, a.pe_start, a.stride, a.pe_size);
 }
 
 template <typename T, ROC_SHMEM_OP Op>
 void launch_one(const rsm::Launch &l, const ReduceArgs &a) {
-  if (a.tile == 0) {
-    launch_form<T, Op, true>(l, a);
+  if (a.static_flags) {
+    launch_active_set<T, Op, kShardedStaticFlags>(l, a);
+  } else if (a.team) {
+    a.tile == 0 ? launch_team<T, Op, true>(l, a) : launch_team<T, Op, false>(l, a);
   } else {
-    launch_form<T, Op, false>(l, a);
+    a.tile == 0 ? launch_active_set<T, Op, kSharded>(l, a) : launch_active_set<T, Op, kTiled>(l, a);
   }
 }
 
@@ -210,7 +240,7 @@ int run(int dtype, int op, const rsm::Launch &l, ReduceArgs a) {
   if (a.n == 0) return 0;  // zero-element reductions are no-ops (context_tmpl_device.hpp:68-70)
   if (a.n > (~size_t{0} >> 4) || !rsm::check_extent(a.dest, a.n * es, "to_all: dest") ||
       !rsm::check_extent(a.source, a.n * es, "to_all: source") ||
-      !rsm::check_extent(a.pSync, static_cast<size_t>(l.wgs_per_pe) * ROC_SHMEM_REDUCE_SYNC_SIZE * sizeof(long),
+      !rsm::check_extent(a.static_flags ? nullptr : a.pSync, static_cast<size_t>(l.wgs_per_pe) * ROC_SHMEM_REDUCE_SYNC_SIZE * sizeof(long),
                          "to_all: pSync (wgs_per_pe slices of ROC_SHMEM_REDUCE_SYNC_SIZE longs)"))
     return -1;
   // tile == 0: the PE's workgroups share one reduction through the sharded
@@ -230,9 +260,66 @@ int run(int dtype, int op, const rsm::Launch &l, ReduceArgs a) {
   return rsm::after_launch("to_all");
 }
 
+// Device address of g_noalloc_flags on each device, looked up once per device.
+constexpr int kMaxDevices = 64;
+long *g_noalloc_flags_at[kMaxDevices] = {};
+
 }  // namespace
 
+namespace rsm {
+
+// Called by rsm_init (and, should a caller switch devices afterwards, by the entry point's
+// first call on the new device), with the device current: asks the runtime where this
+// device's copy of the flag array lives.  Allocates nothing.
+long *noalloc_flags() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    fail("to_all_noalloc: cannot tell the current device");
+    return nullptr;
+  }
+  if (!g_noalloc_flags_at[dev]) {
+    long *at = nullptr;
+    hipError_t e = hipGetSymbolAddress(reinterpret_cast<void **>(&at), HIP_SYMBOL(g_noalloc_flags));
+    if (e != hipSuccess || !at) {
+      fail(std::string("to_all_noalloc: hipGetSymbolAddress: ") + hipGetErrorString(e));
+      return nullptr;
+    }
+    g_noalloc_flags_at[dev] = at;
+  }
+  return g_noalloc_flags_at[dev];
+}
+
+}  // namespace rsm
+
 extern "C" {
+
+int rsm_to_all_noalloc(int dtype, int op, void *dest, const void *source, size_t nreduce,
+                       int pe_start, int log_pe_stride, int pe_size, const rsm_launch_t *launch) {
+  RSM_ENTRY;
+  rsm::Launch l;
+  if (!rsm::resolve_launch(launch, &l)) return -1;
+  host::Runtime *rt = host::Runtime::get();
+  if (!rsm::check_symmetric(dest, "dest") || !rsm::check_symmetric(source, "source")) return -1;
+  if (!rsm::active_set_in_range(pe_start, log_pe_stride, pe_size, rt->num_pes()))
+    return rsm::fail("to_all_noalloc: active set out of range");
+  if (l.tile != 0)
+    return rsm::fail("to_all_noalloc: launch->tile must be 0 (the PE's workgroups share one reduction)");
+  if (l.grid > kNoAllocMaxWgs)
+    return rsm::fail("to_all_noalloc: " + std::to_string(l.grid) + " workgroups (PEs x wgs_per_pe) exceed the " +
+                     std::to_string(kNoAllocMaxWgs) + " the library's flag array has room for");
+  long *flags = rsm::noalloc_flags();
+  if (!flags) return -1;
+  if (nreduce == 0) return 0;
+  // The array is shared by every call on this device and keeps what the last call left: the
+  // slices this grid uses start at zero whatever happened before (a call whose waits gave up
+  // leaves flags set).  A kernel, not hipMemsetAsync, so that the call can be recorded in a graph.
+  const size_t n_flags = static_cast<size_t>(l.grid) * ROC_SHMEM_REDUCE_SYNC_SIZE;
+  hipLaunchKernelGGL(clear_flags_kernel, dim3(static_cast<unsigned>((n_flags + 255) / 256)), dim3(256),
+                     0, l.stream, flags, n_flags);
+  ReduceArgs a{dest, source, nreduce, 0, pe_start, log_pe_stride, pe_size, nullptr, flags,
+               nullptr, 1 << log_pe_stride, true};
+  return run(dtype, op, l, a);
+}
 
 int rsm_to_all(int dtype, int op, void *dest, const void *source, size_t nreduce, int pe_start,
                int log_pe_stride, int pe_size, void *pWrk, long *pSync,
@@ -247,7 +334,7 @@ int rsm_to_all(int dtype, int op, void *dest, const void *source, size_t nreduce
   if (!rsm::active_set_in_range(pe_start, log_pe_stride, pe_size, rt->num_pes()))
     return rsm::fail("to_all: active set out of range");
   ReduceArgs a{dest, source, nreduce, l.tile, pe_start, log_pe_stride, pe_size, pWrk, pSync,
-               nullptr, 1 << log_pe_stride};
+               nullptr, 1 << log_pe_stride, false};
   return run(dtype, op, l, a);
 }
 
@@ -264,7 +351,7 @@ int rsm_to_all_team(int dtype, int op, uint64_t team, void *dest, const void *so
     return rsm::fail("to_all_team: wgs_per_pe exceeds the contexts per PE (team pSync slices)");
   const detail::TeamInfo &ti = rec->image.wrt_world;
   ReduceArgs a{dest, source, nreduce, l.tile, ti.pe_start, 0, ti.size, nullptr,
-               nullptr, reinterpret_cast<roc_shmem_team_t>(team), ti.stride};
+               nullptr, reinterpret_cast<roc_shmem_team_t>(team), ti.stride, false};
   return run(dtype, op, l, a);
 }
 

@@ -291,7 +291,8 @@ __device__ __forceinline__ void reduce_elements(T *dst, const T *src, size_t e_b
 template <typename T, ROC_SHMEM_OP Op>
 __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *source, size_t nreduce,
                                               int pe_start, int pe_stride, int pe_size,
-                                              long *psync, int shard = 0, int nshards = 1) {
+                                              long *psync, int shard = 0, int nshards = 1,
+                                              int64_t psync_pe_step = 0) {
   // Workgroup-collective: every lane holds the same arguments.
   my_pe = uniform(my_pe);
   dest = uniform(dest);
@@ -303,6 +304,7 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
   psync = uniform(psync);
   shard = uniform(shard);
   nshards = uniform(nshards);
+  psync_pe_step = static_cast<int64_t>(uniform(static_cast<unsigned long>(psync_pe_step)));
   if (nreduce == 0) return;  // reference: Context::to_all early-out, context_tmpl_device.hpp:68-70
   if (pe_size > kMaxPes || pe_size <= 0 || nshards <= 0 || shard < 0 || shard >= nshards) {
     status_raise(kStatusBadArgument);
@@ -318,7 +320,7 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
   const size_t parts = static_cast<size_t>(pe_size) * nshards;
   const size_t part = static_cast<size_t>(shard) * pe_size + my_idx;
 
-  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, pe_stride, pe_size);
+  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, pe_stride, pe_size, psync_pe_step);
 
   constexpr size_t E = VecOf<T>::kElems;
   // The vector path stores 16-byte aligned and loads at any 4-byte alignment,
@@ -393,7 +395,7 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
     reduce_elements<T, Op>(dest, source, e0, e1, as, my_pe, tid, nthr);
   }
 
-  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size);
+  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size, psync_pe_step);
 }
 
 }  // namespace detail

@@ -120,17 +120,24 @@ __device__ __forceinline__ bool bounded_wait(const T *ptr, int cmp, T want) {
 // closing workgroup barrier covers every wave that resumes after it.  With a
 // fence per wave, 256 workgroups of 16 waves spent 31 us in one barrier
 // (each fence walks a whole L2); the flag lanes alone need a fraction of it.
+//
+// `pe_step` is the distance in bytes between two PEs' copies of the flag array:
+// 0 stands for the slice stride of the symmetric heap (pSync is a symmetric
+// object); a flag array that lives outside the heap names its own.
 __device__ __forceinline__ void wg_flag_barrier(long *psync, int set, int my_pe, int my_idx,
-                                                int pe_start, int pe_stride, int n_pes) {
+                                                int pe_start, int pe_stride, int n_pes,
+                                                int64_t pe_step = 0) {
   __syncthreads();
   const uint32_t tid = flat_thread_id();
   const uint32_t nthr = flat_block_size();
+  if (pe_step == 0) pe_step = static_cast<int64_t>(g_state.slice_stride);
   if (tid < static_cast<uint32_t>(n_pes)) {
     fence_release_agent();
     for (uint32_t t = tid; t < static_cast<uint32_t>(n_pes); t += nthr) {
       int peer = pe_start + static_cast<int>(t) * pe_stride;
       unsigned long long *slot = reinterpret_cast<unsigned long long *>(
-          translate(psync, my_pe, peer) + set * n_pes + my_idx);
+          reinterpret_cast<char *>(psync) + (static_cast<int64_t>(peer) - my_pe) * pe_step) +
+          set * n_pes + my_idx;
       __hip_atomic_store(slot, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     for (uint32_t t = tid; t < static_cast<uint32_t>(n_pes); t += nthr) {
