@@ -144,6 +144,7 @@ int rsm_copy_to_device(void *dst, const void *host_src, size_t bytes);
 int rsm_copy_to_host(void *host_dst, const void *src, size_t bytes);
 int rsm_fill(void *dst, int byte_value, size_t bytes);
 int rsm_synchronize(void);
+int rsm_stream_synchronize(void *stream);       /* NULL = the default stream */
 void *rsm_device_alloc(size_t bytes);           /* ordinary (non-symmetric) device memory */
 int rsm_device_free(void *ptr);
 void *rsm_stream_create(void);
@@ -282,6 +283,31 @@ int rsm_sq_consume(int pe, int block, void *target_arena, rsm_consume_totals_t *
  * a slot is reused only after rsm_sq_consume retired it; a producer that finds
  * its ring full waits (bounded) and raises the status word. */
 int rsm_sq_set_mode(int queue_mode);
+/* A consumer that runs at the same time as the producers (what the NIC is to the
+ * reference's queues: entries are retired while kernels post, QueuePair::quiet_internal
+ * reads the completions, queue_pair.cpp:118-191, waitSQSpace blocks on retirement,
+ * :400-415).  rsm_sq_consumer_start switches the rings to queue mode, launches a
+ * persistent kernel on a stream of the library's own that checks and retires what the
+ * rings publish (completion entries, `consumed`), and returns when all its waves are
+ * resident.  Until rsm_sq_consumer_stop, producers (rsm_small_ops and any kernel that
+ * posts) block in their post when their ring is full and go on when the consumer has freed
+ * slots; roc_shmem_ctx_quiet collects the completions its queue has asked for (bounded
+ * waits, status word on timeout).  Entries and completions are written through to
+ * memory meanwhile.  rsm_sq_consumer_stop: call it when the producers' streams have been
+ * synchronised (it synchronises the default stream itself); it lets the consumer drain the
+ * rings, waits for it, restores the previous mode and returns what was retired.  Between
+ * the two calls synchronise streams, not the device: entry points that synchronise the
+ * device (rsm_synchronize, rsm_take_status, rsm_sq_reset, rsm_sq_consume) refuse to run,
+ * and a consumer wave whose rings stay silent for ROC_SHMEM_CONSUMER_IDLE_S seconds
+ * (default 5) leaves by itself, which rsm_sq_consumer_stop reports as an error. */
+int rsm_sq_consumer_start(void);
+int rsm_sq_consumer_stop(rsm_consume_totals_t *totals);
+int rsm_sq_consumer_running(void);
+/* Reader side of a completion queue (reference: cq_consumer_counter, quiet_counter,
+ * dbrec_cq, queue_pair.hpp:340-396): completions taken by quiet, completions asked for
+ * and not yet taken, and the completion queue's doorbell record. */
+int rsm_cq_reader_state(int pe, int block, uint32_t *cq_consumer, uint32_t *quiet_counter,
+                        uint32_t *cq_doorbell_record);
 int rsm_sq_consumer_state(int pe, int block, uint32_t *consumed, uint32_t *cq_producer);
 int rsm_cq_image(int pe, int block, void *host_out, size_t bytes);        /* sq_size x 64 B */
 int rsm_atomic_ret_image(int pe, int block, void *host_out, size_t bytes); /* 4096 x 8 B     */

@@ -54,6 +54,11 @@ def _load():
     lib.orc_wqe_build.argtypes = [vp, vp, u32, vp]
     lib.orc_sq_consume.restype = None
     lib.orc_sq_consume.argtypes = [vp, vp, u32, u32, vp, vp, vp, vp, vp, u32, vp, vp]
+    lib.orc_ring_check.restype = C.c_long
+    lib.orc_ring_check.argtypes = [vp, vp, u32, u32, vp, sz, vp, vp, i32, vp, vp, vp, vp]
+    lib.orc_wqe_build_many.restype = None
+    lib.orc_wqe_build_many.argtypes = [vp, vp, u32, vp, sz]
+    lib.orc_small_ops_mt.argtypes = [vp, sz, vp, sz, vp, i32]
     lib.orc_wqe_index.restype = C.c_uint16
     lib.orc_wqe_index.argtypes = [vp]
     lib.orc_wqe_opcode.restype = C.c_uint8
@@ -239,6 +244,14 @@ class WqeReq(C.Structure):
 OP_WRITE, OP_READ, OP_ATOMIC_CS, OP_ATOMIC_FA = 0x08, 0x10, 0x11, 0x12
 
 
+def requests_cqe(sq_counter, max_nwqe, closes_post):
+    """Whether the entry with running number ``sq_counter`` asks for a completion entry: the
+    entry that closes a wave's post always does (multi-thread post policy, reference
+    library/src/gpu_ib/thread_policy.cpp:170-216), and so does whatever lands in slot
+    ``max_nwqe - 2`` of a lap (update_wqe_ce_single<false>, queue_pair.cpp:80-85)."""
+    return bool(closes_post) or sq_counter % max_nwqe == max_nwqe - 2
+
+
 def wqe_build(slot, qp, sq_counter, opcode, size=0, raddr=0, rkey=0, laddr=0, atomic_data=0,
               atomic_cmp=0, inline=b"", atomic_pos=0, request_cqe=False):
     """Write one entry into ``slot`` (a 64-byte uint8 array view), in place."""
@@ -290,6 +303,55 @@ def sq_consume(qp, ring, consumed, published, heap_base0, slice_stride, heap_siz
                         None if sources is None else sources.ctypes.data, atomic_ret.ctypes.data,
                         cq.ctypes.data, cq.size // 64, C.byref(prod), C.byref(totals))
     return prod.value, totals
+
+
+WQE_EXPECT_DTYPE = np.dtype([("raddr", "<u8"), ("data", "<u8"), ("cmp", "<u8"),
+                             ("opcode", "<u4"), ("size", "<u4")])
+RING_CHECK_REASONS = {1: "index field", 2: "opcode", 3: "AMO return slot outside the window",
+                      4: "not an inline write of 1..8 bytes", 5: "completion flag",
+                      6: "no operation of this ring explains the entry (or it appears twice)",
+                      7: "remote address outside the arena", 8: "bytes differ from the builder's"}
+
+
+def sort_wqe_expect(expect):
+    """Order the checker wants: ascending (opcode, raddr, data, cmp)."""
+    order = np.lexsort((expect["cmp"], expect["data"], expect["raddr"], expect["opcode"]))
+    return np.ascontiguousarray(expect[order])
+
+
+def ring_check(image, qp, first_counter, count, expect_sorted, heap_base0, slice_stride, heap_size,
+               rkeys, full_slot):
+    """Entries first_counter .. first_counter+count-1 of a ring image (uint8, max_nwqe*64)
+    against wqe_build (see ringcheck.c).  Returns a dict: ok, position / reason of the first
+    wrong entry, used (which operations were matched), pos_count (uint32[4096] AMO return
+    positions), n_atomic, n_cqe."""
+    image = np.ascontiguousarray(image, dtype=np.uint8).reshape(-1)
+    assert image.size == qp.max_nwqe * 64 and expect_sorted.dtype == WQE_EXPECT_DTYPE
+    rk = np.ascontiguousarray(rkeys, dtype=np.uint32)
+    arena = Arena(heap_base0, slice_stride, heap_size, len(rk), rk.ctypes.data)
+    used = np.zeros(len(expect_sorted), dtype=np.uint8)
+    pos_count = np.zeros(4096, dtype=np.uint32)
+    n_atomic, n_cqe, why = C.c_uint32(0), C.c_uint32(0), C.c_int(0)
+    rc = _lib.orc_ring_check(image.ctypes.data, C.byref(qp), first_counter & 0xFFFFFFFF, count,
+                             expect_sorted.ctypes.data, len(expect_sorted), used.ctypes.data,
+                             C.byref(arena), 1 if full_slot else 0, pos_count.ctypes.data,
+                             C.byref(n_atomic), C.byref(n_cqe), C.byref(why))
+    return {"ok": rc == 0, "position": rc - 1, "reason": RING_CHECK_REASONS.get(why.value, ""),
+            "used": used, "pos_count": pos_count, "n_atomic": n_atomic.value, "n_cqe": n_cqe.value}
+
+
+def wqe_build_many(ring, qp, first_counter, reqs):
+    """The scalar builder over an array of WqeReq (ctypes array) into a ring image."""
+    _lib.orc_wqe_build_many(ring.ctypes.data, C.byref(qp), first_counter & 0xFFFFFFFF, reqs, len(reqs))
+
+
+def small_ops_mt(heap, ops, threads):
+    """8-byte puts and 64-bit fetch-adds of ``ops`` applied by ``threads`` host threads with
+    hardware atomics (the host-centric path's MPI_Put / MPI_Fetch_and_op on one node)."""
+    ops = np.ascontiguousarray(ops, dtype=SMALL_OP_DTYPE)
+    rc = _lib.orc_small_ops_mt(heap.buf.ctypes.data, heap.stride, ops.ctypes.data, len(ops), None, threads)
+    if rc != 0:
+        raise ValueError("small_ops_mt handles 8-byte puts and 64-bit fetch-adds only")
 
 
 def wqe_index(slot):

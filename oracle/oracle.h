@@ -135,6 +135,33 @@ void orc_sq_consume(const orc_qp_t *qp, const uint8_t *ring, uint32_t consumed, 
                     uint64_t *atomic_ret, uint8_t *cq, uint32_t cq_size, uint32_t *cq_producer,
                     orc_consume_totals_t *totals);
 
+/* ---- bulk ring check, bulk / threaded forms for timing (ringcheck.c) ------------ */
+
+/* One operation as its ring entry describes it.  `data`: the atomic operand, or
+ * the inline payload as a little-endian integer; `cmp`: compare operand (0 unless
+ * compare-and-swap); `size`: payload bytes (8 for atomics). */
+typedef struct orc_wqe_expect {
+  uint64_t raddr;
+  uint64_t data;
+  uint64_t cmp;
+  uint32_t opcode;
+  uint32_t size;
+} orc_wqe_expect_t;
+
+/* Entries first_counter .. first_counter+count-1 of a ring image against the
+ * builder; `expect` sorted ascending by (opcode, raddr, data, cmp), `used`
+ * n_expect zero bytes that come back 1 for every operation an entry stood for.
+ * Returns 0 when all entries are right, else 1 + the position of the first
+ * wrong entry with the reason in *why (see ringcheck.c). */
+long orc_ring_check(const uint8_t *image, const orc_qp_t *qp, uint32_t first_counter,
+                    uint32_t count, const orc_wqe_expect_t *expect, size_t n_expect,
+                    uint8_t *used, const orc_arena_t *arena, int full_slot, uint32_t *pos_count,
+                    uint32_t *n_atomic, uint32_t *n_cqe, int *why);
+void orc_wqe_build_many(uint8_t *ring, const orc_qp_t *qp, uint32_t first_counter,
+                        const orc_wqe_req_t *reqs, size_t n);
+int orc_small_ops_mt(char *heap, size_t stride, const orc_small_op_t *ops, size_t n,
+                     int64_t *fetched, int threads);
+
 /* Parse helpers used by the ring checker. */
 uint16_t orc_wqe_index(const uint8_t slot[64]);
 uint8_t orc_wqe_opcode(const uint8_t slot[64]);

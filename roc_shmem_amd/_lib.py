@@ -39,6 +39,7 @@ SIGNATURES = {
     "rsm_copy_to_host": (i32, [vp, vp, sz]),
     "rsm_fill": (i32, [vp, i32, sz]),
     "rsm_synchronize": (i32, []),
+    "rsm_stream_synchronize": (i32, [vp]),
     "rsm_device_alloc": (vp, [sz]),
     "rsm_device_free": (i32, [vp]),
     "rsm_stream_create": (vp, []),
@@ -70,6 +71,10 @@ SIGNATURES = {
     "rsm_sq_rkey": (i32, [i32, C.POINTER(u32)]),
     "rsm_sq_consume": (i32, [i32, i32, vp, vp]),
     "rsm_sq_set_mode": (i32, [i32]),
+    "rsm_sq_consumer_start": (i32, []),
+    "rsm_sq_consumer_stop": (i32, [vp]),
+    "rsm_sq_consumer_running": (i32, []),
+    "rsm_cq_reader_state": (i32, [i32, i32, C.POINTER(u32), C.POINTER(u32), C.POINTER(u32)]),
     "rsm_sq_consumer_state": (i32, [i32, i32, C.POINTER(u32), C.POINTER(u32)]),
     "rsm_cq_image": (i32, [i32, i32, vp, sz]),
     "rsm_atomic_ret_image": (i32, [i32, i32, vp, sz]),

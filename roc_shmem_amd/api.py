@@ -21,7 +21,8 @@ __all__ = [
     "roc_shmem_broadcast", "roc_shmem_team_broadcast", "roc_shmem_alltoall",
     "roc_shmem_fcollect", "roc_shmem_wg_barrier_all", "roc_shmem_small_ops",
     "sq_reset", "sq_read", "sq_image", "sq_state", "sq_constants", "sq_rkey",
-    "sq_consume", "sq_set_mode", "sq_consumer_state", "cq_image", "atomic_ret_image", "arena",
+    "sq_consume", "sq_set_mode", "sq_consumer_state", "sq_consumer_start", "sq_consumer_stop",
+    "sq_consumer_running", "cq_reader_state", "cq_image", "atomic_ret_image", "arena",
     "read_device", "write_device",
     "kat_fetch_incr", "kat_coalesce", "take_status", "synchronize", "heap_bytes_in_use",
     "sym_array", "Event", "device_array", "heap_base",
@@ -249,6 +250,9 @@ class Stream:
         if not self.h:
             raise RocShmemError(L.load().rsm_last_error().decode())
 
+    def synchronize(self):
+        _check(L.load().rsm_stream_synchronize(self.h))
+
     def destroy(self):
         if self.h:
             L.load().rsm_stream_destroy(self.h)
@@ -419,6 +423,29 @@ def sq_consume(pe=-1, block=-1, target_arena=None):
 def sq_set_mode(queue):
     """False: rings are logs that wrap freely; True: slots are freed by sq_consume only."""
     _check(L.load().rsm_sq_set_mode(1 if queue else 0))
+
+
+def sq_consumer_start():
+    """Start the consumer that retires ring entries while producers post (rsm_sq_consumer_start)."""
+    _check(L.load().rsm_sq_consumer_start())
+
+
+def sq_consumer_stop():
+    """Let the live consumer drain the rings and stop it; returns the totals of what it retired."""
+    t = ConsumeTotals()
+    rc = L.load().rsm_sq_consumer_stop(C.byref(t))
+    _check(rc)
+    return t.as_dict()
+
+
+def sq_consumer_running():
+    return bool(L.load().rsm_sq_consumer_running())
+
+
+def cq_reader_state(pe, block):
+    a, b, c = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
+    _check(L.load().rsm_cq_reader_state(pe, block, C.byref(a), C.byref(b), C.byref(c)))
+    return {"cq_consumer": a.value, "quiet_counter": b.value, "cq_doorbell_record": c.value}
 
 
 def sq_consumer_state(pe, block):

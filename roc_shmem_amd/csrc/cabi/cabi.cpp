@@ -144,6 +144,7 @@ int rsm_init(int num_pes, size_t heap_bytes_per_pe, int num_blocks, unsigned sq_
 
 int rsm_finalize(void) {
   RSM_ENTRY;
+  if (Runtime::get()) rsm::consumer_shutdown();
   Runtime::destroy();
   rocshmem::ROC_SHMEM_TEAM_WORLD = nullptr;
   return 0;
@@ -206,6 +207,8 @@ int rsm_state_units(void) { return rocshmem::host::registered_state_units(); }
 int rsm_take_status(void) {
   RSM_ENTRY;
   RSM_NEED_RT(rt);
+  if (rsm::live_consumer_running())
+    return rsm::fail("rsm_take_status: a live send-queue consumer is running (rsm_sq_consumer_stop first)");
   return static_cast<int>(rt->take_status());
 }
 
@@ -264,7 +267,15 @@ int rsm_fill(void *dst, int byte_value, size_t bytes) {
 }
 int rsm_synchronize(void) {
   RSM_ENTRY;
+  if (rsm::live_consumer_running())
+    return rsm::fail("rsm_synchronize: a live send-queue consumer is running; synchronise streams "
+                     "(rsm_stream_synchronize) until rsm_sq_consumer_stop");
   RSM_HIP(hipDeviceSynchronize());
+  return 0;
+}
+int rsm_stream_synchronize(void *stream) {
+  RSM_ENTRY;
+  RSM_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
   return 0;
 }
 void *rsm_device_alloc(size_t bytes) {
@@ -371,6 +382,8 @@ static bool sq_args_ok(Runtime *rt, int pe, int block) {
 int rsm_sq_reset(void) {
   RSM_ENTRY;
   RSM_NEED_RT(rt);
+  if (rsm::live_consumer_running())
+    return rsm::fail("rsm_sq_reset: a live send-queue consumer is running (rsm_sq_consumer_stop first)");
   RSM_HIP(hipDeviceSynchronize());
   rt->reset_queues(nullptr);
   RSM_HIP(hipDeviceSynchronize());

@@ -50,6 +50,14 @@ bool active_set_in_range(int pe_start, int log_pe_stride, int pe_size, int num_p
 // rsm_init makes.  nullptr, with the error set, when the runtime cannot resolve it.
 long *noalloc_flags();
 
+// Stops a live send-queue consumer, if one is running, and releases its stream and control
+// block (drv_consume.hip); rsm_finalize calls it before the runtime is destroyed.
+void consumer_shutdown();
+// True between rsm_sq_consumer_start and rsm_sq_consumer_stop.  A device-wide synchronisation
+// would then wait for the consumer kernel, which runs until it is told to stop: entry points
+// that synchronise the device refuse to run meanwhile (use rsm_stream_synchronize).
+bool live_consumer_running();
+
 // hipGetLastError() after a launch, folded into the error convention.
 int after_launch(const char *what);
 

@@ -106,6 +106,8 @@ __global__ void __launch_bounds__(1024)
     }
     if (fetches && fetched) fetched[i] = got;
   }
+  // One quiet for the workgroup, once all its lanes have issued their operations.
+  __syncthreads();
   if (threadIdx.x == 0) roc_shmem_ctx_quiet(ctx);
   roc_shmem_wg_ctx_destroy(ctx);
   roc_shmem_wg_finalize();

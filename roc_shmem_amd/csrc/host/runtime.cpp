@@ -108,6 +108,11 @@ Options Options::from_env() {
     double d = strtod(s, &end);
     if (end != s && d >= 0) o.wait_limit_s = d;   // 0: waits never give up
   }
+  if (const char *s = getenv("ROC_SHMEM_CONSUMER_IDLE_S")) {
+    char *end = nullptr;
+    double d = strtod(s, &end);
+    if (end != s && d > 0 && d < 1e6) o.consumer_idle_s = d;
+  }
   if (const char *s = getenv("ROC_SHMEM_SQ_MODE")) o.sq_queue_mode = strcmp(s, "queue") == 0;
   if (env_u64("ROC_SHMEM_HEAP_HOST_VISIBLE", &v)) o.heap_host_visible = v != 0;
   return o;
@@ -409,8 +414,12 @@ const TeamRecord *Runtime::team_record(const detail::Team *team) const {
 }
 
 bool Runtime::set_sq_queue_mode(bool queue) {
+  return set_sq_mode(queue ? detail::kSqQueue : detail::kSqLog);
+}
+
+bool Runtime::set_sq_mode(uint32_t mode) {
   (void)hipDeviceSynchronize();
-  state_.sq_queue_mode = queue ? 1u : 0u;
+  state_.sq_queue_mode = mode;
   return upload_state_everywhere(state_);
 }
 

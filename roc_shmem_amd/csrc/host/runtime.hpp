@@ -55,6 +55,8 @@ struct Options {
   size_t slice_pad = 0;            // ROC_SHMEM_SLICE_PAD, extra bytes between slices
   double wait_limit_s = 2.0;       // ROC_SHMEM_WAIT_LIMIT_S, bound of a flag wait; 0 = no limit
   bool sq_queue_mode = false;      // ROC_SHMEM_SQ_MODE=queue: slots are freed by the consumer pass
+  double consumer_idle_s = 5.0;    // ROC_SHMEM_CONSUMER_IDLE_S: a live consumer wave leaves when
+                                   // nothing was published on its rings for this long
   // ROC_SHMEM_HEAP_HOST_VISIBLE (default 1): the arena is fine-grained device memory, which host
   // code can dereference like the reference's heap (hipExtMallocWithFlags, heap_type.hpp:50) and
   // which kernels stream as fast as ordinary device memory; 0: plain hipMalloc.
@@ -113,6 +115,8 @@ class Runtime {
   // slots are freed only by the consumer pass.  Returns false when the state
   // could not be re-uploaded.
   bool set_sq_queue_mode(bool queue);
+  // The same with the mode given as detail::kSqLog / kSqQueue / kSqLive.
+  bool set_sq_mode(uint32_t mode);
   bool sq_queue_mode() const { return state_.sq_queue_mode != 0; }
   const detail::DeviceState &device_state() const { return state_; }
   char *arena() const { return arena_; }

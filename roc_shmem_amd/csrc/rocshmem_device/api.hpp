@@ -173,8 +173,16 @@ __device__ inline void roc_shmem_ctx_fence(roc_shmem_ctx_t) { detail::fence_acq_
 __device__ inline void roc_shmem_ctx_fence(roc_shmem_ctx_t, int) { detail::fence_acq_rel_agent(); }
 __device__ inline void roc_shmem_fence() { detail::fence_acq_rel_agent(); }
 __device__ inline void roc_shmem_fence(int) { detail::fence_acq_rel_agent(); }
-__device__ inline void roc_shmem_ctx_quiet(roc_shmem_ctx_t) { detail::fence_acq_rel_agent(); }
-__device__ inline void roc_shmem_quiet() { detail::fence_acq_rel_agent(); }
+// quiet: everything the calling PE has issued is complete and visible.  The
+// operations themselves are direct stores and atomics, which the fence
+// completes.  With a live consumer on the send queues the call also collects
+// the completions its queue has asked for, as the reference's quiet does
+// (QueuePair::quiet_internal, queue_pair.cpp:118-191).
+__device__ inline void roc_shmem_ctx_quiet(roc_shmem_ctx_t ctx) {
+  detail::fence_acq_rel_agent();
+  if (detail::g_state.sq_queue_mode == detail::kSqLive) detail::quiet_live(detail::ctx_of(ctx));
+}
+__device__ inline void roc_shmem_quiet() { roc_shmem_ctx_quiet(ROC_SHMEM_CTX_DEFAULT); }
 __device__ inline void roc_shmem_ctx_threadfence_system(roc_shmem_ctx_t) {
   __threadfence_system();
 }

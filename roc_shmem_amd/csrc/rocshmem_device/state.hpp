@@ -19,11 +19,14 @@ constexpr int kMaxPes = 128;       // two flag sets of kMaxPes fit ROC_SHMEM_*_S
 constexpr int kSyncSlots = 256;    // longs per pSync slice
 constexpr int kAtomicRetSlots = 4096;  // reference: atomic_return.hpp:34-40
 
+enum : uint32_t { kSqLog = 0, kSqQueue = 1, kSqLive = 2 };
+
 // Sticky status codes written to DeviceState::status[0].
 enum : uint32_t {
   kStatusOk = 0,
   kStatusWaitTimeout = 1,   // a bounded flag wait gave up
   kStatusBadArgument = 2,   // e.g. active set larger than kMaxPes
+  kStatusBadCompletion = 3, // quiet found a completion entry that does not belong to its queue
 };
 
 // Active-set description relative to the world (reference: TeamInfo,
@@ -74,7 +77,9 @@ struct alignas(64) SqCounters {
   uint32_t atomic_counter;  // free-running AMO return-slot index
   uint32_t consumed;        // every WQE below this index has been retired by the consumer pass
   uint32_t cq_producer;     // free-running count of completion entries written
-  uint32_t pad_[11];
+  uint32_t cq_consumer;     // completion entries a reader (quiet) has taken (reference: cq_consumer_counter)
+  uint32_t quiet_counter;   // completions requested from a live consumer and not yet taken by quiet
+  uint32_t pad_[9];
 };
 
 // One context = one (PE, block) pair (reference: GPUIBContext members,
@@ -99,9 +104,12 @@ struct DeviceState {
   Team *team_world;
   uint32_t *status;
   uint64_t wait_limit_ticks;   // wall_clock64() ticks a flag wait may take
-  // 0: a ring is a log, a slot may be rewritten once its previous entry is
-  // published.  1: a ring is a queue, a slot may be rewritten only after the
-  // consumer pass has retired its previous entry.
+  // kSqLog: a ring is a log, a slot may be rewritten once its previous entry
+  // is published.  kSqQueue: a ring is a queue, a slot may be rewritten only
+  // after the consumer pass (run between producer kernels) has retired its
+  // previous entry.  kSqLive: a queue whose consumer runs at the same time as
+  // the producers: entries and completions are written through to memory, and
+  // quiet waits until the ring's entries are retired.
   uint32_t sq_queue_mode;
   uint32_t pad_;
 };
@@ -113,8 +121,8 @@ struct DeviceState {
 // its fingerprint to the library, which refuses to initialise on a mismatch.
 // Bump kStateRevision when a layout changes without changing a size, or when
 // units must agree on how they use shared memory (3: the barrier pool holds
-// call counts, not flags that are reset).
-constexpr uint32_t kStateRevision = 3;
+// call counts, not flags that are reset; 4: live queues, cq_consumer).
+constexpr uint32_t kStateRevision = 4;
 constexpr uint32_t kStateLayout =
     (kStateRevision * 0x01000193u) ^
     static_cast<uint32_t>(sizeof(DeviceState) | (sizeof(DeviceCtx) << 8) | (sizeof(Team) << 16) |

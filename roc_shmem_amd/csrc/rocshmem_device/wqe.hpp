@@ -129,9 +129,16 @@ __device__ __forceinline__ void wave_post_with(DeviceCtx *ctx, bool sends, const
   __amdgpu_buffer_rsrc_t ring_mem = __builtin_amdgcn_make_buffer_rsrc(
       uniform(ring.sq), 0, static_cast<int>(uniform(ring.max_nwqe)) * 64, kRawBufferFlags);
 
+  // A completion is requested by the entry that closes the wave's post (the
+  // multi-thread policy, thread_policy.cpp:170-216) and by the entry in slot
+  // max_nwqe - 2 of every lap (queue_pair.cpp:80-101: the completion queue
+  // must not starve however the posts fall).
+  const uint32_t slot = my_counter & (ring.max_nwqe - 1);
+  const bool wants_cqe = sends && (last || slot == ring.max_nwqe - 2u);
+  const uint32_t n_cqe = __popcll(__ballot(wants_cqe));
+
   uint32_t first8_lo = 0, first8_hi = 0;
   if (sends) {
-    const uint32_t slot = my_counter & (ring.max_nwqe - 1);
     const uint32_t at = slot * 64u;   // byte offset of the entry in the ring
     const uint16_t idx16 = static_cast<uint16_t>(my_counter);
     const bool inl = rq.opcode == kOpcodeRdmaWrite && rq.size <= kInlineThreshold;
@@ -142,7 +149,8 @@ __device__ __forceinline__ void wave_post_with(DeviceCtx *ctx, bool sends, const
     c.x = (static_cast<uint32_t>(rq.opcode) << 24) |
           (static_cast<uint32_t>(__builtin_bswap16(idx16)) << 8);
     c.y = (ds << 24) | ring.ctrl_qp_sq;
-    const uint32_t fm_ce_se = last ? kCqUpdate : static_cast<uint32_t>((ring.ctrl_sig >> 24) & 0xffu);
+    const uint32_t fm_ce_se =
+        wants_cqe ? kCqUpdate : static_cast<uint32_t>((ring.ctrl_sig >> 24) & 0xffu);
     c.z = static_cast<uint32_t>(ring.ctrl_sig & 0xffu) | (fm_ce_se << 24);
     c.w = static_cast<uint32_t>(ring.ctrl_sig >> 32);
     __builtin_amdgcn_raw_buffer_store_b128(c, ring_mem, at, 0, kThrough);
@@ -206,6 +214,10 @@ __device__ __forceinline__ void wave_post_with(DeviceCtx *ctx, bool sends, const
   // before each hand-over.
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   if (last) {
+    // quiet_counter (queue_pair.cpp:80-101): completions asked of a live
+    // consumer that roc_shmem_ctx_quiet has yet to collect.
+    if (g_state.sq_queue_mode == kSqLive)
+      __hip_atomic_fetch_add(&cnt->quiet_counter, n_cqe, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     bounded_wait<uint32_t>(&cnt->published, kWaitEq, base);
     __hip_atomic_store(reinterpret_cast<unsigned long long *>(&ring.mailbox[0]),
                        static_cast<unsigned long long>(be32(base + n)), __ATOMIC_RELAXED,
@@ -218,6 +230,51 @@ __device__ __forceinline__ void wave_post_with(DeviceCtx *ctx, bool sends, const
   }
 }
 
+// quiet on a queue with a live consumer (reference: QueuePair::quiet_internal,
+// queue_pair.cpp:118-191).  Completions arrive in order, so the reader claims
+// every completion requested so far (quiet_counter), polls only the entry of
+// the last one until the consumer has written it - valid when its owner bit
+// equals the lap parity of its running number and its opcode is not "invalid" -
+// then moves the completion queue's consumer index and its doorbell record
+// (mailbox word 2).  The wait is bounded like every other.
+__device__ __forceinline__ void quiet_live(DeviceCtx *ctx) {
+  SqCounters *cnt = ctx->counters;
+  const SqRing &ring = ctx->ring;
+  const uint32_t quiet_val =
+      __hip_atomic_exchange(&cnt->quiet_counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (quiet_val == 0) return;
+  const uint32_t number = __hip_atomic_fetch_add(&cnt->cq_consumer, quiet_val, __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT) +
+                          quiet_val - 1;
+  // last 8 bytes of the completion entry: ... | BE32 qpn | BE16 wqe index | signature | op_own
+  const unsigned long long *tail = reinterpret_cast<const unsigned long long *>(
+      ring.cq + 8ull * (number & (ring.cq_size - 1)) + 7);
+  const uint32_t parity = (number >> ring.cq_log_size) & 1u;
+  uint64_t start = wall_clock64();
+  uint32_t spins = 0;
+  for (;;) {
+    const unsigned long long word =
+        __hip_atomic_load(tail, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t op_own = static_cast<uint32_t>(word >> 56);
+    if ((op_own & 1u) == parity && (op_own >> 4) != 0xFu) {
+      // a requester completion of this queue (opcode 0, the queue's number)
+      if ((op_own >> 4) != 0u ||
+          static_cast<uint32_t>(word) != ((ring.ctrl_qp_sq & 0xffffffu) << 8))
+        status_raise(kStatusBadCompletion);
+      break;
+    }
+    __builtin_amdgcn_s_sleep(1);
+    if ((++spins & 63u) == 0 &&
+        (status_failed() || wall_clock64() - start > g_state.wait_limit_ticks)) {
+      status_raise(kStatusWaitTimeout);
+      break;
+    }
+  }
+  __hip_atomic_store(reinterpret_cast<unsigned long long *>(&ring.mailbox[2]),
+                     static_cast<unsigned long long>(be32(number + 1)), __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // A ring that only one workgroup feeds (at most ROC_SHMEM_NUM_BLOCKS
 // workgroups per PE in the grid) is written with ordinary cached stores.  A
 // ring that several workgroups share may be fed from different XCDs, each
@@ -225,12 +282,15 @@ __device__ __forceinline__ void wave_post_with(DeviceCtx *ctx, bool sends, const
 // (agent-scope stores, sc1), so that a slot two workgroups write one after
 // the other holds the later entry whatever order the L2s are written back
 // in.  Writing through costs a fifth of the small-put rate (10.5 against
-// 13.2 G ops/s for 10 M eight-byte puts), hence the switch.
+// 13.2 G ops/s for 10 M eight-byte puts), hence the switch.  A ring whose
+// consumer runs at the same time as its producers (kSqLive) is written through
+// too: the consumer may sit on another XCD and reads the entries while the
+// producers' kernel is still running.
 __device__ __forceinline__ void wave_post(DeviceCtx *ctx, bool sends, const WqeRequest &rq) {
   const bool shared_ring =
       gridDim.x > static_cast<unsigned>(g_state.num_pes) * static_cast<unsigned>(g_state.num_blocks) ||
       gridDim.y * gridDim.z > 1;
-  if (shared_ring) {
+  if (shared_ring || g_state.sq_queue_mode == kSqLive) {
     wave_post_with<16 /* sc1: write through */>(ctx, sends, rq);
   } else {
     wave_post_with<0>(ctx, sends, rq);

@@ -253,7 +253,8 @@ def test_queue_mode_slots_are_freed_by_the_consumer_pass():
                 assert rs.sq_consumer_state(0, 0)["consumed"] == sq * lap
                 totals = rs.sq_consume()
                 assert totals["retired"] == n_pes * sq and totals["lost"] == 0 and totals["rejected"] == 0
-                assert rs.sq_consumer_state(0, 0) == {"consumed": sq * (lap + 1), "cq_producer": lap + 1}
+                # per lap: the entry in slot sq - 2 and the one that closes the wave's post
+                assert rs.sq_consumer_state(0, 0) == {"consumed": sq * (lap + 1), "cq_producer": 2 * (lap + 1)}
         finally:
             rs.sq_set_mode(False)
         mem.free()
@@ -277,5 +278,112 @@ def test_queue_mode_full_ring_raises_the_status_word_instead_of_hanging():
         assert mem.read(1, 128)[2::4].tolist() == [2] * 32, "the operations themselves still ran"
         rs.sq_set_mode(False)
         mem.free()
+    finally:
+        rs.roc_shmem_finalize()
+
+
+# ---- a consumer that runs while the producers post --------------------------------------
+
+def put_and_add_stream(n_ops, n_pes, words, seed):
+    """8-byte puts to distinct words of the lower halves, fetch-adds anywhere in the upper halves."""
+    rng = np.random.default_rng(seed)
+    ops = np.zeros(n_ops, rs.SMALL_OP_DTYPE)
+    is_put = rng.random(n_ops) < 0.5
+    uniq = rng.permutation(n_pes * (words // 2))[:n_ops]
+    ops["kind"] = np.where(is_put, rs.OP_P64, rs.OP_FADD64)
+    ops["pe"] = np.where(is_put, uniq // (words // 2), rng.integers(0, n_pes, n_ops))
+    ops["offset"] = np.where(is_put, (uniq % (words // 2)) * 8,
+                             (words // 2 + rng.integers(0, 256, n_ops)) * 8)
+    ops["value"] = rng.integers(-(1 << 50), 1 << 50, n_ops)
+    return ops
+
+
+@pytest.mark.parametrize("wgs,wg_size,num_blocks,sq", [(2, 256, 2, 64), (6, 128, 2, 128), (1, 64, 1, 64)])
+def test_live_consumer_retires_entries_while_producers_post(wgs, wg_size, num_blocks, sq):
+    # Rings far smaller than what is posted through them (dozens of laps), several workgroups per
+    # ring in the second shape, two producer kernels in one session: nothing may be lost, producers
+    # must not time out, quiet must have collected every completion.
+    n_pes, words, n_ops = 4, 1 << 15, 40000
+    with runtime(n_pes, heap_size=8 << 20, num_blocks=num_blocks, sq_size=sq):
+        mem = rs.sym_array(words, np.int64, fill=0)
+        heap = oracle.Heap(n_pes, words * 8)
+        stream = rs.Stream()
+        rs.sq_reset()
+        rs.sq_consumer_start()
+        assert rs.sq_consumer_running()
+        devs = []
+        try:
+            with pytest.raises(rs.RocShmemError, match="live send-queue consumer"):
+                rs.synchronize()
+            with pytest.raises(rs.RocShmemError, match="live"):
+                rs.sq_reset()
+            for seed in (31, 32):
+                ops = put_and_add_stream(n_ops, n_pes, words, seed)
+                issue = Issue(n_ops, n_pes, wgs, wg_size, num_blocks)
+                oracle.small_ops(heap, ops, issue.pe)
+                shifted = ops.copy()
+                shifted["offset"] += mem.offset
+                devs.append(rs.device_array(shifted))
+                rs.roc_shmem_small_ops(devs[-1], n_ops, None, rs.Launch(wgs, wg_size, 0, stream))
+            stream.synchronize()
+        finally:
+            totals = rs.sq_consumer_stop()
+        assert not rs.sq_consumer_running()
+        assert rs.take_status() == 0, "a producer's wait for queue space or a quiet gave up"
+        assert totals["retired"] == 2 * n_ops and totals["lost"] == 0 and totals["rejected"] == 0
+        assert totals["bytes"] == 16 * n_ops
+        for p in range(n_pes):
+            assert np.array_equal(mem.read(p), heap.view(p, 0, words, np.int64)), "heap of PE %d" % p
+        for pe in range(n_pes):
+            for block in range(num_blocks):
+                st, cons, reader = rs.sq_state(pe, block), rs.sq_consumer_state(pe, block), rs.cq_reader_state(pe, block)
+                assert st["published"] == st["sq_counter"] == cons["consumed"] > 4 * sq
+                assert reader["quiet_counter"] == 0 and reader["cq_consumer"] == cons["cq_producer"]
+                if wgs <= num_blocks:   # one workgroup per queue: its quiet wrote the record last
+                    assert reader["cq_doorbell_record"] == cons["cq_producer"]
+                # the newest completion entry: owner bit = lap parity of its number, the queue's number
+                number = cons["cq_producer"] - 1
+                cqe = rs.cq_image(pe, block, sq)[number % sq]
+                assert cqe[63] == (number // sq) & 1 and not cqe[:56].any()
+                assert bytes(cqe[57:60]) == rs.sq_constants(pe, block)["ctrl_qp_sq"].to_bytes(3, "little")
+        # the previous mode is back: rings are logs again and a plain pass finds nothing left
+        again = rs.sq_consume()
+        assert again["retired"] == 0
+        for d in devs:
+            d.free()
+        stream.destroy()
+        mem.free()
+
+
+def test_finalize_with_a_running_consumer_stops_it():
+    rs.roc_shmem_init(2, 4 << 20, 1, 64)
+    rs.sq_consumer_start()
+    rs.roc_shmem_finalize()           # must tell the consumer to stop and wait for it, not hang
+    rs.roc_shmem_init(2, 4 << 20, 1, 64)
+    try:
+        assert not rs.sq_consumer_running()
+        rs.sq_consumer_start()
+        assert rs.sq_consumer_stop()["retired"] == 0
+        assert rs.take_status() == 0
+    finally:
+        rs.roc_shmem_finalize()
+
+
+def test_a_consumer_left_alone_leaves_by_itself():
+    # Every wave of the persistent kernel reaches an exit whatever the host does: with nothing
+    # published for ROC_SHMEM_CONSUMER_IDLE_S the waves leave; stop then says so.
+    import time
+    os.environ["ROC_SHMEM_CONSUMER_IDLE_S"] = "0.05"
+    try:
+        rs.roc_shmem_init(2, 4 << 20, 2, 64)
+    finally:
+        del os.environ["ROC_SHMEM_CONSUMER_IDLE_S"]
+    try:
+        rs.sq_consumer_start()
+        time.sleep(0.5)
+        with pytest.raises(rs.RocShmemError, match="had left before the stop request"):
+            rs.sq_consumer_stop()
+        assert not rs.sq_consumer_running()
+        assert rs.take_status() == 0
     finally:
         rs.roc_shmem_finalize()

@@ -102,77 +102,158 @@ def test_config3_sum_max_min_8_slices_2e26(dtype, kind):
                 assert np.array_equal(got, heap.view(0, sample * es, sample, npd))
 
 
-def test_config4_ten_million_small_ops_16_slices_64MiB():
+class Config4:
+    """10 M small operations (8-byte puts to unique words of the lower half of every slice,
+    int64 fetch-adds to random words of the upper half) issued by 1024 workgroups of 256 threads
+    over 16 slices of 64 MiB."""
     n_pes, n_ops, wgs_total, wg_size = 16, 10_000_000, 1024, 256
     slice_bytes = 64 << 20
     words = slice_bytes // 8
     num_blocks = 64
-    with runtime(n_pes, heap_size=256 << 20, num_blocks=num_blocks, sq_size=1024):
-        mem = rs.sym_array(words, np.int64, fill=0)
+
+    def __init__(self):
         rng = np.random.default_rng(4)
+        n_ops, n_pes, words = self.n_ops, self.n_pes, self.words
         ops = np.zeros(n_ops, rs.SMALL_OP_DTYPE)
-        is_put = np.arange(n_ops) % 2 == 0
-        ops["kind"] = np.where(is_put, rs.OP_P64, rs.OP_FADD64)
+        self.is_put = np.arange(n_ops) % 2 == 0
+        ops["kind"] = np.where(self.is_put, rs.OP_P64, rs.OP_FADD64)
         ops["pe"] = rng.integers(0, n_pes, n_ops)
         uniq = rng.permutation(n_pes * (words // 2))[:n_ops]          # puts: unique (pe, word)
-        ops["pe"][is_put] = uniq[is_put] // (words // 2)
-        ops["offset"] = np.where(is_put, (uniq % (words // 2)) * 8,
+        ops["pe"][self.is_put] = uniq[self.is_put] // (words // 2)
+        ops["offset"] = np.where(self.is_put, (uniq % (words // 2)) * 8,
                                  (words // 2 + rng.integers(0, words // 2, n_ops)) * 8)
-        ops["value"] = np.where(is_put, rng.integers(-(1 << 62), 1 << 62, n_ops),
+        ops["value"] = np.where(self.is_put, rng.integers(-(1 << 62), 1 << 62, n_ops),
                                 rng.integers(-1000, 1000, n_ops))
-        shifted = ops.copy()
+        self.ops = ops
+        i = np.arange(n_ops)
+        blk = (i % (self.wgs_total * self.wg_size)) // self.wg_size
+        self.issuer = (blk % n_pes).astype(np.uint32)
+        self.ring = self.issuer.astype(np.int64) * self.num_blocks + (blk // n_pes) % self.num_blocks
+
+    def run(self, mem, launch_stream=None):
+        shifted = self.ops.copy()
         shifted["offset"] += mem.offset
         dev = rs.device_array(shifted)
-        rs.sq_reset()
-        rs.roc_shmem_small_ops(dev, n_ops, None, rs.Launch(wgs_total // n_pes, wg_size))
-        rs.synchronize()
-        # final heap state, bit for bit
-        i = np.arange(n_ops)
-        total_threads = wgs_total * wg_size
-        blk = (i % total_threads) // wg_size
-        issuer = (blk % n_pes).astype(np.uint32)
-        heap = oracle.Heap(n_pes, slice_bytes)
-        oracle.small_ops(heap, ops, issuer)
-        for p in range(n_pes):
-            assert np.array_equal(mem.read(p), heap.view(p, 0, words, np.int64)), "heap of PE %d" % p
-        # every ring: producer indices equal the number of entries its workgroup posted
-        ring_block = (blk // n_pes) % num_blocks
-        per_ring = np.bincount(issuer.astype(np.int64) * num_blocks + ring_block,
-                               minlength=n_pes * num_blocks)
-        per_ring_amo = np.bincount((issuer.astype(np.int64) * num_blocks + ring_block)[~is_put],
-                                   minlength=n_pes * num_blocks)
+        rs.roc_shmem_small_ops(dev, self.n_ops, None,
+                               rs.Launch(self.wgs_total // self.n_pes, self.wg_size, 0, launch_stream))
+        return dev, shifted
+
+    def check_heap(self, mem):
+        heap = oracle.Heap(self.n_pes, self.slice_bytes)
+        oracle.small_ops(heap, self.ops, self.issuer)
+        for p in range(self.n_pes):
+            assert np.array_equal(mem.read(p), heap.view(p, 0, self.words, np.int64)), "heap of PE %d" % p
+
+    def check_rings(self, shifted, sq):
+        """Every entry the rings hold against the CPU builder, byte for byte: all entries when no
+        ring wrapped (then every operation must also be found exactly once), else the newest `sq`
+        of every ring."""
+        n_pes, num_blocks = self.n_pes, self.num_blocks
         base0, stride = rs.heap_base(0), rs.heap_base(1) - rs.heap_base(0)
+        expect = np.zeros(self.n_ops, oracle.WQE_EXPECT_DTYPE)
+        expect["opcode"] = np.where(self.is_put, oracle.OP_WRITE, oracle.OP_ATOMIC_FA)
+        expect["raddr"] = (base0 + shifted["pe"].astype(np.int64) * stride +
+                           shifted["offset"].astype(np.int64)).astype(np.uint64)
+        expect["data"] = shifted["value"].astype(np.int64).view(np.uint64)
+        expect["size"] = 8
+        order = np.argsort(self.ring, kind="stable")
+        bounds = np.searchsorted(self.ring[order], np.arange(n_pes * num_blocks + 1))
+        rkeys = [rs.sq_rkey(p) for p in range(n_pes)]
+        checked = 0
         for pe in range(n_pes):
-            for block in range(0, num_blocks, 9):          # a sample of rings in full detail
+            for block in range(num_blocks):
+                r = pe * num_blocks + block
+                mine = order[bounds[r]:bounds[r + 1]]
                 st = rs.sq_state(pe, block)
-                assert st["sq_counter"] == st["published"] == per_ring[pe * num_blocks + block]
-                assert st["atomic_counter"] == per_ring_amo[pe * num_blocks + block]
-                image = rs.sq_image(pe, block, 1024)
                 count = int(st["sq_counter"])
-                assert count > 1024            # the ring wrapped several times
-                # the ring holds the last 1024 entries: indices form one cyclic run
-                idx = (image[:, 1].astype(np.int64) << 8) | image[:, 2]
-                slot = np.arange(1024)
-                newest = (count - 1) % 1024
-                want = np.where(slot <= newest, count - 1 - (newest - slot),
-                                count - 1 - (newest + 1024 - slot)) & 0xFFFF
-                assert np.array_equal(idx, want)
-                # every entry is one of this ring's operations: check target and operand
-                mine = np.nonzero((issuer == pe) & (ring_block == block))[0]
-                raddr_of = base0 + shifted["pe"][mine].astype(np.int64) * stride + shifted["offset"][mine].astype(np.int64)
-                put_keys = set(zip(raddr_of[is_put[mine]].tolist(), shifted["value"][mine][is_put[mine]].tolist()))
-                amo_keys = set(zip(raddr_of[~is_put[mine]].tolist(), shifted["value"][mine][~is_put[mine]].tolist()))
-                for k in range(0, 1024, 7):
-                    e = image[k]
-                    raddr = int.from_bytes(bytes(e[16:24]), "big")
-                    if e[3] == oracle.OP_WRITE:
-                        val = int.from_bytes(bytes(e[36:44]), "little", signed=True)
-                        assert bytes(e[32:36]) == bytes([0x80, 0, 0, 8]) and (raddr, val) in put_keys
-                    else:
-                        val = int.from_bytes(bytes(e[32:40]), "big", signed=True)
-                        assert e[3] == oracle.OP_ATOMIC_FA and e[7] == 4 and (raddr, val) in amo_keys
-                    dest = (raddr - base0) // stride
-                    assert int.from_bytes(bytes(e[24:28]), "little") == rs.sq_rkey(dest)
+                assert count == st["published"] == len(mine), (pe, block)
+                assert st["atomic_counter"] == int((~self.is_put[mine]).sum())
+                wrapped = count > sq
+                first = count - sq if wrapped else 0
+                image = rs.sq_image(pe, block, sq)
+                c = rs.sq_constants(pe, block)
+                qp = oracle.Qp()
+                qp.ctrl_qp_sq, qp.ctrl_sig, qp.lkey = c["ctrl_qp_sq"], c["ctrl_sig"], c["lkey"]
+                qp.atomic_lkey, qp.atomic_ret_base, qp.max_nwqe = c["atomic_lkey"], c["atomic_ret_base"], sq
+                res = oracle.ring_check(image, qp, first, count - first, oracle.sort_wqe_expect(expect[mine]),
+                                        base0, stride, self.slice_bytes * 4, rkeys, full_slot=not wrapped)
+                assert res["ok"], "ring %d/%d entry %d: %s" % (pe, block, first + res["position"], res["reason"])
+                checked += count - first
+                newest = image[(count - 1) % sq]
+                assert newest[11] == 8, "the entry that closes the last post asks for a completion"
+                assert np.array_equal(st["mailbox"], oracle.doorbell(newest, count))
+                if not wrapped:
+                    assert res["used"].all(), "an operation of ring %d/%d left no entry" % (pe, block)
+                    n_atomic = res["n_atomic"]
+                    dense = n_atomic // 4096 + (np.arange(4096) < n_atomic % 4096)
+                    assert np.array_equal(res["pos_count"], dense), "AMO return slots are handed out densely"
+                    assert not image[count:].any(), "slots beyond the producer index stay untouched"
+        return checked
+
+
+def test_config4_every_ring_entry_of_ten_million_small_ops_byte_exact():
+    # Rings of 16384 entries hold everything a workgroup posts (about 9766 entries each): all
+    # 10 M entries are compared with the CPU builder and every operation is accounted for.
+    cfg = Config4()
+    with runtime(cfg.n_pes, heap_size=256 << 20, num_blocks=cfg.num_blocks, sq_size=16384):
+        mem = rs.sym_array(cfg.words, np.int64, fill=0)
+        rs.sq_reset()
+        dev, shifted = cfg.run(mem)
+        rs.synchronize()
+        cfg.check_heap(mem)
+        assert cfg.check_rings(shifted, 16384) == cfg.n_ops
+        totals = rs.sq_consume()
+        assert totals["retired"] == cfg.n_ops and totals["rejected"] == 0 and totals["lost"] == 0
+        assert totals["writes"] == cfg.n_ops // 2 and totals["atomics"] == cfg.n_ops // 2
+        dev.free()
+
+
+def test_config4_ten_million_small_ops_16_slices_64MiB():
+    # The benchmark's shape: 1024-entry rings that wrap about nine times.  The heap is compared
+    # in full, and all 1 Mi entries that survive in the rings with the CPU builder.
+    cfg = Config4()
+    with runtime(cfg.n_pes, heap_size=256 << 20, num_blocks=cfg.num_blocks, sq_size=1024):
+        mem = rs.sym_array(cfg.words, np.int64, fill=0)
+        rs.sq_reset()
+        dev, shifted = cfg.run(mem)
+        rs.synchronize()
+        cfg.check_heap(mem)
+        assert cfg.check_rings(shifted, 1024) == cfg.n_pes * cfg.num_blocks * 1024
+        dev.free()
+
+
+def test_config4_through_queues_with_a_live_consumer_nothing_lost():
+    # The same stream through 1024-entry rings run as queues: a consumer kernel retires entries
+    # while the producers post, producers wait for space instead of overwriting, quiet collects
+    # the completions.  Every one of the 10 M entries is seen by the consumer.
+    cfg = Config4()
+    with runtime(cfg.n_pes, heap_size=256 << 20, num_blocks=cfg.num_blocks, sq_size=1024):
+        mem = rs.sym_array(cfg.words, np.int64, fill=0)
+        rs.sq_reset()
+        stream = rs.Stream()
+        rs.sq_consumer_start()
+        try:
+            dev, shifted = cfg.run(mem, stream)
+            stream.synchronize()
+        finally:
+            totals = rs.sq_consumer_stop()
+        assert totals["lost"] == 0 and totals["rejected"] == 0, totals
+        assert totals["retired"] == cfg.n_ops and totals["bytes"] == 8 * cfg.n_ops
+        assert totals["writes"] == cfg.n_ops // 2 and totals["atomics"] == cfg.n_ops // 2
+        assert rs.take_status() == 0
+        cfg.check_heap(mem)
+        assert cfg.check_rings(shifted, 1024) == cfg.n_pes * cfg.num_blocks * 1024
+        completions = 0
+        for pe in range(cfg.n_pes):
+            for block in range(cfg.num_blocks):
+                cons, reader = rs.sq_consumer_state(pe, block), rs.cq_reader_state(pe, block)
+                assert cons["consumed"] == rs.sq_state(pe, block)["published"]
+                # quiet took every completion the queue had asked for
+                assert reader == {"cq_consumer": cons["cq_producer"], "quiet_counter": 0,
+                                  "cq_doorbell_record": cons["cq_producer"]}, (pe, block)
+                completions += cons["cq_producer"]
+        assert completions == totals["completions"]
+        stream.destroy()
         dev.free()
 
 

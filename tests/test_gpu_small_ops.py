@@ -135,6 +135,8 @@ def check_rings(shifted_ops, issue, n_pes, num_blocks, sq_size, masked_ce=True):
                                  atomic_data=key[3], atomic_cmp=key[4], inline=key[5], atomic_pos=pos,
                                  request_cqe=bool(slot[11] == 8))
                 assert slot[11] in (8, (qp.ctrl_sig >> 24) & 0xFF)
+                if k == sq_size - 2:
+                    assert slot[11] == 8, "slot max_nwqe - 2 asks for a completion (queue_pair.cpp:80-85)"
                 assert np.array_equal(slot, exp), "ring %d/%d slot %d" % (pe, block, k)
             assert all(v == 0 for v in pending.values())
             assert positions == set(range(n_atomic)), "AMO return slots are handed out densely"
@@ -347,7 +349,7 @@ def test_ring_history_with_wraparound_is_byte_exact():
                     oracle.wqe_build(ring[counter % sq], qp, counter, opcode, size=size, raddr=raddr,
                                      rkey=rs.sq_rkey(int(shifted[i]["pe"])), atomic_data=adata,
                                      atomic_cmp=acmp, inline=inl, atomic_pos=pos,
-                                     request_cqe=(j == len(idx) - 1))
+                                     request_cqe=oracle.requests_cqe(counter, sq, j == len(idx) - 1))
                     counter += 1
             st = rs.sq_state(pe, 0)
             assert st["sq_counter"] == counter and st["published"] == counter

@@ -183,3 +183,150 @@ def test_fetch_incr_known_answers():
         out, counter = oracle.fetch_incr(0xFFFFFFFFFFFFFFFF, counter)
         assert out[1] % 64 == 1
     assert counter == 1048576
+
+
+# ---- the bulk ring checker used by the full-size GPU tests ---------------------------------
+
+BASE0, STRIDE, N_PES = 0x7F1000000000, 1 << 26, 4
+RKEYS = [oracle.bswap32(0x1000 + p) for p in range(N_PES)]
+
+
+def ring_of(q, ops, first_counter=0, closes=64, background=0):
+    """Ring image the scalar builder leaves for `ops` = [(opcode, raddr, data, cmp, size)] posted
+    in that order from running number first_counter; every `closes`-th entry closes a post."""
+    ring = np.full((q.max_nwqe, 64), background, np.uint8)
+    n_atomic = 0
+    for k, (opcode, raddr, data, cmp_, size) in enumerate(ops):
+        c = first_counter + k
+        pos = 0
+        if opcode in (oracle.OP_ATOMIC_FA, oracle.OP_ATOMIC_CS):
+            pos = n_atomic % 4096
+            n_atomic += 1
+        oracle.wqe_build(ring[c % q.max_nwqe], q, c, opcode, size=size, raddr=raddr,
+                         rkey=RKEYS[(raddr - BASE0) // STRIDE], atomic_data=data, atomic_cmp=cmp_,
+                         inline=(data & (2 ** 64 - 1)).to_bytes(8, "little"), atomic_pos=pos,
+                         request_cqe=oracle.requests_cqe(c, q.max_nwqe, (k + 1) % closes == 0 or k == len(ops) - 1))
+    return ring
+
+
+def expect_of(ops):
+    e = np.zeros(len(ops), oracle.WQE_EXPECT_DTYPE)
+    for k, (opcode, raddr, data, cmp_, size) in enumerate(ops):
+        e[k] = (raddr, data & (2 ** 64 - 1), cmp_ & (2 ** 64 - 1), opcode, size)
+    return oracle.sort_wqe_expect(e)
+
+
+def random_ops(rng, n):
+    ops = []
+    for k in range(n):
+        pe = int(rng.integers(0, N_PES))
+        raddr = BASE0 + pe * STRIDE + 8 * int(rng.integers(0, 50))     # collisions on purpose
+        kind = int(rng.integers(0, 3))
+        if kind == 0:
+            ops.append((oracle.OP_WRITE, raddr, int(rng.integers(0, 1 << 63)), 0, int(rng.choice([4, 8]))))
+            if ops[-1][4] == 4:
+                ops[-1] = ops[-1][:2] + (ops[-1][2] & 0xFFFFFFFF,) + ops[-1][3:]
+        elif kind == 1:
+            ops.append((oracle.OP_ATOMIC_FA, raddr, int(rng.integers(0, 4)), 0, 8))
+        else:
+            ops.append((oracle.OP_ATOMIC_CS, raddr, int(rng.integers(0, 1 << 40)), int(rng.integers(0, 3)), 8))
+    return ops
+
+
+def run_check(q, ring, first, count, expect, full):
+    return oracle.ring_check(ring, q, first, count, expect, BASE0, STRIDE, STRIDE, RKEYS, full_slot=full)
+
+
+def test_ring_check_accepts_what_the_builder_writes_and_counts():
+    rng = np.random.default_rng(21)
+    q = qp(n=256)
+    ops = random_ops(rng, 200)
+    ring = ring_of(q, ops, closes=64)
+    res = run_check(q, ring, 0, len(ops), expect_of(ops), full=True)
+    assert res["ok"], res
+    assert res["used"].all()
+    n_atomic = sum(1 for o in ops if o[0] != oracle.OP_WRITE)
+    assert res["n_atomic"] == n_atomic and res["pos_count"][:n_atomic].tolist() == [1] * n_atomic
+    assert res["n_cqe"] == 4                    # entries 63, 127, 191 and the last one (199)
+    # a ring that wrapped: leftover bytes of older entries are not compared, the newest 256 are checked
+    ops = random_ops(rng, 700)
+    ring = ring_of(q, ops, closes=64, background=0)
+    assert not run_check(q, ring, 700 - 256, 256, expect_of(ops), full=True)["ok"]
+    res = run_check(q, ring, 700 - 256, 256, expect_of(ops), full=False)
+    assert res["ok"] and res["used"].sum() == 256
+
+
+def test_ring_check_catches_each_kind_of_damage():
+    rng = np.random.default_rng(22)
+    q = qp(n=256)
+    ops = random_ops(rng, 255)
+    ops[254] = (oracle.OP_WRITE, BASE0 + 3 * STRIDE + 4096, 0x1122334455667788, 0, 8)
+    ops[100] = (oracle.OP_ATOMIC_FA, BASE0 + 2 * STRIDE + 8192, 7, 0, 8)
+    good = ring_of(q, ops, closes=64)
+    expect = expect_of(ops)
+    assert run_check(q, good, 0, 255, expect, True)["ok"]
+
+    def damaged(slot, byte, value=None, xor=None):
+        ring = good.copy()
+        ring[slot, byte] = value if value is not None else ring[slot, byte] ^ xor
+        return run_check(q, ring, 0, 255, expect, True)
+
+    assert damaged(7, 2, xor=1)["reason"] == "index field"
+    assert damaged(7, 3, value=0x10)["reason"] == "opcode"
+    assert damaged(100, 63, xor=4)["reason"] == "AMO return slot outside the window"   # misaligned
+    assert damaged(100, 57, xor=0x80)["reason"] == "AMO return slot outside the window"
+    assert damaged(254, 32, value=0)["reason"] == "not an inline write of 1..8 bytes"
+    assert damaged(9, 11, value=3)["reason"] == "completion flag"
+    assert damaged(254, 11, value=0)["reason"] == "completion flag"                     # slot max_nwqe - 2
+    r = damaged(254, 40, xor=0x10)                                                      # payload byte
+    assert r["reason"].startswith("no operation") and r["position"] == 254
+    assert damaged(100, 23, xor=8)["reason"].startswith("no operation")                 # remote address
+    for byte in (4, 7, 8, 12, 24, 27):                                                  # qpn, DS, sig, imm, rkey
+        r = damaged(100, byte, xor=0x21)
+        assert not r["ok"] and r["reason"] == "bytes differ from the builder's" and r["position"] == 100
+    for byte in (48, 52):                                                               # AMO data segment
+        assert damaged(100, byte, xor=1)["reason"] == "bytes differ from the builder's"
+    assert damaged(254, 50, value=9)["reason"] == "bytes differ from the builder's"     # must stay zero
+    # an entry that appears twice, an operation that is missing from the list
+    ring = good.copy()
+    ring[10] = ring[254]
+    ring[10, 1:3] = [0, 10]
+    r = run_check(q, ring, 0, 255, expect, True)
+    assert not r["ok"]
+    r = run_check(q, good, 0, 255, expect_of(ops[:100] + ops[101:]), True)
+    assert r["reason"].startswith("no operation") and r["position"] == 100
+
+
+def test_bulk_builder_and_threaded_small_ops_agree_with_the_scalar_forms():
+    rng = np.random.default_rng(23)
+    q = qp(n=64)
+    ops = random_ops(rng, 300)
+    reqs = (oracle.WqeReq * len(ops))()
+    ring_a = np.zeros((64, 64), np.uint8)
+    for k, (opcode, raddr, data, cmp_, size) in enumerate(ops):
+        r = reqs[k]
+        r.opcode, r.size, r.raddr, r.rkey = opcode, size, raddr, RKEYS[(raddr - BASE0) // STRIDE]
+        r.atomic_data, r.atomic_cmp, r.atomic_pos, r.request_cqe = data, cmp_, k % 4096, int(k % 7 == 0)
+        for i, b in enumerate((data & (2 ** 64 - 1)).to_bytes(8, "little")):
+            r.inline_bytes[i] = b
+        oracle.wqe_build(ring_a[(5 + k) % 64], q, 5 + k, opcode, size=size, raddr=raddr, rkey=r.rkey,
+                         atomic_data=data, atomic_cmp=cmp_, inline=bytes(r.inline_bytes), atomic_pos=k % 4096,
+                         request_cqe=bool(r.request_cqe))
+    ring_b = np.zeros((64, 64), np.uint8)
+    oracle.wqe_build_many(ring_b, q, 5, reqs)
+    assert np.array_equal(ring_a, ring_b)
+    # threaded puts + fetch-adds leave the heap the sequential model leaves
+    n_pes, words = 4, 4096
+    n = n_pes * (words // 2)                      # puts get distinct words of the lower halves
+    stream = np.zeros(n, oracle.SMALL_OP_DTYPE)
+    is_put = rng.random(n) < 0.5
+    stream["kind"] = np.where(is_put, oracle.OP_P64, oracle.OP_FADD64)
+    uniq = rng.permutation(n)
+    stream["pe"] = np.where(is_put, uniq // (words // 2), rng.integers(0, n_pes, len(stream)))
+    stream["offset"] = np.where(is_put, (uniq % (words // 2)) * 8,
+                                (words // 2 + rng.integers(0, 32, len(stream))) * 8)
+    stream["value"] = rng.integers(-1000, 1000, len(stream))
+    a, b = oracle.Heap(n_pes, words * 8), oracle.Heap(n_pes, words * 8)
+    oracle.small_ops(a, stream, np.zeros(len(stream), np.uint32))
+    oracle.small_ops_mt(b, stream, 6)
+    assert np.array_equal(a.buf, b.buf)
