@@ -24,11 +24,14 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
 
-# HBM bytes per launch of the headline kernel measured with rocprofv3 --pmc:
-# FETCH_SIZE 1 048 810.1 KiB and WRITE_SIZE 2 099 768.7 KiB per dispatch, each scaled by
-# what the same counter reads for a wg-putmem copy of known size (2 GiB read, 2 GiB
-# written: 1 048 667.0 and 2 097 754.6 KiB); see profiles/to_all_float_sum_8pe_2e26.md.
-MEASURED_TRAFFIC_BYTES = 4297372262
+# HBM bytes per launch of the headline kernel come from two rocprofv3 --pmc runs (FETCH_SIZE, then
+# WRITE_SIZE) of `bench.py --counter-pair`, each counter scaled by what it reads for a wg-putmem copy
+# of known size in the same run.  `bench.py --record-traffic FETCH.csv WRITE.csv` turns the two
+# counter files into TRAFFIC_JSON together with a fingerprint of the kernel's sources; when the
+# sources have changed since, `roofline.traffic` is reported as null instead of a stale figure.
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "to_all_float_sum_8pe_2e26.traffic.json")
+KERNEL_SOURCES = ["roc_shmem_amd/csrc/rocshmem_device/reduce.hpp", "roc_shmem_amd/csrc/rocshmem_device/copy.hpp",
+                  "roc_shmem_amd/csrc/rocshmem_device/sync.hpp", "roc_shmem_amd/csrc/cabi/drv_reduce.hip"]
 
 # Launch shapes chosen by measurement on MI355X (256 CUs).
 TO_ALL_LAUNCH = dict(wgs_per_pe=32, wg_size=1024)
@@ -61,18 +64,73 @@ def per_launch_ms(rs, fn, iters):
     return out
 
 
-def hbm_ceilings():
-    """What bare streaming kernels reach on this card (roc_shmem_amd/csrc/probes/hbm_ceiling.hip),
-    run as a child process before this process touches the GPU."""
-    import subprocess
-    probe = os.path.join(ROOT, "roc_shmem_amd", "hbm_ceiling")
-    if not os.path.exists(probe):
-        return {"unavailable": "roc_shmem_amd/hbm_ceiling is not built"}
+def kernel_fingerprint():
+    import hashlib
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic():
+    """(bytes per launch or None, note) from the tracked counter summary."""
     try:
-        out = subprocess.run([probe], capture_output=True, text=True, timeout=120)
-        return json.loads(out.stdout.strip().splitlines()[-1])
-    except Exception as e:
-        return {"unavailable": str(e)}
+        with open(TRAFFIC_JSON) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return None, "no counter summary (%s)" % os.path.relpath(TRAFFIC_JSON, ROOT)
+    if rec.get("kernel_sources_sha256_16") != kernel_fingerprint():
+        return None, "stale: the kernel's sources changed after the counters were read; rerun the --pmc pair"
+    return int(rec["traffic_bytes_per_launch"]), "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/"
+
+
+def record_traffic(fetch_csv, write_csv):
+    """Reads the two rocprofv3 counter files of `bench.py --counter-pair` and writes TRAFFIC_JSON."""
+    import csv
+
+    def mean_kib(path, counter, kernel_prefix):
+        vals = []
+        with open(path, newline="") as f:
+            for row in csv.DictReader(f):
+                if row["Counter_Name"] == counter and row["Kernel_Name"].startswith(kernel_prefix):
+                    vals.append(float(row["Counter_Value"]))
+        if not vals:
+            raise SystemExit("%s: no %s rows for %s" % (path, counter, kernel_prefix))
+        return sum(vals) / len(vals), len(vals)
+
+    known = 8 * (256 << 20)                          # the copy reads and writes 2 GiB
+    reduce_kernel = "void (anonymous namespace)::to_all_kernel<float"
+    copy_kernel = "(anonymous namespace)::rma_kernel"
+    out = {"kernel": "to_all_kernel<float, ROC_SHMEM_SUM, sharded>", "copy_bytes_known": known}
+    total = 0.0
+    for name, path in (("FETCH_SIZE", fetch_csv), ("WRITE_SIZE", write_csv)):
+        k, n_k = mean_kib(path, name, reduce_kernel)
+        c, n_c = mean_kib(path, name, copy_kernel)
+        scale = known / (c * 1024.0)
+        out[name] = {"to_all_kib_per_dispatch": k, "dispatches": n_k, "copy_kib_per_dispatch": c,
+                     "copy_dispatches": n_c, "scale_known_over_counter": scale,
+                     "to_all_bytes": k * 1024.0 * scale}
+        total += k * 1024.0 * scale
+    out["traffic_bytes_per_launch"] = int(round(total))
+    out["algorithmic_bytes_per_launch"] = 2 * 8 * (1 << 26) * 4
+    out["kernel_sources_sha256_16"] = kernel_fingerprint()
+    out["kernel_sources"] = KERNEL_SOURCES
+    with open(TRAFFIC_JSON, "w") as f:
+        json.dump(out, f, indent=1)
+        f.write("\n")
+    print(json.dumps(out))
+
+
+def host_threads():
+    """Threads for the CPU legs: the cores this process may run on, capped by the box's
+    per-GPU share of host cores where the environment states one (OMP_NUM_THREADS)."""
+    avail = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    share = os.environ.get("OMP_NUM_THREADS", "")
+    share = int(share) if share.isdigit() and int(share) > 0 else None
+    used = min(avail, share) if share else avail
+    return used, {"os_cpu_count": os.cpu_count(), "cores_this_process_may_use": avail,
+                  "OMP_NUM_THREADS": share}
 
 
 def device_report():
@@ -153,7 +211,7 @@ def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, c
                     "parity check failed"
         out["parity_checked_elements"] = m
     if cpu:
-        cores = min(16, os.cpu_count() or 1)
+        cores, host = host_threads()
 
         def cpu_rate(threads, passes):
             best = None
@@ -170,12 +228,88 @@ def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, c
                       "sample": "same workload, full size (%d slices x 2^%d %s, sum), CPU oracle "
                                 "chunked over %d host threads, best of 3 passes after one warm-up"
                                 % (n_pes, int(np.log2(n)), np.dtype(npd).name, cores),
+                      "host": host,
                       "one_thread_per_pe": {"value": round(cpu_rate(min(n_pes, cores), 2), 2),
                                             "cores": min(n_pes, cores)},
                       "single_thread": {"value": round(cpu_rate(1, 1), 2), "cores": 1}}
     src.free()
     dst.free()
     psync.free()
+    return out
+
+
+def cpu_other_legs(oracle):
+    """The other two legs of the metric on the host cores, next to the reduction's: what the
+    reference's host-centric path does for them on one node (MPI_Put -> memcpy,
+    MPI_Fetch_and_op -> an atomic add, host_helpers.hpp:52-88, host_templates.hpp:285-307), and
+    the scalar 64-byte WQE builder."""
+    cores, _ = host_threads()
+    out = {}
+    # putmem: 8 PEs each move one 64 MiB message to the next PE's slice
+    n_pes, msg = 8, 64 << 20
+    src = np.full(n_pes * msg, 7, dtype=np.uint8)
+    dst = np.zeros(n_pes * msg, dtype=np.uint8)
+
+    def copy_rate(threads):
+        best = None
+        for i in range(4):
+            t0 = time.perf_counter()
+            oracle.copy_mt(dst, src, threads)
+            dt = time.perf_counter() - t0
+            if i and (best is None or dt < best):
+                best = dt
+        return 2.0 * n_pes * msg / best / 1e9
+
+    out["putmem_64MiB_8pe"] = {"value": round(copy_rate(cores), 2), "unit": "GB/s (read + write)", "cores": cores,
+                               "single_thread": round(copy_rate(1), 2), "kind": "port",
+                               "sample": "8 x 64 MiB memcpy, best of 3 passes after one warm-up"}
+    del src, dst
+    # small operations: 5 M 8-byte puts + 5 M int64 fetch-adds, 16 slices x 64 MiB, random targets
+    n_ops, n_slices, words = 10_000_000, 16, (64 << 20) // 8
+    rng = np.random.default_rng(4)
+    ops = np.zeros(n_ops, oracle.SMALL_OP_DTYPE)
+    is_put = np.arange(n_ops) % 2 == 0
+    ops["kind"] = np.where(is_put, oracle.OP_P64, oracle.OP_FADD64)
+    ops["pe"] = rng.integers(0, n_slices, n_ops)
+    ops["offset"] = np.where(is_put, rng.integers(0, words // 2, n_ops), words // 2 + rng.integers(0, words // 2, n_ops)) * 8
+    ops["value"] = rng.integers(-1000, 1000, n_ops)
+    heap = oracle.Heap(n_slices, 64 << 20)
+    t0 = time.perf_counter()
+    oracle.small_ops(heap, ops[:2_000_000], np.zeros(2_000_000, np.uint32))
+    one = 2_000_000 / (time.perf_counter() - t0) / 1e6
+    best = None
+    for i in range(3):
+        t0 = time.perf_counter()
+        oracle.small_ops_mt(heap, ops, cores)
+        dt = time.perf_counter() - t0
+        if i and (best is None or dt < best):
+            best = dt
+    out["small_ops_put8_fetch_add"] = {"value": round(n_ops / best / 1e6, 1), "unit": "Mops/s", "cores": cores,
+                                       "single_thread": round(one, 1), "kind": "port",
+                                       "sample": "10 M operations (half 8-byte puts, half int64 fetch-adds) on 16 x "
+                                                 "64 MiB host slices with hardware atomics, best of 2 passes after "
+                                                 "one warm-up; single thread: the sequential model on 2 M of them"}
+    del heap
+    # WQE builder: 10 M entries (1 M distinct requests, ten laps) into a 1024-entry ring
+    import ctypes
+    n_req = 1_000_000
+    reqs = (oracle.WqeReq * n_req)()
+    view = np.frombuffer(reqs, dtype=np.uint8).reshape(n_req, ctypes.sizeof(oracle.WqeReq))
+    view[:] = 0
+    view[:, oracle.WqeReq.opcode.offset] = np.where(np.arange(n_req) % 2 == 0, 0x08, 0x12)
+    view[:, oracle.WqeReq.size.offset] = 8
+    raddr = (0x7F0000000000 + rng.integers(0, 1 << 30, n_req) * 8).astype(np.uint64)
+    view[:, oracle.WqeReq.raddr.offset:oracle.WqeReq.raddr.offset + 8] = raddr.view(np.uint8).reshape(n_req, 8)
+    qp = oracle.Qp()
+    qp.ctrl_qp_sq, qp.lkey, qp.atomic_lkey, qp.atomic_ret_base, qp.max_nwqe = 0x000100, 0x2000, 0x3000, 1 << 40, 1024
+    ring = np.zeros(1024 * 64, np.uint8)
+    t0 = time.perf_counter()
+    for lap in range(10):
+        oracle.wqe_build_many(ring, qp, lap * n_req, reqs)
+    out["wqe_build"] = {"value": round(10 * n_req / (time.perf_counter() - t0) / 1e6, 1), "unit": "M entries/s",
+                        "cores": 1, "kind": "port",
+                        "sample": "10 M entries (inline 8-byte writes and fetch-adds alternating) by the scalar "
+                                  "builder into a 1024-entry ring, one thread"}
     return out
 
 
@@ -337,6 +471,50 @@ def bench_small_ops(rs, n_pes, n_ops, wgs_total, wg_size, slice_bytes, seed):
     ms = event_time_ms(rs, coalesced, 3) / 3
     res["putmem8_lane_contiguous"] = {"Mops_per_s": n_ops / ms / 1e3, "ms": ms,
                                       "note": "64 lanes x 8 B coalesced into one 512-byte WQE per wave"}
+    dev.free()
+    # The mixed stream through queues with a live consumer: a consumer kernel retires entries while
+    # the producers post (1024-entry rings, producers wait for space, quiet collects completions).
+    ops = np.zeros(n_ops, rs.SMALL_OP_DTYPE)
+    is_put = np.arange(n_ops) % 2 == 0
+    uniq = rng.permutation(n_pes * (words // 2))[:n_ops]
+    ops["kind"] = np.where(is_put, rs.OP_P64, rs.OP_FADD64)
+    ops["pe"] = np.where(is_put, uniq // (words // 2), rng.integers(0, n_pes, n_ops))
+    ops["offset"] = np.where(is_put, (uniq % (words // 2)) * 8,
+                             (words // 2 + rng.integers(0, words // 2, n_ops)) * 8) + mem.offset
+    ops["value"] = rng.integers(-1000, 1000, n_ops)
+    dev = rs.device_array(ops)
+    stream = rs.Stream()
+    live_launch = rs.Launch(wgs_total // n_pes, wg_size, 0, stream)
+    rs.synchronize()
+    rs.sq_reset()
+    rs.sq_consumer_start()
+    try:
+        rs.roc_shmem_small_ops(dev, n_ops, None, live_launch)
+        stream.synchronize()
+        start, stop, reps = rs.Event(), rs.Event(), 3
+        start.record(stream)
+        for _ in range(reps):
+            rs.roc_shmem_small_ops(dev, n_ops, None, live_launch)
+        stop.record(stream)
+        ms = start.elapsed_ms(stop) / reps
+        stream.synchronize()
+    finally:
+        totals = rs.sq_consumer_stop()
+    if totals["lost"] or totals["rejected"] or totals["retired"] != (reps + 1) * n_ops:
+        raise RuntimeError("live consumer: %r" % (totals,))
+    res["mixed_through_live_queues"] = {"Mops_per_s": n_ops / ms / 1e3, "ms": ms, "retired": totals["retired"],
+                                        "lost": 0, "rejected": 0,
+                                        "note": "1024-entry rings in queue mode, consumer kernel running beside the "
+                                                "producers, entries written through to memory"}
+    start.destroy()
+    stop.destroy()
+    stream.destroy()
+    dev.free()
+    # The same stream once more with the rings as logs, for the consumer pass below.
+    dev = rs.device_array(ops)
+    rs.sq_reset()
+    rs.roc_shmem_small_ops(dev, n_ops, None, launch)
+    rs.synchronize()
     dev.free()
     # Consumer pass over what the last stream left in the rings (each ring keeps its newest
     # sq_size entries): check + complete only, host-timed around the synchronous call.
@@ -557,7 +735,13 @@ def main():
                     help="for rocprofv3: broadcast, alltoall and fcollect over 16 slices x 64 MiB, nothing else")
     ap.add_argument("--alignment", action="store_true",
                     help="large put / broadcast / reduction with shifted source and destination, nothing else")
+    ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no GPU work: read the two rocprofv3 --pmc counter files of --counter-pair runs and "
+                         "write the tracked traffic summary under profiles/")
     args = ap.parse_args()
+    if args.record_traffic:
+        record_traffic(*args.record_traffic)
+        return
     if args.gpus != 1:
         print("bench.py: every PE slice lives in one GPU's HBM; this build measures one GPU only "
               "(--gpus %d is not supported)" % args.gpus, file=sys.stderr)
@@ -597,7 +781,6 @@ def main():
         print(json.dumps({"GBps_by_source_shift/destination_shift_8pe": out}))
         return
     device = device_report() if not args.counter_pair else {}
-    ceilings = hbm_ceilings() if not (args.counter_pair or args.quick) else {}
     # ---- headline: fp32 sum_to_all, 8 slices x 2^26 elements (4 GiB algorithmic traffic) ----
     n_pes, n = 8, 1 << 26
     rs.roc_shmem_init(n_pes, 1 << 30, 64, 1024)
@@ -614,7 +797,15 @@ def main():
     if not args.quick:
         extra["to_all_bf16_sum_8x2^26"] = {k: v for k, v in bench_to_all(
             rs, oracle, max(args.steps // 2, 3), 2, rs.BF16, n_pes, n, seed=3).items() if k != "cpu"}
-        extra["putmem_wg_8pe"] = bench_putmem(rs, 5, n_pes, [8, 4096, 65536, 1 << 20, 64 << 20])
+        # every power of two from 8 B to 64 MiB (BASELINE configs[1]; the reference's own sweep,
+        # clients/functional_tests/tester.cpp:503-563)
+        extra["putmem_wg_8pe"] = bench_putmem(rs, 5, n_pes, [1 << k for k in range(3, 27)])
+        # the unchanged standard call, one per 2^20-element tile, tiles dealt to 64 workgroups per PE
+        extra["to_all_float_sum_8x2^26_standard_api_tiled"] = {
+            k: v for k, v in bench_to_all(rs, oracle, max(args.steps // 2, 3), 2, rs.FLOAT, n_pes, n, seed=3,
+                                          launch_shape=dict(wgs_per_pe=64, wg_size=512, tile=1 << 20)).items()}
+        extra["to_all_float_sum_8x2^26_standard_api_tiled"]["api"] = \
+            "roc_shmem_ctx_float_sum_wg_to_all, one call per tile of 2^20 elements"
         extra["putmem_getmem_per_wave_and_thread_8pe"] = bench_granularities(rs, 5, n_pes)
         extra["collectives_4KiB_8pe_one_wg_of_256"] = bench_small_latencies(rs, n_pes)
     rs.roc_shmem_finalize()
@@ -642,6 +833,9 @@ def main():
         rs.roc_shmem_finalize()
 
     cpu = head.pop("cpu")
+    if not args.quick:
+        cpu["other_legs"] = cpu_other_legs(oracle)
+    traffic, traffic_note = measured_traffic()
     line = {
         "metric": "to_all reduce + putmem GB/s (% of HBM peak); small-put/AMO Mops/s",
         "value": round(head["GBps"], 1),
@@ -657,16 +851,18 @@ def main():
         "data": "synthetic",
         "config": {"workload": "float sum_to_all over 8 PE slices x 2^26 elements, N(0,1) inputs, "
                                "all slices in one GPU's HBM (BASELINE configs[2], fp32 sum)",
+                   "api": "roc_shmemx_ctx_float_sum_wg_to_all_shard (the sharded extension: the 32 workgroups of "
+                          "a PE share one reduction); the unchanged roc_shmem_ctx_float_sum_wg_to_all, tiled over "
+                          "workgroups, is extra.to_all_float_sum_8x2^26_standard_api_tiled",
                    "pes": n_pes, "elements_per_pe": n, "algorithmic_bytes_per_step": head["bytes_per_step"],
                    "launch": TO_ALL_LAUNCH, "parity_checked_elements": head.get("parity_checked_elements")},
         "roofline": {"bound": "hbm", "achieved": round(head["GBps"], 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(head["GBps"] / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES},
+                     "traffic": traffic, "traffic_source": traffic_note},
         "cpu_baseline": {k: (round(v, 2) if isinstance(v, float) else v) for k, v in cpu.items()},
         "per_launch_ms": {"median": round(head["ms_median"], 4), "min": round(head["ms_min"], 4),
                           "max": round(head["ms_max"], 4)},
         "device": device,
-        "hbm_ceilings_of_bare_kernels": ceilings,
         "extra": extra,
     }
     print(json.dumps(line))

@@ -30,6 +30,7 @@ def _load():
     lib.orc_dtype_size.argtypes = [i32]
     lib.orc_to_all.argtypes = [i32, i32, vp, sz, sz, sz, sz, i32, i32, i32]
     lib.orc_to_all_team.argtypes = [i32, i32, vp, sz, sz, sz, sz, i32, i32, i32]
+    lib.orc_to_all_rounded_once.argtypes = [i32, i32, vp, sz, sz, sz, sz, i32, i32, i32]
     lib.orc_to_all_mt.argtypes = [i32, i32, vp, sz, sz, sz, sz, i32, i32, i32, i32]
     lib.orc_to_all_f64.argtypes = [i32, i32, vp, sz, sz, sz, i32, i32, i32, vp]
     lib.orc_abs_sum_f64.argtypes = [i32, vp, sz, sz, sz, i32, i32, i32, vp]
@@ -136,6 +137,19 @@ def to_all(heap, dtype, op, dest_off, src_off, n, pe_start=0, log_stride=0, pe_s
     else:
         rc = _lib.orc_to_all(dtype, op, heap.ptr, heap.stride, dest_off, src_off, n, pe_start,
                              log_stride, pe_size)
+    if rc != 0:
+        raise ValueError("reduction not defined for this (dtype, op)")
+
+
+def to_all_rounded_once(heap, dtype, op, dest_off, src_off, n, pe_start=0, log_stride=0, pe_size=None,
+                        pe_stride=None):
+    """The GPU library's floating-point contract (float sum/prod folded in double, bfloat16 sum in
+    float, ascending member order, one rounding; everything else as ``to_all``): bit-exact
+    expectation for its results."""
+    pe_size = heap.n_pes if pe_size is None else pe_size
+    stride = (1 << log_stride) if pe_stride is None else pe_stride
+    rc = _lib.orc_to_all_rounded_once(dtype, op, heap.ptr, heap.stride, dest_off, src_off, n, pe_start,
+                                      stride, pe_size)
     if rc != 0:
         raise ValueError("reduction not defined for this (dtype, op)")
 

@@ -34,6 +34,10 @@ int orc_to_all(int dtype, int op, char *heap, size_t stride, size_t dest_off, si
 /* Team form: members pe_start + k * pe_stride, any pe_stride >= 1. */
 int orc_to_all_team(int dtype, int op, char *heap, size_t stride, size_t dest_off, size_t src_off,
                     size_t n, int pe_start, int pe_stride, int pe_size);
+/* The GPU library's floating-point contract (float sum/prod folded in double, bfloat16 sum
+ * in float, ascending members, one rounding); see reduce.c. */
+int orc_to_all_rounded_once(int dtype, int op, char *heap, size_t stride, size_t dest_off,
+                            size_t src_off, size_t n, int pe_start, int pe_stride, int pe_size);
 /* Ground truth: the same reduction evaluated in long double on the exact
  * values of the inputs, returned as double.  out[n]. */
 int orc_to_all_f64(int dtype, int op, const char *heap, size_t stride, size_t src_off, size_t n,

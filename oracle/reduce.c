@@ -180,6 +180,56 @@ int orc_to_all_team(int dtype, int op, char *heap, size_t stride, size_t dest_of
   return 0;
 }
 
+/* The arithmetic the GPU library documents for its floating-point reductions,
+ * restated so that its results can be compared bit for bit instead of by
+ * tolerance: float sum and prod are folded in double in ascending member order
+ * and rounded to float once; bfloat16 sum is folded in float and rounded to
+ * bfloat16 once (nearest, ties to even); everything else is the in-type fold of
+ * orc_to_all_team.  This is the library's contract, not the reference's: the
+ * reference folds in the element type in an order that differs per PE and per
+ * algorithm (context_ib_tmpl_device.hpp:120-236) and through MPI_Allreduce on
+ * the host path, so its floating-point bits are not fixed by anything.  Pinned
+ * by the ground truth: wherever the wide fold is exact (eight float terms
+ * within 2^26 of each other, eight bfloat16 terms within 2^13), the result must
+ * be the correctly rounded true sum, i.e. the long-double result of
+ * orc_to_all_f64 rounded to the element type (tests/test_oracle_reduce.py). */
+int orc_to_all_rounded_once(int dtype, int op, char *heap, size_t stride, size_t dest_off,
+                            size_t src_off, size_t n, int pe_start, int pe_stride, int pe_size) {
+  if (!op_defined(dtype, op) || pe_stride < 1) return -1;
+  const int wide_float = dtype == ORC_FLOAT && (op == ORC_SUM || op == ORC_PROD);
+  const int wide_bf16 = dtype == ORC_BF16 && op == ORC_SUM;
+  if (!wide_float && !wide_bf16) {
+    reduce_range(dtype, op, heap, stride, dest_off, src_off, 0, n, pe_start, pe_stride, pe_size);
+    return 0;
+  }
+  const size_t es = orc_dtype_size(dtype);
+  for (size_t i = 0; i < n; ++i) {
+    char out[4];
+    if (wide_float) {
+      double acc = 0;
+      for (int k = 0; k < pe_size; ++k) {
+        float x;
+        memcpy(&x, heap + (size_t)member_pe(k, pe_start, pe_stride) * stride + src_off + i * es, 4);
+        acc = k == 0 ? (double)x : (op == ORC_SUM ? acc + (double)x : acc * (double)x);
+      }
+      float r = (float)acc;
+      memcpy(out, &r, 4);
+    } else {
+      float acc = 0;
+      for (int k = 0; k < pe_size; ++k) {
+        uint16_t b;
+        memcpy(&b, heap + (size_t)member_pe(k, pe_start, pe_stride) * stride + src_off + i * es, 2);
+        acc = k == 0 ? orc_bf16_to_float(b) : acc + orc_bf16_to_float(b);
+      }
+      uint16_t r = orc_float_to_bf16(acc);
+      memcpy(out, &r, 2);
+    }
+    for (int m = 0; m < pe_size; ++m)
+      memcpy(heap + (size_t)member_pe(m, pe_start, pe_stride) * stride + dest_off + i * es, out, es);
+  }
+  return 0;
+}
+
 static long double load_ld(int dtype, const char *p) {
   switch (dtype) {
     case ORC_SHORT: { int16_t v; memcpy(&v, p, 2); return v; }

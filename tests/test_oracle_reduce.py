@@ -198,3 +198,57 @@ def test_undefined_type_operator_pairs_are_refused():
     for dtype, op in ((oracle.FLOAT, oracle.AND), (oracle.DOUBLE, oracle.XOR), (oracle.BF16, oracle.PROD)):
         with pytest.raises(ValueError):
             oracle.to_all(h, dtype, op, 64, 0, 4)
+
+
+def test_rounded_once_fold_is_the_correctly_rounded_true_sum_where_the_wide_fold_is_exact():
+    # float: eight N(0,1) terms lie within 2^26 of each other, so their double sum is exact and the
+    # result must be the true sum rounded to float once; an in-type float fold (rounding after
+    # every step) differs from it in a visible fraction of the elements, so a fold in the wrong
+    # type would fail here.  math.fsum gives the exact sum independently of the oracle.
+    npes, n = 8, 4000
+    rng = np.random.default_rng(7)
+    vals = [rng.standard_normal(n).astype(np.float32) for _ in range(npes)]
+    h, _, off = heap_with(npes, oracle.FLOAT, lambda me: vals[me], n=n)
+    oracle.to_all_rounded_once(h, oracle.FLOAT, oracle.SUM, off, 0, n)
+    exact = np.array([math.fsum(float(v[k]) for v in vals) for k in range(n)])
+    want = exact.astype(np.float32)
+    for p in range(npes):
+        assert np.array_equal(h.view(p, off, n, np.float32), want)
+    assert np.array_equal(oracle.to_all_f64(h, oracle.FLOAT, oracle.SUM, 0, n).astype(np.float32), want)
+    in_type = results(h, oracle.FLOAT, oracle.SUM, n=n)[0]
+    assert (in_type != want).mean() > 0.05
+    # prod of small exactly representable factors: exact in double, so equal to the exact product
+    ints = [rng.integers(1, 8, n).astype(np.float32) / 2 for _ in range(npes)]
+    h, _, off = heap_with(npes, oracle.FLOAT, lambda me: ints[me], n=n)
+    oracle.to_all_rounded_once(h, oracle.FLOAT, oracle.PROD, off, 0, n)
+    assert np.array_equal(h.view(3, off, n, np.float32),
+                          np.prod(np.stack(ints).astype(np.float64), axis=0).astype(np.float32))
+    # bfloat16: eight terms within 2^13 of each other sum exactly in float
+    bvals = [oracle.float_to_bf16(rng.uniform(0.5, 4.0, n).astype(np.float32) * rng.choice([-1, 1], n).astype(np.float32))
+             for _ in range(npes)]
+    h, _, off = heap_with(npes, oracle.BF16, lambda me: bvals[me], n=n)
+    oracle.to_all_rounded_once(h, oracle.BF16, oracle.SUM, off, 0, n)
+    exact = np.array([math.fsum(float(oracle.bf16_to_float(v[k:k + 1])[0]) for v in bvals) for k in range(n)])
+    want = oracle.float_to_bf16(exact.astype(np.float32))
+    for p in range(npes):
+        assert np.array_equal(h.view(p, off, n, np.uint16), want)
+    in_type = results(h, oracle.BF16, oracle.SUM, n=n)[0]
+    assert (in_type != want).mean() > 0.05
+    # everything else is the in-type fold
+    for dtype, op in ((oracle.FLOAT, oracle.MAX), (oracle.BF16, oracle.MIN), (oracle.DOUBLE, oracle.SUM),
+                      (oracle.INT, oracle.PROD)):
+        gen = (lambda me: bvals[me]) if dtype == oracle.BF16 else (lambda me: vals[me] * 1000)
+        h1, _, off = heap_with(npes, dtype, gen, n=n)
+        h2, _, _ = heap_with(npes, dtype, gen, n=n)
+        oracle.to_all(h1, dtype, op, off, 0, n)
+        oracle.to_all_rounded_once(h2, dtype, op, off, 0, n)
+        assert np.array_equal(h1.buf, h2.buf)
+    # active sets and teams address the same members as to_all
+    h1, _, off = heap_with(npes, oracle.FLOAT, lambda me: vals[me], n=n)
+    oracle.to_all_rounded_once(h1, oracle.FLOAT, oracle.SUM, off, 0, n, pe_start=1, log_stride=1, pe_size=3)
+    want = (vals[1].astype(np.float64) + vals[3] + vals[5]).astype(np.float32)
+    assert np.array_equal(h1.view(5, off, n, np.float32), want) and not h1.view(0, off, n, np.float32).any()
+    h1, _, off = heap_with(npes, oracle.FLOAT, lambda me: vals[me], n=n)
+    oracle.to_all_rounded_once(h1, oracle.FLOAT, oracle.SUM, off, 0, n, pe_start=0, pe_stride=3, pe_size=3)
+    want = (vals[0].astype(np.float64) + vals[3] + vals[6]).astype(np.float32)
+    assert np.array_equal(h1.view(6, off, n, np.float32), want)
