@@ -115,6 +115,7 @@ Options Options::from_env() {
   }
   if (const char *s = getenv("ROC_SHMEM_SQ_MODE")) o.sq_queue_mode = strcmp(s, "queue") == 0;
   if (env_u64("ROC_SHMEM_HEAP_HOST_VISIBLE", &v)) o.heap_host_visible = v != 0;
+  if (env_u64("ROC_SHMEM_REBASE_ARGS", &v)) o.rebase_args = v != 0;
   return o;
 }
 
@@ -266,7 +267,9 @@ std::string Runtime::init(const Options &opt) {
                                 ? static_cast<uint64_t>(opt_.wait_limit_s * 100e6)
                                 : ~0ull;
   state_.sq_queue_mode = opt_.sq_queue_mode ? 1u : 0u;
-  state_.pad_ = 0;
+  state_.rebase_args = opt_.rebase_args ? 1u : 0u;
+  state_.arena_bytes = stride_ * static_cast<uint64_t>(P);
+  state_.stride_mask = (stride_ & (stride_ - 1)) == 0 ? stride_ - 1 : 0;
   reset_queues(nullptr);
   if (!state_layouts_agree())
     return "a translation unit of this program was compiled against other device headers than "

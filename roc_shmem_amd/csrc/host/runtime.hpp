@@ -61,6 +61,9 @@ struct Options {
   // code can dereference like the reference's heap (hipExtMallocWithFlags, heap_type.hpp:50) and
   // which kernels stream as fast as ordinary device memory; 0: plain hipMalloc.
   bool heap_host_visible = true;
+  // ROC_SHMEM_REBASE_ARGS (default 1): device calls move symmetric-heap arguments into the
+  // calling PE's slice, so a kernel may pass roc_shmem_malloc's pointer straight through.
+  bool rebase_args = true;
   static Options from_env();
 };
 

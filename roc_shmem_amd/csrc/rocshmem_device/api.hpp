@@ -146,7 +146,8 @@ __device__ inline int roc_shmem_team_translate_pe(roc_shmem_team_t src_team, int
 // Every slice is directly addressable (reference: shmem_ptr returns nullptr
 // when the target is not IPC-mapped, context_ib_device.cpp:128-137).
 __device__ inline void *roc_shmem_ptr(const void *dest, int pe) {
-  return detail::translate(const_cast<void *>(dest), detail::launch_pe(), pe);
+  return detail::translate(detail::own(const_cast<void *>(dest), detail::launch_pe()),
+                           detail::launch_pe(), pe);
 }
 
 // extension: the calling PE's address of the symmetric object that `ptr`
@@ -199,19 +200,23 @@ __device__ inline void roc_shmem_ctx_putmem(roc_shmem_ctx_t ctx, void *dest, con
   // visibility comes with quiet/fence/barrier; the reference adds a device-wide
   // __threadfence here (fence_.flush(), context_ib_device.cpp:164), which on a
   // multi-XCD part means writing back a whole L2 per call.
-  detail::thread_put(detail::ctx_of(ctx), dest, source, nelems, detail::world_pe(ctx, pe));
+  detail::DeviceCtx *c = detail::ctx_of(ctx);
+  detail::thread_put(c, detail::own(dest, c), detail::own(source, c), nelems, detail::world_pe(ctx, pe));
 }
 __device__ inline void roc_shmem_ctx_putmem_nbi(roc_shmem_ctx_t ctx, void *dest,
                                                 const void *source, size_t nelems, int pe) {
-  detail::thread_put(detail::ctx_of(ctx), dest, source, nelems, detail::world_pe(ctx, pe));
+  detail::DeviceCtx *c = detail::ctx_of(ctx);
+  detail::thread_put(c, detail::own(dest, c), detail::own(source, c), nelems, detail::world_pe(ctx, pe));
 }
 __device__ inline void roc_shmem_ctx_getmem(roc_shmem_ctx_t ctx, void *dest, const void *source,
                                             size_t nelems, int pe) {
-  detail::thread_get(detail::ctx_of(ctx), dest, source, nelems, detail::world_pe(ctx, pe));
+  detail::DeviceCtx *c = detail::ctx_of(ctx);
+  detail::thread_get(c, detail::own(dest, c), detail::own(source, c), nelems, detail::world_pe(ctx, pe));
 }
 __device__ inline void roc_shmem_ctx_getmem_nbi(roc_shmem_ctx_t ctx, void *dest,
                                                 const void *source, size_t nelems, int pe) {
-  detail::thread_get(detail::ctx_of(ctx), dest, source, nelems, detail::world_pe(ctx, pe));
+  detail::DeviceCtx *c = detail::ctx_of(ctx);
+  detail::thread_get(c, detail::own(dest, c), detail::own(source, c), nelems, detail::world_pe(ctx, pe));
 }
 __device__ inline void roc_shmem_putmem(void *dest, const void *source, size_t nelems, int pe) {
   roc_shmem_ctx_putmem(ROC_SHMEM_CTX_DEFAULT, dest, source, nelems, pe);
@@ -239,21 +244,28 @@ __device__ inline void roc_shmemx_ctx_putmem_nbi_wg(roc_shmem_ctx_t ctx, void *d
                                                     const void *source, size_t nelems, int pe) {
   if (nelems == 0) return;
   const detail::DeviceCtx *c = detail::ctx_of(ctx);
-  detail::wg_copy(detail::translate(dest, c->my_pe, pe), source, nelems);
+  detail::wg_copy(detail::translate(detail::own(dest, c), c->my_pe, pe), detail::own(source, c), nelems);
 }
 __device__ inline void roc_shmemx_ctx_putmem_wg(roc_shmem_ctx_t ctx, void *dest,
                                                 const void *source, size_t nelems, int pe) {
-  // The source is reusable on return: a lane's loads have returned before its
-  // stores issue, and the lanes meet once all have issued theirs.  Nobody
-  // waits for the stores themselves.
+  // On return the source is reusable and every wave's stores have been taken by
+  // this XCD's L2 (each wave waits for its own, then the waves meet), so one
+  // lane's roc_shmem_ctx_quiet or fence afterwards covers the whole workgroup's
+  // put.  What is not done here is the L2 write-back that makes the bytes
+  // visible to PEs on other XCDs: that is quiet's (the reference flushes in
+  // the put itself, context_ib_device.cpp:148-165,219-236; with one L2 per XCD a
+  // flush per call costs most of the bandwidth of small messages).
   roc_shmemx_ctx_putmem_nbi_wg(ctx, dest, source, nelems, pe);
-  if (nelems != 0) detail::wg_rendezvous();
+  if (nelems != 0) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    detail::wg_rendezvous();
+  }
 }
 __device__ inline void roc_shmemx_ctx_getmem_nbi_wg(roc_shmem_ctx_t ctx, void *dest,
                                                     const void *source, size_t nelems, int pe) {
   if (nelems == 0) return;
   const detail::DeviceCtx *c = detail::ctx_of(ctx);
-  detail::wg_copy(dest, detail::translate(source, c->my_pe, pe), nelems);
+  detail::wg_copy(detail::own(dest, c), detail::translate(detail::own(source, c), c->my_pe, pe), nelems);
 }
 __device__ inline void roc_shmemx_ctx_getmem_wg(roc_shmem_ctx_t ctx, void *dest,
                                                 const void *source, size_t nelems, int pe) {
@@ -272,21 +284,23 @@ __device__ inline void roc_shmemx_ctx_putmem_wg_shard(roc_shmem_ctx_t ctx, void 
                                                       int shard, int nshards) {
   if (nelems == 0) return;
   const detail::DeviceCtx *c = detail::ctx_of(ctx);
-  detail::wg_copy_shard(detail::translate(dest, c->my_pe, pe), source, nelems, shard, nshards);
+  detail::wg_copy_shard(detail::translate(detail::own(dest, c), c->my_pe, pe), detail::own(source, c), nelems,
+                        shard, nshards);
 }
 __device__ inline void roc_shmemx_ctx_getmem_wg_shard(roc_shmem_ctx_t ctx, void *dest,
                                                       const void *source, size_t nelems, int pe,
                                                       int shard, int nshards) {
   if (nelems == 0) return;
   const detail::DeviceCtx *c = detail::ctx_of(ctx);
-  detail::wg_copy_shard(dest, detail::translate(source, c->my_pe, pe), nelems, shard, nshards);
+  detail::wg_copy_shard(detail::own(dest, c), detail::translate(detail::own(source, c), c->my_pe, pe), nelems,
+                        shard, nshards);
 }
 __device__ inline void roc_shmemx_ctx_putmem_nbi_wave(roc_shmem_ctx_t ctx, void *dest,
                                                       const void *source, size_t nelems,
                                                       int pe) {
   if (nelems == 0) return;
   const detail::DeviceCtx *c = detail::ctx_of(ctx);
-  detail::wave_copy(detail::translate(dest, c->my_pe, pe), source, nelems);
+  detail::wave_copy(detail::translate(detail::own(dest, c), c->my_pe, pe), detail::own(source, c), nelems);
 }
 __device__ inline void roc_shmemx_ctx_putmem_wave(roc_shmem_ctx_t ctx, void *dest,
                                                   const void *source, size_t nelems, int pe) {
@@ -299,7 +313,7 @@ __device__ inline void roc_shmemx_ctx_getmem_nbi_wave(roc_shmem_ctx_t ctx, void 
                                                       int pe) {
   if (nelems == 0) return;
   const detail::DeviceCtx *c = detail::ctx_of(ctx);
-  detail::wave_copy(dest, detail::translate(source, c->my_pe, pe), nelems);
+  detail::wave_copy(detail::own(dest, c), detail::translate(detail::own(source, c), c->my_pe, pe), nelems);
 }
 __device__ inline void roc_shmemx_ctx_getmem_wave(roc_shmem_ctx_t ctx, void *dest,
                                                   const void *source, size_t nelems, int pe) {
@@ -378,14 +392,16 @@ ROCSHMEM_X_DEFAULT_CTX_MEM(getmem_nbi_wave)
   }                                                                                            \
   __device__ inline void roc_shmem_ctx_##TNAME##_p(roc_shmem_ctx_t ctx, T *dest, T value,      \
                                                    int pe) {                                   \
-    detail::thread_p<T>(detail::ctx_of(ctx), dest, value, detail::world_pe(ctx, pe));          \
+    detail::DeviceCtx *c = detail::ctx_of(ctx);                                                \
+    detail::thread_p<T>(c, detail::own(dest, c), value, detail::world_pe(ctx, pe));            \
   }                                                                                            \
   __device__ inline void roc_shmem_##TNAME##_p(T *dest, T value, int pe) {                     \
     roc_shmem_ctx_##TNAME##_p(ROC_SHMEM_CTX_DEFAULT, dest, value, pe);                         \
   }                                                                                            \
   __device__ inline T roc_shmem_ctx_##TNAME##_g(roc_shmem_ctx_t ctx, const T *source,          \
                                                 int pe) {                                      \
-    return detail::thread_g<T>(detail::ctx_of(ctx), source, detail::world_pe(ctx, pe));        \
+    detail::DeviceCtx *c = detail::ctx_of(ctx);                                                \
+    return detail::thread_g<T>(c, detail::own(source, c), detail::world_pe(ctx, pe));          \
   }                                                                                            \
   __device__ inline T roc_shmem_##TNAME##_g(const T *source, int pe) {                         \
     return roc_shmem_ctx_##TNAME##_g(ROC_SHMEM_CTX_DEFAULT, source, pe);                       \
@@ -749,12 +765,13 @@ ROCSHMEM_AMO_BITWISE_TYPES(ROCSHMEM_AMO_BITWISE)
 
 #define ROCSHMEM_WAIT(T, TNAME)                                                                \
   __device__ inline void roc_shmem_##TNAME##_wait_until(T *ptr, roc_shmem_cmps cmp, T val) {   \
-    detail::bounded_wait<T>(ptr, static_cast<int>(cmp), val);                                  \
+    detail::bounded_wait<T>(detail::own(ptr, detail::launch_pe()), static_cast<int>(cmp), val); \
     detail::fence_acquire_agent();                                                             \
   }                                                                                            \
   __device__ inline int roc_shmem_##TNAME##_test(T *ptr, roc_shmem_cmps cmp, T val) {          \
     using W = typename detail::WaitWord<T>::type;                                              \
-    W raw = __hip_atomic_load(reinterpret_cast<W *>(ptr), __ATOMIC_RELAXED,                    \
+    W raw = __hip_atomic_load(reinterpret_cast<W *>(detail::own(ptr, detail::launch_pe())),    \
+                              __ATOMIC_RELAXED,                                                \
                               __HIP_MEMORY_SCOPE_AGENT);                                       \
     T have;                                                                                    \
     __builtin_memcpy(&have, &raw, sizeof(T));                                                  \

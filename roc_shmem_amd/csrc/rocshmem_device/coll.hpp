@@ -169,14 +169,14 @@ __device__ __forceinline__ void wg_broadcast_bytes(int my_pe, void *dest, const 
   my_pe = uniform(my_pe);
   shard = uniform(shard);
   nshards = uniform(nshards);
-  dest = uniform(dest);
-  source = uniform(source);
+  dest = own(uniform(dest), my_pe);       // symmetric arguments: the caller's own copies
+  source = own(uniform(source), my_pe);
   nbytes = uniform(nbytes);
   root_idx = uniform(root_idx);
   pe_start = uniform(pe_start);
   pe_stride = uniform(pe_stride);
   pe_size = uniform(pe_size);
-  psync = uniform(psync);
+  psync = own(uniform(psync), my_pe);
   if (nbytes == 0) return;
   if (pe_size > kMaxPes || pe_size <= 0 || root_idx < 0 || root_idx >= pe_size || nshards <= 0 ||
       shard < 0 || shard >= nshards) {
@@ -218,15 +218,15 @@ __device__ __forceinline__ void wg_alltoall_bytes(int my_pe, void *dest, const v
                                                   int pe_start, int pe_stride, int pe_size,
                                                   long *psync) {
   my_pe = uniform(my_pe);
-  dest = uniform(dest);
-  source = uniform(source);
+  dest = own(uniform(dest), my_pe);       // symmetric arguments: the caller's own copies
+  source = own(uniform(source), my_pe);
   block_bytes = uniform(block_bytes);
   shard = uniform(shard);
   nshards = uniform(nshards);
   pe_start = uniform(pe_start);
   pe_stride = uniform(pe_stride);
   pe_size = uniform(pe_size);
-  psync = uniform(psync);
+  psync = own(uniform(psync), my_pe);
   if (block_bytes == 0) return;
   if (pe_size > kMaxPes || pe_size <= 0 || nshards <= 0 || shard < 0 || shard >= nshards) {
     status_raise(kStatusBadArgument);
@@ -297,15 +297,15 @@ __device__ __forceinline__ void wg_fcollect_bytes(int my_pe, void *dest, const v
                                                   int pe_start, int pe_stride, int pe_size,
                                                   long *psync) {
   my_pe = uniform(my_pe);
-  dest = uniform(dest);
-  source = uniform(source);
+  dest = own(uniform(dest), my_pe);       // symmetric arguments: the caller's own copies
+  source = own(uniform(source), my_pe);
   block_bytes = uniform(block_bytes);
   shard = uniform(shard);
   nshards = uniform(nshards);
   pe_start = uniform(pe_start);
   pe_stride = uniform(pe_stride);
   pe_size = uniform(pe_size);
-  psync = uniform(psync);
+  psync = own(uniform(psync), my_pe);
   if (block_bytes == 0) return;
   if (pe_size > kMaxPes || pe_size <= 0 || nshards <= 0 || shard < 0 || shard >= nshards) {
     status_raise(kStatusBadArgument);
@@ -339,7 +339,7 @@ __device__ __forceinline__ void wg_sync_members(int my_pe, int pe_start, int pe_
   pe_start = uniform(pe_start);
   pe_stride = uniform(pe_stride);
   pe_size = uniform(pe_size);
-  psync = uniform(psync);
+  psync = own(uniform(psync), my_pe);
   if (pe_size > kMaxPes || pe_size <= 0) {
     status_raise(kStatusBadArgument);
     return;

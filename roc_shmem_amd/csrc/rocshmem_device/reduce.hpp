@@ -295,13 +295,13 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
                                               int64_t psync_pe_step = 0) {
   // Workgroup-collective: every lane holds the same arguments.
   my_pe = uniform(my_pe);
-  dest = uniform(dest);
-  source = uniform(source);
+  dest = own(uniform(dest), my_pe);       // symmetric arguments: the caller's own copies
+  source = own(uniform(source), my_pe);
   nreduce = uniform(nreduce);
   pe_start = uniform(pe_start);
   pe_stride = uniform(pe_stride);
   pe_size = uniform(pe_size);
-  psync = uniform(psync);
+  psync = own(uniform(psync), my_pe);
   shard = uniform(shard);
   nshards = uniform(nshards);
   psync_pe_step = static_cast<int64_t>(uniform(static_cast<unsigned long>(psync_pe_step)));

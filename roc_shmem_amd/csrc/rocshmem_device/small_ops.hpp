@@ -104,7 +104,7 @@ __device__ __forceinline__ T element_load(const T *p) {
 
 template <typename T>
 __device__ __forceinline__ void thread_p(DeviceCtx *ctx, T *dest, T value, int pe) {
-  T *remote = translate(dest, ctx->my_pe, pe);
+  T *remote = translate(own(dest, ctx), ctx->my_pe, pe);
   element_store(remote, value);
   uint64_t bits = 0;
   __builtin_memcpy(&bits, &value, sizeof(T));
@@ -249,7 +249,7 @@ __device__ __forceinline__ T wave_fetch_add(T *remote, T value) {
 
 template <typename T>
 __device__ __forceinline__ T amo_fetch_add(DeviceCtx *ctx, T *dest, T value, int pe) {
-  T *remote = translate(dest, ctx->my_pe, pe);
+  T *remote = translate(own(dest, ctx), ctx->my_pe, pe);
   const T old = wave_fetch_add(remote, value);
   amo_record<T>(ctx, kOpcodeAtomicFa, remote, value, T(0), pe);
   return old;
@@ -257,7 +257,7 @@ __device__ __forceinline__ T amo_fetch_add(DeviceCtx *ctx, T *dest, T value, int
 
 template <typename T>
 __device__ __forceinline__ void amo_add(DeviceCtx *ctx, T *dest, T value, int pe) {
-  T *remote = translate(dest, ctx->my_pe, pe);
+  T *remote = translate(own(dest, ctx), ctx->my_pe, pe);
   (void)wave_fetch_add(remote, value);
   amo_record<T>(ctx, kOpcodeAtomicFa, remote, value, T(0), pe);
 }
@@ -265,7 +265,7 @@ __device__ __forceinline__ void amo_add(DeviceCtx *ctx, T *dest, T value, int pe
 // compare_swap(dest, cond, value): store `value` iff *dest == cond; returns the old value.
 template <typename T>
 __device__ __forceinline__ T amo_fetch_cas(DeviceCtx *ctx, T *dest, T value, T cond, int pe) {
-  T *remote = translate(dest, ctx->my_pe, pe);
+  T *remote = translate(own(dest, ctx), ctx->my_pe, pe);
   using W = typename AtomicWord<T>::type;
   W expected, desired;
   __builtin_memcpy(&expected, &cond, sizeof(T));
@@ -286,7 +286,7 @@ __device__ __forceinline__ T amo_fetch_cas(DeviceCtx *ctx, T *dest, T value, T c
 // would post: a compare-and-swap with compare operand 0.
 template <typename T>
 __device__ __forceinline__ T amo_swap(DeviceCtx *ctx, T *dest, T value, int pe) {
-  T *remote = translate(dest, ctx->my_pe, pe);
+  T *remote = translate(own(dest, ctx), ctx->my_pe, pe);
   using W = typename AtomicWord<T>::type;
   W desired;
   __builtin_memcpy(&desired, &value, sizeof(T));
@@ -301,7 +301,7 @@ __device__ __forceinline__ T amo_swap(DeviceCtx *ctx, T *dest, T value, int pe) 
 template <typename T>
 __device__ __forceinline__ T amo_fetch(DeviceCtx *ctx, T *dest, int pe) {
   // reference: fetch == fetch_add(0), roc_shmem_gpu.cpp:589-598
-  T *remote = translate(dest, ctx->my_pe, pe);
+  T *remote = translate(own(dest, ctx), ctx->my_pe, pe);
   using W = typename AtomicWord<T>::type;
   W raw = __hip_atomic_load(reinterpret_cast<W *>(remote), __ATOMIC_RELAXED,
                             __HIP_MEMORY_SCOPE_AGENT);
@@ -317,7 +317,7 @@ enum BitOp { kBitAnd, kBitOr, kBitXor };
 // context_ib_tmpl_device.hpp:408-445); they run natively and leave no WQE.
 template <typename T, int Op>
 __device__ __forceinline__ T amo_fetch_bitwise(DeviceCtx *ctx, T *dest, T value, int pe) {
-  T *remote = translate(dest, ctx->my_pe, pe);
+  T *remote = translate(own(dest, ctx), ctx->my_pe, pe);
   if constexpr (Op == kBitAnd)
     return __hip_atomic_fetch_and(remote, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   else if constexpr (Op == kBitOr)

@@ -111,7 +111,12 @@ struct DeviceState {
   // the producers: entries and completions are written through to memory, and
   // quiet waits until the ring's entries are retired.
   uint32_t sq_queue_mode;
-  uint32_t pad_;
+  // 1: roc_shmem_* calls move symmetric-heap arguments into the calling PE's
+  // slice before they use them (one kernel argument then serves the workgroups
+  // of every PE); 0: arguments are used as given.
+  uint32_t rebase_args;
+  uint64_t arena_bytes;        // num_pes * slice_stride
+  uint64_t stride_mask;        // slice_stride - 1 when the stride is a power of two, else 0
 };
 
 // Fingerprint of the structures device code and the host library share.  Device
@@ -121,8 +126,9 @@ struct DeviceState {
 // its fingerprint to the library, which refuses to initialise on a mismatch.
 // Bump kStateRevision when a layout changes without changing a size, or when
 // units must agree on how they use shared memory (3: the barrier pool holds
-// call counts, not flags that are reset; 4: live queues, cq_consumer).
-constexpr uint32_t kStateRevision = 4;
+// call counts, not flags that are reset; 4: live queues, cq_consumer;
+// 5: arguments rebased into the caller's slice).
+constexpr uint32_t kStateRevision = 5;
 constexpr uint32_t kStateLayout =
     (kStateRevision * 0x01000193u) ^
     static_cast<uint32_t>(sizeof(DeviceState) | (sizeof(DeviceCtx) << 8) | (sizeof(Team) << 16) |

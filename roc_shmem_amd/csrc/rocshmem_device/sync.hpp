@@ -49,6 +49,31 @@ __device__ __forceinline__ T *translate(T *ptr, int from_pe, int to_pe) {
       reinterpret_cast<uintptr_t>(ptr) + static_cast<uintptr_t>(delta));
 }
 
+// The calling PE's address of the symmetric object that `ptr` names in any
+// PE's slice; pointers outside the symmetric heap (and every pointer when
+// DeviceState::rebase_args is off) come back unchanged.  All PEs live in one
+// process, so a kernel argument holds one value for the workgroups of every
+// PE - the address roc_shmem_malloc returned, which lies in one PE's slice.
+// The roc_shmem_* calls pass their symmetric and local buffer arguments through
+// this, which lets a kernel written for the reference (one process per PE,
+// every process passing its own address: reduction_tester.cpp:74-104,
+// primitive_tester.cpp:32-82) run unchanged.  An address inside the caller's
+// own slice maps to itself.
+template <typename T>
+__device__ __forceinline__ T *own(T *ptr, int my_pe) {
+  const uint64_t rel =
+      reinterpret_cast<uint64_t>(ptr) - reinterpret_cast<uint64_t>(g_state.heap_base0);
+  if (!g_state.rebase_args || rel >= g_state.arena_bytes) return ptr;   // below the arena: rel wraps
+  const uint64_t off = g_state.stride_mask ? (rel & g_state.stride_mask) : rel % g_state.slice_stride;
+  return reinterpret_cast<T *>(const_cast<char *>(g_state.heap_base0) +
+                               static_cast<uint64_t>(my_pe) * g_state.slice_stride + off);
+}
+template <typename T>
+__device__ __forceinline__ T *own(T *ptr, const DeviceCtx *c) {
+  return own(ptr, c->my_pe);
+}
+
+
 enum WaitCmp { kWaitEq, kWaitNe, kWaitGt, kWaitGe, kWaitLt, kWaitLe };
 
 template <typename T>

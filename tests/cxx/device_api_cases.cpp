@@ -4,8 +4,10 @@
 // hosts every PE": the grid carries the workgroups of all PEs
 // (blockIdx.x % n_pes is the PE, blockIdx.x / n_pes the workgroup's index within
 // it, where the reference uses blockIdx.x), kernel arguments that name
-// symmetric objects pass through roc_shmemx_my_addr, and "only rank 0
-// launches" becomes "only PE 0's workgroups act".
+// symmetric objects and are dereferenced by the kernel itself pass through
+// roc_shmemx_my_addr (the library's calls find the caller's copy themselves, see
+// reference_kernels_unchanged), and "only rank 0 launches" becomes "only PE 0's
+// workgroups act".
 // Exit code 0 and a final line "DEVICE_API_OK" mean every case passed.
 #include <cstdio>
 #include <cstdlib>
@@ -1041,6 +1043,188 @@ static void back_to_back_collectives() {
   roc_shmem_free(src);
 }
 
+// ---- reduction_tester.cpp:74-104 and primitive_tester.cpp:32-82, kernels unchanged ---------
+// The reference's tester kernels hand the pointers roc_shmem_malloc returned straight to the
+// library: every process passes its own address.  Here one value serves the workgroups of
+// every PE (it lies in PE 0's slice), and the roc_shmem_* calls move it into the caller's
+// slice themselves, so the kernels below contain no roc_shmemx_my_addr.  Only the grid
+// differs from the reference's launch (one workgroup per PE instead of one per process).
+__global__ void ReductionTestUnchanged(int loop, int skip, uint64_t *timer, int *s_buf, int *r_buf,
+                                       int *pWrk, long *pSync, int size) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  int n_pes = roc_shmem_ctx_n_pes(ctx);
+  __syncthreads();
+  uint64_t start = 0;
+  for (int i = 0; i < loop + skip; i++) {
+    if (i == skip && hipThreadIdx_x == 0) start = roc_shmem_timer();
+    roc_shmem_ctx_int_sum_wg_to_all(ctx, r_buf, s_buf, size, 0, 0, n_pes, pWrk, pSync);
+    roc_shmem_ctx_wg_barrier_all(ctx);
+  }
+  __syncthreads();
+  if (hipThreadIdx_x == 0) timer[hipBlockIdx_x] = roc_shmem_timer() - start;
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+__global__ void PrimitiveTestUnchanged(int loop, char *s_buf, char *r_buf, long *counter, long *flag,
+                                       int size, int type) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  const int me = roc_shmem_ctx_my_pe(ctx), np = roc_shmem_ctx_n_pes(ctx);
+  if (hipThreadIdx_x == 0) {
+    for (int i = 0; i < loop; i++) {
+      switch (type) {
+        case 0: roc_shmem_ctx_putmem(ctx, r_buf, s_buf, size, (me + 1) % np); break;
+        case 1: roc_shmem_ctx_getmem(ctx, r_buf, s_buf, size, (me + 1) % np); break;
+        case 2: roc_shmem_ctx_putmem_nbi(ctx, r_buf, s_buf, size, (me + 1) % np); break;
+        default: roc_shmem_ctx_getmem_nbi(ctx, r_buf, s_buf, size, (me + 1) % np); break;
+      }
+    }
+    roc_shmem_ctx_long_atomic_add(ctx, counter, me + 1, 0);
+    roc_shmem_ctx_quiet(ctx);
+    // tell the neighbour, wait for the other neighbour: p and wait_until on symmetric words
+    roc_shmem_ctx_long_p(ctx, flag, me + 100, (me + 1) % np);
+    roc_shmem_long_wait_until(flag, ROC_SHMEM_CMP_EQ, (me + np - 1) % np + 100);
+  }
+  __syncthreads();
+  roc_shmemx_ctx_putmem_wg(ctx, r_buf + size, s_buf, size, (me + 1) % np);
+  roc_shmem_ctx_quiet(ctx);
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+static void reference_kernels_unchanged() {
+  current_case = "tester kernels without roc_shmemx_my_addr";
+  const int size = 3000;
+  int *s_buf = static_cast<int *>(roc_shmem_malloc(size * sizeof(int)));
+  int *r_buf = static_cast<int *>(roc_shmem_malloc(size * sizeof(int)));
+  int *pWrk = static_cast<int *>(roc_shmem_malloc(ROC_SHMEM_REDUCE_MIN_WRKDATA_SIZE * sizeof(int)));
+  long *pSync = static_cast<long *>(roc_shmem_malloc(ROC_SHMEM_REDUCE_SYNC_SIZE * sizeof(long)));
+  uint64_t *timer;
+  EXPECT(hipMalloc(&timer, npes * sizeof(uint64_t)) == hipSuccess, "hipMalloc");
+  std::vector<int> v(size);
+  for (int pe = 0; pe < npes; ++pe) {
+    for (int k = 0; k < size; ++k) v[k] = (pe + 1) * 1000 + k;
+    roc_shmem_putmem(s_buf, v.data(), size * sizeof(int), pe);
+    fill(r_buf, size, -1, pe);
+    fill(pSync, static_cast<int>(ROC_SHMEM_REDUCE_SYNC_SIZE), 0L, pe);
+  }
+  ReductionTestUnchanged<<<npes, 256>>>(5, 2, timer, s_buf, r_buf, pWrk, pSync, size);
+  finish_kernel("ReductionTestUnchanged");
+  for (int pe = 0; pe < npes; ++pe) {
+    std::vector<int> got = load(r_buf, size, pe);
+    for (int k = 0; k < size; ++k) {
+      const int want = 1000 * npes * (npes + 1) / 2 + npes * k;
+      if (got[k] != want) {
+        EXPECT(false, "PE %d r_buf[%d] = %d, expected %d", pe, k, got[k], want);
+        break;
+      }
+    }
+  }
+  roc_shmem_free(pSync);
+  roc_shmem_free(pWrk);
+  roc_shmem_free(r_buf);
+  roc_shmem_free(s_buf);
+  EXPECT(hipFree(timer) == hipSuccess, "hipFree");
+
+  const int bytes = 5000;
+  char *cs = static_cast<char *>(roc_shmem_malloc(bytes));
+  char *cr = static_cast<char *>(roc_shmem_malloc(2 * bytes));
+  long *counter = static_cast<long *>(roc_shmem_malloc(sizeof(long)));
+  long *flag = static_cast<long *>(roc_shmem_malloc(sizeof(long)));
+  for (int type = 0; type < 4; ++type) {
+    std::vector<char> c(bytes);
+    for (int pe = 0; pe < npes; ++pe) {
+      for (int k = 0; k < bytes; ++k) c[k] = static_cast<char>(pe * 31 + k * 7 + type);
+      roc_shmem_putmem(cs, c.data(), bytes, pe);
+      fill(cr, 2 * bytes, static_cast<char>(0x55), pe);
+      fill(counter, 1, 0L, pe);
+      fill(flag, 1, 0L, pe);
+    }
+    PrimitiveTestUnchanged<<<npes, 128>>>(2, cs, cr, counter, flag, bytes, type);
+    finish_kernel("PrimitiveTestUnchanged");
+    const bool is_put = type == 0 || type == 2;
+    for (int pe = 0; pe < npes; ++pe) {
+      // put: PE pe holds what its left neighbour sent; get: what its right neighbour owns
+      const int from = is_put ? (pe + npes - 1) % npes : (pe + 1) % npes;
+      const int from_wg = (pe + npes - 1) % npes;        // the workgroup put is always a put
+      std::vector<char> got = load(cr, 2 * bytes, pe);
+      for (int k = 0; k < bytes; ++k) {
+        if (got[k] != static_cast<char>(from * 31 + k * 7 + type) ||
+            got[bytes + k] != static_cast<char>(from_wg * 31 + k * 7 + type)) {
+          EXPECT(false, "type %d PE %d byte %d", type, pe, k);
+          break;
+        }
+      }
+      EXPECT(load(flag, 1, pe)[0] == (pe + npes - 1) % npes + 100, "flag on PE %d", pe);
+    }
+    EXPECT(load(counter, 1, 0)[0] == static_cast<long>(npes) * (npes + 1) / 2, "counter on PE 0 = %ld",
+           load(counter, 1, 0)[0]);
+  }
+  roc_shmem_free(flag);
+  roc_shmem_free(counter);
+  roc_shmem_free(cr);
+  roc_shmem_free(cs);
+}
+
+// ---- blocking put, quiet, flag: the payload is there when the flag is ----------------------
+// Reference: putmem_wg completes and flushes before it returns (context_ib_device.cpp:
+// 148-165,219-236).  Here a blocking put gives local completion and quiet makes it visible:
+// PE p puts 64 KiB into PE p+1 (another XCD, another L2), calls quiet, then sets a flag there
+// with p; PE p+1 waits for the flag and must find every byte of the payload.
+__global__ void PutQuietFlagTest(int rounds, char *s_buf, char *r_buf, long *flag, int size, int *errors) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  const int me = roc_shmem_ctx_my_pe(ctx), np = roc_shmem_ctx_n_pes(ctx);
+  const int right = (me + 1) % np, left = (me + np - 1) % np;
+  s_buf = roc_shmemx_my_addr(s_buf);      // dereferenced below, not only passed to the library
+  r_buf = roc_shmemx_my_addr(r_buf);
+  int bad = 0;
+  for (int r = 1; r <= rounds; ++r) {
+    for (int k = threadIdx.x; k < size; k += blockDim.x) s_buf[k] = static_cast<char>(me * 17 + k + r);
+    __syncthreads();
+    roc_shmemx_ctx_putmem_wg(ctx, r_buf, s_buf, size, right);
+    if (threadIdx.x == 0) {
+      roc_shmem_ctx_quiet(ctx);
+      roc_shmem_ctx_long_p(ctx, flag, r, right);
+      roc_shmem_long_wait_until(flag, ROC_SHMEM_CMP_EQ, r);
+    }
+    __syncthreads();
+    for (int k = threadIdx.x; k < size; k += blockDim.x)
+      if (r_buf[k] != static_cast<char>(left * 17 + k + r)) ++bad;
+    // nobody overwrites r_buf before its owner has checked it
+    roc_shmem_ctx_wg_barrier_all(ctx);
+  }
+  if (bad) atomicAdd(errors, bad);
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+static void put_quiet_flag() {
+  current_case = "blocking put + quiet, then a flag";
+  const int size = 64 << 10, rounds = 20;
+  char *s_buf = static_cast<char *>(roc_shmem_malloc(size));
+  char *r_buf = static_cast<char *>(roc_shmem_malloc(size));
+  long *flag = static_cast<long *>(roc_shmem_malloc(sizeof(long)));
+  int *errors;
+  EXPECT(hipMalloc(&errors, sizeof(int)) == hipSuccess, "hipMalloc");
+  EXPECT(hipMemset(errors, 0, sizeof(int)) == hipSuccess, "hipMemset");
+  for (int pe = 0; pe < npes; ++pe) fill(flag, 1, 0L, pe);
+  PutQuietFlagTest<<<npes, 1024>>>(rounds, s_buf, r_buf, flag, size, errors);
+  finish_kernel("PutQuietFlagTest");
+  int bad = -1;
+  EXPECT(hipMemcpy(&bad, errors, sizeof(int), hipMemcpyDeviceToHost) == hipSuccess, "copy");
+  EXPECT(bad == 0, "%d payload bytes were not there when the flag was", bad);
+  EXPECT(hipFree(errors) == hipSuccess, "hipFree");
+  roc_shmem_free(flag);
+  roc_shmem_free(r_buf);
+  roc_shmem_free(s_buf);
+}
+
 int main() {
   if (!getenv("ROC_SHMEM_NUM_PES")) setenv("ROC_SHMEM_NUM_PES", "4", 1);
   setenv("ROC_SHMEM_HEAP_SIZE", "67108864", 0);
@@ -1058,11 +1242,13 @@ int main() {
                {"random_access", random_access},
                {"default_ctx", default_ctx},   {"primitive_mr", primitive_mr},
                {"primitive_amo", primitive_amo},
-               {"back_to_back_collectives", back_to_back_collectives}};
+               {"back_to_back_collectives", back_to_back_collectives},
+               {"reference_kernels_unchanged", reference_kernels_unchanged},
+               {"put_quiet_flag", put_quiet_flag}};
   for (auto &c : cases) {
     const int before = failures;
     c.run();
-    printf("%-20s %s\n", c.name, failures == before ? "ok" : "FAILED");
+    printf("%-28s %s\n", c.name, failures == before ? "ok" : "FAILED");
     fflush(stdout);
   }
   roc_shmem_finalize();

@@ -64,13 +64,16 @@ def test_reference_host_programs_restated(num_pes):
 
 
 @pytest.mark.gpu
-def test_reference_functional_testers_restated():
+@pytest.mark.parametrize("num_pes", [4, 8])
+def test_reference_functional_testers_restated(num_pes):
     # tests/cxx/device_api_cases.cpp: user kernels in the style of clients/functional_tests.
+    # With 8 PEs the members of every exchange sit on eight different XCDs.
     if not os.path.exists(DEVICE_BINARY):
         pytest.fail("tests/cxx/device_api_cases is not built: run __graft_entry__.build()")
     assert os.path.getmtime(DEVICE_BINARY) >= newest_header(), "stale check program: run __graft_entry__.build()"
-    print("running", DEVICE_BINARY, flush=True)
-    out = subprocess.run([DEVICE_BINARY], capture_output=True, text=True, timeout=110)
+    print("running", DEVICE_BINARY, "with", num_pes, "PEs", flush=True)
+    env = dict(os.environ, ROC_SHMEM_NUM_PES=str(num_pes))
+    out = subprocess.run([DEVICE_BINARY], capture_output=True, text=True, timeout=110, env=env)
     tail = (out.stdout + out.stderr)[-3000:]
     print(out.stdout[-1500:], flush=True)
     assert out.returncode == 0, tail
