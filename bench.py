@@ -35,7 +35,12 @@ KERNEL_SOURCES = ["roc_shmem_amd/csrc/rocshmem_device/reduce.hpp", "roc_shmem_am
 
 # Launch shapes chosen by measurement on MI355X (256 CUs).
 TO_ALL_LAUNCH = dict(wgs_per_pe=32, wg_size=1024)
+# Shapes the pacing tuner is tried with: running free, 32 x 1024 per PE is best; paced, 32 x 512.
+TUNE_SHAPES = (dict(wgs_per_pe=32, wg_size=1024), dict(wgs_per_pe=32, wg_size=512))
 PUT_LAUNCH = dict(wgs_per_pe=32, wg_size=512)
+# one large message shared by the PE's workgroups (sharded extension): 1024-lane workgroups
+# (6.36 against 6.17 TB/s with 512 lanes; standard 256 KiB calls prefer 512: 6.12 against 5.87)
+PUT_SHARED_LAUNCH = dict(wgs_per_pe=32, wg_size=1024)
 PUT_TILE = 256 << 10
 
 
@@ -146,14 +151,17 @@ def device_report():
 
 
 def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, cpu=False,
-                 spread=False, launch_shape=None):
-    """Returns a dict with ms_per_step, GB/s (algorithmic 2*P*N*s bytes) and optional CPU figures."""
+                 spread=False, launch_shape=None, tune=False, pace=0):
+    """Returns a dict with ms_per_step, GB/s (algorithmic 2*P*N*s bytes) and optional CPU figures.
+    tune: let the library measure, outside the timed region, whether pacing its workgroups in
+    lockstep pays for this reduction on this card, with the launch shapes of TUNE_SHAPES; the
+    timed steps then run with the better shape and the rate the tuner set (0 = free running)."""
     npd = rs.NP_DTYPE[dtype]
     es = np.dtype(npd).itemsize
     src = rs.sym_array(n, npd)
     dst = rs.sym_array(n, npd, fill=0x5A)
     launch = rs.Launch(**(launch_shape or TO_ALL_LAUNCH))
-    psync = rs.sym_array(launch.wgs_per_pe * rs.ROC_SHMEM_REDUCE_SYNC_SIZE, np.int64, fill=0)
+    psync = rs.sym_array(max(launch.wgs_per_pe, 64) * rs.ROC_SHMEM_REDUCE_SYNC_SIZE, np.int64, fill=0)
     rng = np.random.default_rng(seed)
     host = []
     for p in range(n_pes):
@@ -169,6 +177,18 @@ def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, c
     def step():
         rs.roc_shmem_to_all(dtype, rs.SUM, dst, src, n, 0, 0, n_pes, None, psync, launch)
 
+    tuning = None
+    rs.set_pacing(0, pace)
+    if tune:
+        tuning, best = {}, None
+        for shape in TUNE_SHAPES:
+            rs.set_pacing(0, 0)
+            res = rs.tune_reduce_pacing(dtype, rs.SUM, dst, src, n, 0, 0, n_pes, psync, rs.Launch(**shape))
+            tuning["%dx%d" % (shape["wgs_per_pe"], shape["wg_size"])] = {k: round(v, 4) for k, v in res.items()}
+            if best is None or res["paced_ms"] < best[1]["paced_ms"]:
+                best = (shape, res)
+        launch = rs.Launch(**best[0])
+        rs.set_pacing(0, best[1]["rate"])
     for _ in range(warmup):
         step()
     rs.synchronize()
@@ -178,7 +198,11 @@ def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, c
     if status:
         raise RuntimeError("device status word raised: %d" % status)
     out = {"ms_per_step": ms / steps, "GBps": 2.0 * n_pes * n * es / (ms / steps) / 1e6,
-           "bytes_per_step": 2 * n_pes * n * es}
+           "bytes_per_step": 2 * n_pes * n * es,
+           "launch": {"wgs_per_pe": launch.wgs_per_pe, "wg_size": launch.wg_size, "tile": launch.tile},
+           "pacing_bytes_per_tick": rs.get_pacing()[1]}
+    if tuning is not None:
+        out["pacing_tuner"] = tuning
     if spread:
         each = sorted(per_launch_ms(rs, step, steps))
         rs.synchronize()
@@ -232,6 +256,7 @@ def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, c
                       "one_thread_per_pe": {"value": round(cpu_rate(min(n_pes, cores), 2), 2),
                                             "cores": min(n_pes, cores)},
                       "single_thread": {"value": round(cpu_rate(1, 1), 2), "cores": 1}}
+    rs.set_pacing(0, 0)
     src.free()
     dst.free()
     psync.free()
@@ -353,7 +378,7 @@ def bench_putmem(rs, steps, n_pes, msg_bytes_list):
                               "calls_per_pe": total // PUT_TILE, "bytes_per_call": PUT_TILE}
     # one 64 MiB message per PE moved by all of the PE's workgroups together (sharded extension)
     msg = 64 << 20
-    launch = rs.Launch(**PUT_LAUNCH)
+    launch = rs.Launch(**PUT_SHARED_LAUNCH)
 
     def shared():
         rs.roc_shmem_rma(rs.PUT, rs.WG_SHARED, dst, src, msg, total // msg, msg, msg, 1, launch)
@@ -362,7 +387,17 @@ def bench_putmem(rs, steps, n_pes, msg_bytes_list):
     rs.synchronize()
     ms = event_time_ms(rs, shared, steps) / steps
     res["67108864_shared"] = {"GBps": 2.0 * n_pes * total / ms / 1e6, "ms": ms, "calls_per_pe": total // msg,
-                              "bytes_per_call": msg, "note": "roc_shmemx_ctx_putmem_wg_shard"}
+                              "bytes_per_call": msg, "note": "roc_shmemx_ctx_putmem_wg_shard", "launch": PUT_SHARED_LAUNCH}
+
+    def shared_get():
+        rs.roc_shmem_rma(rs.GET, rs.WG_SHARED, dst, src, msg, total // msg, msg, msg, 1, launch)
+
+    shared_get()
+    rs.synchronize()
+    ms = event_time_ms(rs, shared_get, steps) / steps
+    res["getmem_67108864_shared"] = {"GBps": 2.0 * n_pes * total / ms / 1e6, "ms": ms, "calls_per_pe": total // msg,
+                                     "bytes_per_call": msg, "note": "roc_shmemx_ctx_getmem_wg_shard",
+                                     "launch": PUT_SHARED_LAUNCH}
     src.free()
     dst.free()
     return res
@@ -735,6 +770,11 @@ def main():
                     help="for rocprofv3: broadcast, alltoall and fcollect over 16 slices x 64 MiB, nothing else")
     ap.add_argument("--alignment", action="store_true",
                     help="large put / broadcast / reduction with shifted source and destination, nothing else")
+    ap.add_argument("--pace-reduce", type=int, default=0, metavar="BYTES_PER_TICK",
+                    help="with --counter-pair: run the headline kernel paced at this rate (32 x 512 per PE), "
+                         "no tuner, for profiler runs of the paced kernel")
+    ap.add_argument("--no-pacing", action="store_true",
+                    help="do not run the library's pacing tuner: every reduction runs free")
     ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="no GPU work: read the two rocprofv3 --pmc counter files of --counter-pair runs and "
                          "write the tracked traffic summary under profiles/")
@@ -785,18 +825,22 @@ def main():
     n_pes, n = 8, 1 << 26
     rs.roc_shmem_init(n_pes, 1 << 30, 64, 1024)
     if args.counter_pair:
-        out = bench_to_all(rs, oracle, 3, 1, rs.FLOAT, n_pes, n, seed=3, check=False)
+        out = bench_to_all(rs, oracle, 3, 1, rs.FLOAT, n_pes, n, seed=3, check=False,
+                           launch_shape=TUNE_SHAPES[1] if args.pace_reduce else None, pace=args.pace_reduce)
         put = bench_putmem(rs, 3, n_pes, [64 << 20])
         rs.roc_shmem_finalize()
         print(json.dumps({"to_all": out, "putmem_copy": put,
                           "copy_bytes_read": n_pes * (256 << 20), "copy_bytes_written": n_pes * (256 << 20)}))
         return
     head = bench_to_all(rs, oracle, args.steps, args.warmup, rs.FLOAT, n_pes, n, seed=3, cpu=True,
-                        spread=True)
+                        spread=True, tune=not args.no_pacing)
     extra = {}
     if not args.quick:
+        extra["to_all_float_sum_8x2^26_free_running"] = bench_to_all(
+            rs, oracle, max(args.steps // 2, 3), 2, rs.FLOAT, n_pes, n, seed=3, check=False)
         extra["to_all_bf16_sum_8x2^26"] = {k: v for k, v in bench_to_all(
-            rs, oracle, max(args.steps // 2, 3), 2, rs.BF16, n_pes, n, seed=3).items() if k != "cpu"}
+            rs, oracle, max(args.steps // 2, 3), 2, rs.BF16, n_pes, n, seed=3,
+            tune=not args.no_pacing).items() if k != "cpu"}
         # every power of two from 8 B to 64 MiB (BASELINE configs[1]; the reference's own sweep,
         # clients/functional_tests/tester.cpp:503-563)
         extra["putmem_wg_8pe"] = bench_putmem(rs, 5, n_pes, [1 << k for k in range(3, 27)])
@@ -855,7 +899,9 @@ def main():
                           "a PE share one reduction); the unchanged roc_shmem_ctx_float_sum_wg_to_all, tiled over "
                           "workgroups, is extra.to_all_float_sum_8x2^26_standard_api_tiled",
                    "pes": n_pes, "elements_per_pe": n, "algorithmic_bytes_per_step": head["bytes_per_step"],
-                   "launch": TO_ALL_LAUNCH, "parity_checked_elements": head.get("parity_checked_elements")},
+                   "launch": head["launch"], "pacing_bytes_per_tick": head["pacing_bytes_per_tick"],
+                   "pacing_tuner": head.get("pacing_tuner"),
+                   "parity_checked_elements": head.get("parity_checked_elements")},
         "roofline": {"bound": "hbm", "achieved": round(head["GBps"], 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(head["GBps"] / HBM_PEAK_GBPS, 4),
                      "traffic": traffic, "traffic_source": traffic_note},

@@ -130,6 +130,28 @@ void *rsm_heap_base(int pe);                    /* first byte of PE `pe`'s slice
 int rsm_state_units(void);                      /* translation units holding a copy of the device state */
 int rsm_take_status(void);                      /* sticky device status word, cleared by the call */
 
+/* Lockstep pacing of large sharded transfers and reductions (no counterpart in the
+ * reference).  Rates are bytes of memory traffic per tick of the GPU's 100 MHz constant
+ * clock; 0 switches pacing off (the default, also settable through ROC_SHMEM_PACE_COPY /
+ * ROC_SHMEM_PACE_REDUCE).  With a rate set, the workgroups of rsm_rma(..., RSM_WG_SHARED)
+ * transfers (roc_shmemx_ctx_{put,get}mem_wg_shard) and of sharded reductions issue their
+ * loads and stores in time slots derived from it instead of running free; results are the
+ * same, only the timing changes.  The right rate is a property of the card: a rate set too
+ * high makes workgroups miss their slots and costs a quarter of the bandwidth, so take it
+ * from rsm_tune_pacing rather than from a table. */
+int rsm_set_pacing(unsigned copy_bytes_per_tick, unsigned reduce_bytes_per_tick);
+int rsm_get_pacing(unsigned *copy_bytes_per_tick, unsigned *reduce_bytes_per_tick);
+/* Measures, on this card and for this very reduction (same arguments as rsm_to_all, tile 0),
+ * the rate at which sharded reductions are best paced: runs the reduction free and at rates
+ * from 5.6 to 7.2 TB/s, nine launches each (about 0.25 s for 4 GiB of traffic), and sets the
+ * reduce rate 2 % below the best one - or to 0 when pacing does not gain at least 1.5 %
+ * over running free.  `dest` receives the reduction's ordinary result.  Outputs (may be
+ * NULL): the rate set, milliseconds per launch free and as set.  Synchronous. */
+int rsm_tune_reduce_pacing(int dtype, int op, void *dest, const void *source, size_t nreduce,
+                           int pe_start, int log_pe_stride, int pe_size, long *pSync,
+                           const rsm_launch_t *launch, unsigned *rate_out, float *free_ms_out,
+                           float *paced_ms_out);
+
 /* ---- teams (reference: roc_shmem.cpp:188-313, team.cpp:47-107) ------------ */
 
 uint64_t rsm_team_world(void);

@@ -30,6 +30,10 @@ SIGNATURES = {
     "rsm_heap_base": (vp, [i32]),
     "rsm_state_units": (i32, []),
     "rsm_take_status": (i32, []),
+    "rsm_set_pacing": (i32, [C.c_uint, C.c_uint]),
+    "rsm_get_pacing": (i32, [C.POINTER(C.c_uint), C.POINTER(C.c_uint)]),
+    "rsm_tune_reduce_pacing": (i32, [i32, i32, vp, vp, sz, i32, i32, i32, vp, LP, C.POINTER(C.c_uint),
+                                     C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "rsm_team_world": (u64, []),
     "rsm_team_split_strided": (i32, [u64, i32, i32, i32, C.POINTER(u64)]),
     "rsm_team_destroy": (i32, [u64]),

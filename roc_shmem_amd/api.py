@@ -24,7 +24,7 @@ __all__ = [
     "sq_consume", "sq_set_mode", "sq_consumer_state", "sq_consumer_start", "sq_consumer_stop",
     "sq_consumer_running", "cq_reader_state", "cq_image", "atomic_ret_image", "arena",
     "read_device", "write_device",
-    "kat_fetch_incr", "kat_coalesce", "take_status", "synchronize", "heap_bytes_in_use",
+    "kat_fetch_incr", "kat_coalesce", "take_status", "set_pacing", "get_pacing", "tune_reduce_pacing", "synchronize", "heap_bytes_in_use",
     "sym_array", "Event", "device_array", "heap_base",
     "SHORT", "INT", "LONG", "LONGLONG", "FLOAT", "DOUBLE", "BF16",
     "SUM", "MAX", "MIN", "PROD", "AND", "OR", "XOR",
@@ -106,6 +106,27 @@ def heap_base(pe):
 
 def heap_bytes_in_use():
     return L.load().rsm_heap_bytes_in_use()
+
+
+def set_pacing(copy_bytes_per_tick=0, reduce_bytes_per_tick=0):
+    """Lockstep pacing rates of large sharded copies / reductions (rsm_set_pacing); 0 = off."""
+    _check(L.load().rsm_set_pacing(int(copy_bytes_per_tick), int(reduce_bytes_per_tick)))
+
+
+def tune_reduce_pacing(dtype, op, dest, source, nreduce, PE_start, logPE_stride, PE_size, pSync, launch=None):
+    """Measure and set the pacing rate of sharded reductions on this card, for this reduction
+    (rsm_tune_reduce_pacing).  Returns {"rate", "free_ms", "paced_ms"}; rate 0 = pacing stays off."""
+    rate, free_ms, paced_ms = C.c_uint(0), C.c_float(0), C.c_float(0)
+    _check(L.load().rsm_tune_reduce_pacing(dtype, op, _addr(dest), _addr(source), nreduce, PE_start,
+                                           logPE_stride, PE_size, _addr(pSync), _launch(launch),
+                                           C.byref(rate), C.byref(free_ms), C.byref(paced_ms)))
+    return {"rate": rate.value, "free_ms": free_ms.value, "paced_ms": paced_ms.value}
+
+
+def get_pacing():
+    a, b = C.c_uint(0), C.c_uint(0)
+    _check(L.load().rsm_get_pacing(C.byref(a), C.byref(b)))
+    return a.value, b.value
 
 
 def take_status():

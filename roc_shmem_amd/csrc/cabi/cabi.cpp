@@ -212,6 +212,23 @@ int rsm_take_status(void) {
   return static_cast<int>(rt->take_status());
 }
 
+int rsm_set_pacing(unsigned copy_bytes_per_tick, unsigned reduce_bytes_per_tick) {
+  RSM_ENTRY;
+  RSM_NEED_RT(rt);
+  if (rsm::live_consumer_running()) return rsm::fail("rsm_set_pacing: a live send-queue consumer is running");
+  if (!rt->set_pacing(copy_bytes_per_tick, reduce_bytes_per_tick))
+    return rsm::fail("rsm_set_pacing: could not update the device state");
+  return 0;
+}
+
+int rsm_get_pacing(unsigned *copy_bytes_per_tick, unsigned *reduce_bytes_per_tick) {
+  RSM_ENTRY;
+  RSM_NEED_RT(rt);
+  if (copy_bytes_per_tick) *copy_bytes_per_tick = rt->device_state().pace_copy_bytes_per_tick;
+  if (reduce_bytes_per_tick) *reduce_bytes_per_tick = rt->device_state().pace_reduce_bytes_per_tick;
+  return 0;
+}
+
 uint64_t rsm_team_world(void) {
   RSM_ENTRY;
   Runtime *rt = Runtime::get();

@@ -321,6 +321,76 @@ int rsm_to_all_noalloc(int dtype, int op, void *dest, const void *source, size_t
   return run(dtype, op, l, a);
 }
 
+int rsm_tune_reduce_pacing(int dtype, int op, void *dest, const void *source, size_t nreduce,
+                           int pe_start, int log_pe_stride, int pe_size, long *pSync,
+                           const rsm_launch_t *launch, unsigned *rate_out, float *free_ms_out,
+                           float *paced_ms_out) {
+  RSM_ENTRY;
+  host::Runtime *rt = host::Runtime::get();
+  if (!rt) return rsm::fail("rsm_init has not been called");
+  if (rsm::live_consumer_running()) return rsm::fail("rsm_tune_reduce_pacing: a live send-queue consumer is running");
+  if (!launch) return rsm::fail("launch description is NULL");
+  hipStream_t stream = static_cast<hipStream_t>(launch->stream);
+  const unsigned copy_rate = rt->device_state().pace_copy_bytes_per_tick;
+  hipEvent_t t0 = nullptr, t1 = nullptr;
+  if (hipEventCreate(&t0) != hipSuccess || hipEventCreate(&t1) != hipSuccess)
+    return rsm::fail("rsm_tune_reduce_pacing: hipEventCreate failed");
+  int rc = 0;
+  // milliseconds per launch at `rate` (0 = free running): eight launches queued back to back
+  // after a warm-up, the way a caller's loop issues them (launches timed one by one on an idle
+  // device tolerate a rate about 2 % higher than a queue of them does)
+  auto measure = [&](unsigned rate, float *ms_out) -> bool {
+    constexpr int kLaunches = 8;
+    if (!rt->set_pacing(copy_rate, rate)) return false;
+    for (int i = 0; i <= kLaunches; ++i) {
+      if (i == 1 && hipEventRecord(t0, stream) != hipSuccess) return false;
+      if (rsm_to_all(dtype, op, dest, source, nreduce, pe_start, log_pe_stride, pe_size, nullptr, pSync,
+                     launch) != 0)
+        return false;
+    }
+    if (hipEventRecord(t1, stream) != hipSuccess || hipEventSynchronize(t1) != hipSuccess) return false;
+    float ms = 0;
+    if (hipEventElapsedTime(&ms, t0, t1) != hipSuccess) return false;
+    *ms_out = ms / kLaunches;
+    return true;
+  };
+  float free_ms = 0, best_ms = 0;
+  unsigned best_rate = 0;
+  if (!measure(0, &free_ms)) rc = -1;
+  // Rates the memory system of an MI355X may sustain in lockstep: 5.6 .. 7.2 TB/s in 1 % steps.
+  for (unsigned rate = 56000; rc == 0 && rate <= 72000; rate += 600) {
+    float ms = 0;
+    if (!measure(rate, &ms)) { rc = -1; break; }
+    if (best_rate == 0 || ms < best_ms) { best_ms = ms; best_rate = rate; }
+  }
+  unsigned chosen = 0;
+  float chosen_ms = free_ms;
+  if (rc == 0 && best_rate != 0) {
+    // Just above the best rate the workgroups start to miss their slots, below it the time
+    // grows in proportion: stay 2 % below, and keep the pacing only if it still gains 1.5 %.
+    const unsigned safe = best_rate - best_rate / 50;
+    float safe_ms = 0, again_free = 0;
+    if (!measure(safe, &safe_ms) || !measure(0, &again_free)) {
+      rc = -1;
+    } else {
+      if (again_free < free_ms) free_ms = again_free;
+      chosen_ms = free_ms;
+      if (safe_ms < free_ms * 0.985f) { chosen = safe; chosen_ms = safe_ms; }
+    }
+  }
+  if (!rt->set_pacing(copy_rate, rc == 0 ? chosen : 0) && rc == 0) rc = -1;
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
+  if (rc != 0) {
+    if (rsm_last_error()[0] == 0) rsm::fail("rsm_tune_reduce_pacing: a launch or an event failed");
+    return -1;
+  }
+  if (rate_out) *rate_out = chosen;
+  if (free_ms_out) *free_ms_out = free_ms;
+  if (paced_ms_out) *paced_ms_out = chosen_ms;
+  return 0;
+}
+
 int rsm_to_all(int dtype, int op, void *dest, const void *source, size_t nreduce, int pe_start,
                int log_pe_stride, int pe_size, void *pWrk, long *pSync,
                const rsm_launch_t *launch) {

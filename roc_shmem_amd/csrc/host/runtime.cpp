@@ -116,6 +116,8 @@ Options Options::from_env() {
   if (const char *s = getenv("ROC_SHMEM_SQ_MODE")) o.sq_queue_mode = strcmp(s, "queue") == 0;
   if (env_u64("ROC_SHMEM_HEAP_HOST_VISIBLE", &v)) o.heap_host_visible = v != 0;
   if (env_u64("ROC_SHMEM_REBASE_ARGS", &v)) o.rebase_args = v != 0;
+  if (env_u64("ROC_SHMEM_PACE_COPY", &v)) o.pace_copy = static_cast<uint32_t>(v);
+  if (env_u64("ROC_SHMEM_PACE_REDUCE", &v)) o.pace_reduce = static_cast<uint32_t>(v);
   return o;
 }
 
@@ -267,6 +269,8 @@ std::string Runtime::init(const Options &opt) {
                                 ? static_cast<uint64_t>(opt_.wait_limit_s * 100e6)
                                 : ~0ull;
   state_.sq_queue_mode = opt_.sq_queue_mode ? 1u : 0u;
+  state_.pace_copy_bytes_per_tick = opt_.pace_copy;
+  state_.pace_reduce_bytes_per_tick = opt_.pace_reduce;
   state_.rebase_args = opt_.rebase_args ? 1u : 0u;
   state_.arena_bytes = stride_ * static_cast<uint64_t>(P);
   state_.stride_mask = (stride_ & (stride_ - 1)) == 0 ? stride_ - 1 : 0;
@@ -418,6 +422,13 @@ const TeamRecord *Runtime::team_record(const detail::Team *team) const {
 
 bool Runtime::set_sq_queue_mode(bool queue) {
   return set_sq_mode(queue ? detail::kSqQueue : detail::kSqLog);
+}
+
+bool Runtime::set_pacing(uint32_t copy_bytes_per_tick, uint32_t reduce_bytes_per_tick) {
+  (void)hipDeviceSynchronize();
+  state_.pace_copy_bytes_per_tick = copy_bytes_per_tick;
+  state_.pace_reduce_bytes_per_tick = reduce_bytes_per_tick;
+  return upload_state_everywhere(state_);
 }
 
 bool Runtime::set_sq_mode(uint32_t mode) {

@@ -64,6 +64,10 @@ struct Options {
   // ROC_SHMEM_REBASE_ARGS (default 1): device calls move symmetric-heap arguments into the
   // calling PE's slice, so a kernel may pass roc_shmem_malloc's pointer straight through.
   bool rebase_args = true;
+  // ROC_SHMEM_PACE_COPY / ROC_SHMEM_PACE_REDUCE: bytes per tick of the 100 MHz clock for the
+  // lockstep pacing of large sharded copies / reductions (device Pacer); 0 = off.
+  uint32_t pace_copy = 0;
+  uint32_t pace_reduce = 0;
   static Options from_env();
 };
 
@@ -120,6 +124,8 @@ class Runtime {
   bool set_sq_queue_mode(bool queue);
   // The same with the mode given as detail::kSqLog / kSqQueue / kSqLive.
   bool set_sq_mode(uint32_t mode);
+  // Rates of the lockstep pacing (0 = off); false when the state could not be re-uploaded.
+  bool set_pacing(uint32_t copy_bytes_per_tick, uint32_t reduce_bytes_per_tick);
   bool sq_queue_mode() const { return state_.sq_queue_mode != 0; }
   const detail::DeviceState &device_state() const { return state_; }
   char *arena() const { return arena_; }

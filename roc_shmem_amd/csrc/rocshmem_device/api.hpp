@@ -285,7 +285,7 @@ __device__ inline void roc_shmemx_ctx_putmem_wg_shard(roc_shmem_ctx_t ctx, void 
   if (nelems == 0) return;
   const detail::DeviceCtx *c = detail::ctx_of(ctx);
   detail::wg_copy_shard(detail::translate(detail::own(dest, c), c->my_pe, pe), detail::own(source, c), nelems,
-                        shard, nshards);
+                        shard, nshards, detail::g_state.pace_copy_bytes_per_tick);
 }
 __device__ inline void roc_shmemx_ctx_getmem_wg_shard(roc_shmem_ctx_t ctx, void *dest,
                                                       const void *source, size_t nelems, int pe,
@@ -293,7 +293,7 @@ __device__ inline void roc_shmemx_ctx_getmem_wg_shard(roc_shmem_ctx_t ctx, void 
   if (nelems == 0) return;
   const detail::DeviceCtx *c = detail::ctx_of(ctx);
   detail::wg_copy_shard(detail::own(dest, c), detail::translate(detail::own(source, c), c->my_pe, pe), nelems,
-                        shard, nshards);
+                        shard, nshards, detail::g_state.pace_copy_bytes_per_tick);
 }
 __device__ inline void roc_shmemx_ctx_putmem_nbi_wave(roc_shmem_ctx_t ctx, void *dest,
                                                       const void *source, size_t nelems,

@@ -171,7 +171,7 @@ template <typename T, ROC_SHMEM_OP Op, int U = kReduceUnroll, int C = kReducePeC
 __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_begin,
                                                size_t v_end, const ActiveSet &as, int my_pe,
                                                uint32_t tid, uint32_t nthr, size_t first_pass = 0,
-                                               size_t pass_step = 1) {
+                                               size_t pass_step = 1, Pacer pacer = Pacer{0u, 0u}) {
   using Acc = typename AccOf<T, Op>::type;
   using V = VecOf<T>;
   constexpr int E = V::kElems;
@@ -203,6 +203,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
     const size_t left = byte_end - b;
     const int valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
     Acc acc[U][E];
+    pacer.wait_slot(0);
     {
       __amdgpu_buffer_rsrc_t rs = uniform_rsrc(src0 + b, valid);
 #pragma unroll
@@ -247,6 +248,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
     for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int e = 0; e < E; ++e) out[u].e[e] = from_acc<T, Acc>(acc[u][e]);
+    pacer.wait_slot(1);
     for (int m = 0; m < as.size; ++m) {
       __amdgpu_buffer_rsrc_t rd = uniform_rsrc(dst0 + m * member_step + b, valid);
 #pragma unroll
@@ -378,7 +380,14 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
       if (nvec < parts * static_cast<size_t>(kReduceUnroll) * nthr) {
         reduce_vectors<T, Op, 2, 4>(dest, source, 0, nvec, as, my_pe, tid, nthr, part, parts);
       } else {
-        reduce_vectors<T, Op>(dest, source, 0, nvec, as, my_pe, tid, nthr, part, parts);
+        // Paced (see Pacer) when the library has a measured rate and every workgroup has
+        // enough passes for the slots' start-up to disappear.
+        const uint64_t pass_bytes = static_cast<uint64_t>(kReduceUnroll) * nthr * 16u;
+        Pacer pacer{0u, 0u};
+        if (g_state.pace_reduce_bytes_per_tick != 0 && nvec * 16u >= 6 * parts * pass_bytes)
+          pacer = make_pacer(g_state.pace_reduce_bytes_per_tick,
+                             parts * pass_bytes * static_cast<uint64_t>(pe_size));
+        reduce_vectors<T, Op>(dest, source, 0, nvec, as, my_pe, tid, nthr, part, parts, pacer);
       }
     }
     if (part == parts - 1) {

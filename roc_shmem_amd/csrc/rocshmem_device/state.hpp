@@ -117,6 +117,11 @@ struct DeviceState {
   uint32_t rebase_args;
   uint64_t arena_bytes;        // num_pes * slice_stride
   uint64_t stride_mask;        // slice_stride - 1 when the stride is a power of two, else 0
+  // Lockstep pacing of large streaming copies / reductions (see Pacer in copy.hpp): bytes of
+  // traffic the memory system takes per tick of the 100 MHz clock when all workgroups issue in
+  // step; 0 = workgroups run free.
+  uint32_t pace_copy_bytes_per_tick;
+  uint32_t pace_reduce_bytes_per_tick;
 };
 
 // Fingerprint of the structures device code and the host library share.  Device
@@ -127,8 +132,8 @@ struct DeviceState {
 // Bump kStateRevision when a layout changes without changing a size, or when
 // units must agree on how they use shared memory (3: the barrier pool holds
 // call counts, not flags that are reset; 4: live queues, cq_consumer;
-// 5: arguments rebased into the caller's slice).
-constexpr uint32_t kStateRevision = 5;
+// 5: arguments rebased into the caller's slice; 6: pacing).
+constexpr uint32_t kStateRevision = 6;
 constexpr uint32_t kStateLayout =
     (kStateRevision * 0x01000193u) ^
     static_cast<uint32_t>(sizeof(DeviceState) | (sizeof(DeviceCtx) << 8) | (sizeof(Team) << 16) |
