@@ -44,6 +44,15 @@ PUT_SHARED_LAUNCH = dict(wgs_per_pe=32, wg_size=1024)
 PUT_TILE = 256 << 10
 
 
+def random_payload(rs, arr, n_pes, seed):
+    """Uniform random bytes in every PE's copy of `arr` (one random block, rotated per PE)."""
+    block = np.random.default_rng(seed).integers(0, 256, min(arr.nbytes, 64 << 20), dtype=np.uint8)
+    reps = -(-arr.nbytes // block.size)
+    for p in range(n_pes):
+        data = np.tile(np.roll(block, 4099 * p), reps)[:arr.nbytes]
+        arr.write(p, data.view(arr.dtype))
+
+
 def event_time_ms(rs, fn, iters):
     start, stop = rs.Event(), rs.Event()
     start.record()
@@ -341,8 +350,9 @@ def cpu_other_legs(oracle):
 def bench_putmem(rs, steps, n_pes, msg_bytes_list):
     """wg putmem from every PE p to PE p+1: GB/s counted as 2*m bytes per message (read+write)."""
     total = 256 << 20
-    src = rs.sym_array(total, np.uint8, fill=7)
+    src = rs.sym_array(total, np.uint8)
     dst = rs.sym_array(total, np.uint8, fill=0)
+    random_payload(rs, src, n_pes, seed=2)
     res = {}
     for m in msg_bytes_list:
         if m >= PUT_TILE:
@@ -403,12 +413,52 @@ def bench_putmem(rs, steps, n_pes, msg_bytes_list):
     return res
 
 
+def bench_pacing_sweep(rs, n_pes):
+    """Rate of the headline reduction and of a sharded 64 MiB put, running free and paced at fixed
+    rates (no tuner), for two launch shapes: GB/s by rate in bytes per tick of the 100 MHz clock."""
+    out = {"float_sum_to_all_8x2^26": {}, "putmem_wg_shard_64MiB": {}}
+    n = 1 << 26
+    src = rs.sym_array(n, np.float32)
+    dst = rs.sym_array(n, np.float32, fill=0)
+    psync = rs.sym_array(64 * rs.ROC_SHMEM_REDUCE_SYNC_SIZE, np.int64, fill=0)
+    rng = np.random.default_rng(3)
+    for p in range(n_pes):                     # N(0,1) like the headline's inputs, not zeros
+        src.write(p, rng.standard_normal(n, dtype=np.float32))
+    rates = [0] + list(range(58000, 70001, 1000))
+    for shape in TUNE_SHAPES:
+        launch = rs.Launch(**shape)
+        key = "%dx%d" % (shape["wgs_per_pe"], shape["wg_size"])
+
+        def reduce():
+            rs.roc_shmem_to_all(rs.FLOAT, rs.SUM, dst, src, n, 0, 0, n_pes, None, psync, launch)
+
+        def put():
+            rs.roc_shmem_rma(rs.PUT, rs.WG_SHARED, dst, src, 64 << 20, 4, 64 << 20, 64 << 20, 1, launch)
+
+        for name, fn, nbytes, which in (("float_sum_to_all_8x2^26", reduce, 2.0 * n_pes * n * 4, 1),
+                                        ("putmem_wg_shard_64MiB", put, 2.0 * n_pes * (256 << 20), 0)):
+            row = {}
+            for r in rates:
+                rs.set_pacing(r if which == 0 else 0, r if which == 1 else 0)
+                fn()
+                rs.synchronize()
+                row["free" if r == 0 else str(r)] = round(nbytes / (event_time_ms(rs, fn, 10) / 10) / 1e6, 1)
+            out[name][key] = row
+    rs.set_pacing(0, 0)
+    if rs.take_status():
+        raise RuntimeError("device status word raised")
+    for a in (psync, dst, src):
+        a.free()
+    return out
+
+
 def bench_granularities(rs, steps, n_pes):
     """putmem / getmem issued per wave and per thread (every wave or lane moves its own message to
     or from the next PE): GB/s counted as 2*m bytes per message, and messages per second."""
     total = 256 << 20
-    src = rs.sym_array(total, np.uint8, fill=7)
+    src = rs.sym_array(total, np.uint8)
     dst = rs.sym_array(total, np.uint8, fill=0)
+    random_payload(rs, src, n_pes, seed=2)
     res = {}
     shapes = [(rs.WAVE, "wave", m) for m in (256, 4096, 65536, 1 << 20)] + \
              [(rs.THREAD, "thread", m) for m in (8, 256, 4096)]
@@ -674,8 +724,9 @@ def bench_small_collectives(rs, n_pes, n, calls):
 def bench_bcast_a2a(rs, n_pes, slice_bytes):
     world = rs.roc_shmem_team_world()
     res = {}
-    src = rs.sym_array(slice_bytes, np.uint8, fill=3)
+    src = rs.sym_array(slice_bytes, np.uint8)
     dst = rs.sym_array(slice_bytes, np.uint8, fill=0)
+    random_payload(rs, src, n_pes, seed=5)
     # best of a sweep over 8/16/32 workgroups per PE x 512/1024 threads for each
     launch = rs.Launch(16, 1024)
     bcast_launch = fcollect_launch = rs.Launch(8, 1024)
@@ -773,6 +824,11 @@ def main():
     ap.add_argument("--pace-reduce", type=int, default=0, metavar="BYTES_PER_TICK",
                     help="with --counter-pair: run the headline kernel paced at this rate (32 x 512 per PE), "
                          "no tuner, for profiler runs of the paced kernel")
+    ap.add_argument("--pacing-sweep", action="store_true",
+                    help="the headline reduction and a sharded 64 MiB put, free and paced at fixed rates, nothing else")
+    ap.add_argument("--reduce-lds", action="store_true",
+                    help="headline workload only, through the LDS-staged form of the reduction "
+                         "(ROC_SHMEM_REDUCE_LDS=1), running free, for 32 x 512 and 32 x 1024 lanes per PE")
     ap.add_argument("--no-pacing", action="store_true",
                     help="do not run the library's pacing tuner: every reduction runs free")
     ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
@@ -790,6 +846,26 @@ def main():
     import oracle
     import roc_shmem_amd as rs
 
+    if args.reduce_lds:
+        out = {}
+        for staged in (1, 0):
+            os.environ["ROC_SHMEM_REDUCE_LDS"] = str(staged)
+            rs.roc_shmem_init(8, 1 << 30, 64, 1024)
+            for shape in TUNE_SHAPES:
+                r = bench_to_all(rs, oracle, 10, 3, rs.FLOAT, 8, 1 << 26, seed=3, launch_shape=shape)
+                out["%s_%dx%d" % ("lds_staged" if staged else "registers", shape["wgs_per_pe"], shape["wg_size"])] = \
+                    {"GBps": round(r["GBps"], 1), "ms": round(r["ms_per_step"], 4),
+                     "parity_checked_elements": r["parity_checked_elements"]}
+            rs.roc_shmem_finalize()
+        del os.environ["ROC_SHMEM_REDUCE_LDS"]
+        print(json.dumps({"to_all_float_sum_8x2^26_free_running": out}))
+        return
+    if args.pacing_sweep:
+        rs.roc_shmem_init(8, 1 << 30, 64, 1024)
+        out = bench_pacing_sweep(rs, 8)
+        rs.roc_shmem_finalize()
+        print(json.dumps({"GBps_by_pacing_rate_8pe": out}))
+        return
     if args.small_ops:
         rs.roc_shmem_init(16, 256 << 20, 64, 1024)
         out = bench_small_ops(rs, 16, 10_000_000, 1024, 256, 64 << 20, seed=4)

@@ -84,7 +84,9 @@ __global__ void __launch_bounds__(256) clear_flags_kernel(long *flags, size_t n)
 // same with the flags in the library's own array (`pSync0` is its device address).  Separate
 // kernels rather than branches: with more than one form inlined into one kernel the compiler
 // ran out of scalar registers.
-enum ToAllForm { kTiled = 0, kSharded = 1, kShardedStaticFlags = 2 };
+// kShardedLds: the sharded form with the loads staged through dynamic LDS (a measured
+// alternative, built for the three benchmark reductions only; see reduce_vectors_lds).
+enum ToAllForm { kTiled = 0, kSharded = 1, kShardedStaticFlags = 2, kShardedLds = 3 };
 
 template <typename T, ROC_SHMEM_OP Op, int kForm>
 __global__ void __launch_bounds__(1024)
@@ -103,7 +105,13 @@ __global__ void __launch_bounds__(1024)
   if (member) {
     T *dest = roc_shmemx_my_addr(dest0);
     const T *source = roc_shmemx_my_addr(source0);
-    if constexpr (kForm == kShardedStaticFlags) {
+    if constexpr (kForm == kShardedLds) {
+      extern __shared__ __attribute__((aligned(16))) char lds_stage[];
+      long *pSync = roc_shmemx_my_addr(pSync0) + w * ROC_SHMEM_REDUCE_SYNC_SIZE;
+      detail::wg_all_reduce<T, Op>(me, dest, source, n, pe_start, 1 << log_stride, pe_size, pSync,
+                                   static_cast<int>(w), static_cast<int>(nw), 0, lds_stage,
+                                   static_cast<uint32_t>(tile));
+    } else if constexpr (kForm == kShardedStaticFlags) {
       long *flags = pSync0 + (static_cast<size_t>(me) * nw + w) * ROC_SHMEM_REDUCE_SYNC_SIZE;
       const int64_t pe_step = static_cast<int64_t>(nw) * ROC_SHMEM_REDUCE_SYNC_SIZE * sizeof(long);
       detail::wg_all_reduce<T, Op>(me, dest, source, n, pe_start, 1 << log_stride, pe_size, flags,
@@ -168,6 +176,7 @@ struct ReduceArgs {
   roc_shmem_team_t team;
   int stride;
   bool static_flags;   // pSync is the device address of the library's own flag array
+  bool lds;            // loads staged through LDS (ROC_SHMEM_REDUCE_LDS=1)
 };
 
 template <typename T, ROC_SHMEM_OP Op, int kForm>
@@ -184,8 +193,32 @@ void launch_team(const rsm::Launch &l, const ReduceArgs &a) {
                      a.n, a.tile, a.pe_start, a.stride, a.pe_size);
 }
 
+// Dynamic LDS of the LDS-staged form: room for all members at two vectors per lane, at most
+// 128 KiB (the form then stages the members in several rounds).
+constexpr size_t kLdsStageLimit = 128u << 10;
+
+template <typename T, ROC_SHMEM_OP Op>
+bool launch_lds(const rsm::Launch &l, const ReduceArgs &a) {
+  const size_t per_member = static_cast<size_t>(l.wg_size) * 16u * 2u;
+  size_t bytes = per_member * static_cast<size_t>(a.pe_size);
+  if (bytes > kLdsStageLimit) bytes = kLdsStageLimit / per_member * per_member;
+  const void *kernel = reinterpret_cast<const void *>(&to_all_kernel<T, Op, kShardedLds>);
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)) !=
+      hipSuccess)
+    return false;
+  // `tile` carries the size of the stage to the kernel (the form has no tiles)
+  hipLaunchKernelGGL((to_all_kernel<T, Op, kShardedLds>), dim3(l.grid), dim3(l.wg_size), bytes, l.stream,
+                     static_cast<T *>(a.dest), static_cast<const T *>(a.source), a.n, bytes, a.pe_start,
+                     a.log_stride, a.pe_size, static_cast<T *>(a.pWrk), a.pSync);
+  return true;
+}
+
 template <typename T, ROC_SHMEM_OP Op>
 void launch_one(const rsm::Launch &l, const ReduceArgs &a) {
+  if constexpr ((std::is_same<T, float>::value || std::is_same<T, long>::value ||
+                 std::is_same<T, __hip_bfloat16>::value) && Op == ROC_SHMEM_SUM) {
+    if (a.lds && !a.team && !a.static_flags && a.tile == 0 && launch_lds<T, Op>(l, a)) return;
+  }
   if (a.static_flags) {
     launch_active_set<T, Op, kShardedStaticFlags>(l, a);
   } else if (a.team) {
@@ -317,7 +350,7 @@ int rsm_to_all_noalloc(int dtype, int op, void *dest, const void *source, size_t
   hipLaunchKernelGGL(clear_flags_kernel, dim3(static_cast<unsigned>((n_flags + 255) / 256)), dim3(256),
                      0, l.stream, flags, n_flags);
   ReduceArgs a{dest, source, nreduce, 0, pe_start, log_pe_stride, pe_size, nullptr, flags,
-               nullptr, 1 << log_pe_stride, true};
+               nullptr, 1 << log_pe_stride, true, false};
   return run(dtype, op, l, a);
 }
 
@@ -404,7 +437,7 @@ int rsm_to_all(int dtype, int op, void *dest, const void *source, size_t nreduce
   if (!rsm::active_set_in_range(pe_start, log_pe_stride, pe_size, rt->num_pes()))
     return rsm::fail("to_all: active set out of range");
   ReduceArgs a{dest, source, nreduce, l.tile, pe_start, log_pe_stride, pe_size, pWrk, pSync,
-               nullptr, 1 << log_pe_stride, false};
+               nullptr, 1 << log_pe_stride, false, rt->options().reduce_lds};
   return run(dtype, op, l, a);
 }
 
@@ -421,7 +454,7 @@ int rsm_to_all_team(int dtype, int op, uint64_t team, void *dest, const void *so
     return rsm::fail("to_all_team: wgs_per_pe exceeds the contexts per PE (team pSync slices)");
   const detail::TeamInfo &ti = rec->image.wrt_world;
   ReduceArgs a{dest, source, nreduce, l.tile, ti.pe_start, 0, ti.size, nullptr,
-               nullptr, reinterpret_cast<roc_shmem_team_t>(team), ti.stride, false};
+               nullptr, reinterpret_cast<roc_shmem_team_t>(team), ti.stride, false, false};
   return run(dtype, op, l, a);
 }
 

@@ -116,6 +116,7 @@ Options Options::from_env() {
   if (const char *s = getenv("ROC_SHMEM_SQ_MODE")) o.sq_queue_mode = strcmp(s, "queue") == 0;
   if (env_u64("ROC_SHMEM_HEAP_HOST_VISIBLE", &v)) o.heap_host_visible = v != 0;
   if (env_u64("ROC_SHMEM_REBASE_ARGS", &v)) o.rebase_args = v != 0;
+  if (env_u64("ROC_SHMEM_REDUCE_LDS", &v)) o.reduce_lds = v != 0;
   if (env_u64("ROC_SHMEM_PACE_COPY", &v)) o.pace_copy = static_cast<uint32_t>(v);
   if (env_u64("ROC_SHMEM_PACE_REDUCE", &v)) o.pace_reduce = static_cast<uint32_t>(v);
   return o;

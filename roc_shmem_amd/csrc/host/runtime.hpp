@@ -68,6 +68,9 @@ struct Options {
   // lockstep pacing of large sharded copies / reductions (device Pacer); 0 = off.
   uint32_t pace_copy = 0;
   uint32_t pace_reduce = 0;
+  // ROC_SHMEM_REDUCE_LDS=1: rsm_to_all runs float / long / bfloat16 sums through the LDS-staged
+  // form of the sharded reduction (a measured alternative, slower on MI355X; default 0).
+  bool reduce_lds = false;
   static Options from_env();
 };
 

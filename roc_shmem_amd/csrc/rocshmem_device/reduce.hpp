@@ -258,6 +258,83 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
   }
 }
 
+// The same reduction with the loads staged through LDS: every lane's 16-byte
+// loads go straight from memory into the workgroup's LDS (global_load_lds,
+// no vector registers in between), `chunk` members' worth at a time, and the
+// fold reads them back from LDS.  Each lane reads only what it loaded itself,
+// so the waves need no barrier among themselves.  `stage` holds `stage_bytes`
+// of dynamic LDS; only whole passes are handled here (the caller gives the
+// remainder to reduce_vectors).  Kept as a measured alternative: with eight
+// members it frees some sixty vector registers per lane and lets all members'
+// loads of a pass be in flight together, and on MI355X it is slower all the
+// same (the stream is bound by the memory system, not by registers or by
+// loads in flight), so the register path above is the one every call takes
+// unless the caller asks for this one.
+template <typename T, ROC_SHMEM_OP Op, int U>
+__device__ __forceinline__ void reduce_vectors_lds(T *dst, const T *src, size_t n_passes,
+                                                   const ActiveSet &as, int my_pe, uint32_t tid,
+                                                   uint32_t nthr, size_t first_pass, size_t pass_step,
+                                                   char *stage, uint32_t stage_bytes) {
+  using Acc = typename AccOf<T, Op>::type;
+  using V = VecOf<T>;
+  constexpr int E = V::kElems;
+  constexpr int kNt = 2;
+  const int64_t stride = static_cast<int64_t>(g_state.slice_stride);
+  char *src0 = const_cast<char *>(reinterpret_cast<const char *>(src)) +
+               (static_cast<int64_t>(as.pe_start) - my_pe) * stride;
+  char *dst0 =
+      reinterpret_cast<char *>(dst) + (static_cast<int64_t>(as.pe_start) - my_pe) * stride;
+  const int64_t member_step = stride * as.pe_stride;
+  const uint32_t lane_off = tid * 16u;
+  const uint32_t wave_off = (tid & ~63u) * 16u;     // where this wave's 64 slots start
+  const uint32_t access_bytes = nthr * 16u;
+  const uint32_t pass_bytes = access_bytes * U;
+  int chunk = static_cast<int>(stage_bytes / pass_bytes);   // members staged together
+  if (chunk > as.size) chunk = as.size;
+  if (chunk < 1) return;
+  typedef __attribute__((address_space(3))) void *LdsPtr;
+  typedef const __attribute__((address_space(1))) void *GlobalPtr;
+  for (size_t pass = first_pass; pass < n_passes; pass += pass_step) {
+    const size_t b = pass * pass_bytes;
+    Acc acc[U][E];
+    for (int k0 = 0; k0 < as.size; k0 += chunk) {
+      const int members = as.size - k0 < chunk ? as.size - k0 : chunk;
+      for (int c = 0; c < members; ++c) {
+        const char *from = src0 + (k0 + c) * member_step + b + lane_off;
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          __builtin_amdgcn_global_load_lds(
+              (GlobalPtr)(from + u * access_bytes),   // address-space casts: C style only
+              (LdsPtr)(stage + (c * U + u) * access_bytes + wave_off), 16, 0, kNt);
+      }
+      __builtin_amdgcn_s_waitcnt(0);
+      for (int c = 0; c < members; ++c) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          typename V::Pack p;
+          p.raw = *reinterpret_cast<const u32x4 *>(stage + (c * U + u) * access_bytes + lane_off);
+#pragma unroll
+          for (int e = 0; e < E; ++e) {
+            const Acc x = to_acc<T, Acc>(p.e[e]);
+            acc[u][e] = (k0 + c == 0) ? x : fold<Op, Acc>(acc[u][e], x);
+          }
+        }
+      }
+    }
+    typename V::Pack out[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int e = 0; e < E; ++e) out[u].e[e] = from_acc<T, Acc>(acc[u][e]);
+    for (int m = 0; m < as.size; ++m) {
+      __amdgpu_buffer_rsrc_t rd = uniform_rsrc(dst0 + m * member_step + b, static_cast<int>(pass_bytes));
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        __builtin_amdgcn_raw_buffer_store_b128(out[u].raw, rd, lane_off, u * access_bytes, kNt);
+    }
+  }
+}
+
 // Scalar path for element range [e_begin, e_end): unaligned arrays and tails.
 template <typename T, ROC_SHMEM_OP Op>
 __device__ __forceinline__ void reduce_elements(T *dst, const T *src, size_t e_begin,
@@ -294,7 +371,8 @@ template <typename T, ROC_SHMEM_OP Op>
 __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *source, size_t nreduce,
                                               int pe_start, int pe_stride, int pe_size,
                                               long *psync, int shard = 0, int nshards = 1,
-                                              int64_t psync_pe_step = 0) {
+                                              int64_t psync_pe_step = 0, char *lds_stage = nullptr,
+                                              uint32_t lds_stage_bytes = 0) {
   // Workgroup-collective: every lane holds the same arguments.
   my_pe = uniform(my_pe);
   dest = own(uniform(dest), my_pe);       // symmetric arguments: the caller's own copies
@@ -387,7 +465,18 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
         if (g_state.pace_reduce_bytes_per_tick != 0 && nvec * 16u >= 6 * parts * pass_bytes)
           pacer = make_pacer(g_state.pace_reduce_bytes_per_tick,
                              parts * pass_bytes * static_cast<uint64_t>(pe_size));
-        reduce_vectors<T, Op>(dest, source, 0, nvec, as, my_pe, tid, nthr, part, parts, pacer);
+        if (lds_stage != nullptr) {
+          // whole passes through LDS, two vectors per lane per member; what is left of the
+          // range goes the usual way, to whoever's turn it would have been
+          const size_t lds_pass_vecs = 2u * nthr;
+          const size_t whole = nvec / lds_pass_vecs;
+          reduce_vectors_lds<T, Op, 2>(dest, source, whole, as, my_pe, tid, nthr, part, parts, lds_stage,
+                                       uniform(lds_stage_bytes));
+          if (whole * lds_pass_vecs < nvec && whole % parts == part)
+            reduce_vectors<T, Op, 2, 1>(dest, source, whole * lds_pass_vecs, nvec, as, my_pe, tid, nthr);
+        } else {
+          reduce_vectors<T, Op>(dest, source, 0, nvec, as, my_pe, tid, nthr, part, parts, pacer);
+        }
       }
     }
     if (part == parts - 1) {

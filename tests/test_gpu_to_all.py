@@ -300,3 +300,25 @@ def test_closed_forms_of_the_reference_tests():
         rs.synchronize()
         for p in range(npes):
             assert (fdst.read(p) == float(npes)).all()
+
+
+@pytest.mark.parametrize("dtype", [rs.FLOAT, rs.LONG, rs.BF16])
+def test_lds_staged_form_gives_the_same_bits(dtype):
+    # ROC_SHMEM_REDUCE_LDS=1 sends float / long / bfloat16 sums of rsm_to_all (tile 0) through the
+    # LDS-staged form of the sharded reduction: whole passes through LDS, the remainder the usual way.
+    import os
+    os.environ["ROC_SHMEM_REDUCE_LDS"] = "1"
+    try:
+        rs.roc_shmem_init(8, 64 << 20, 16, 1024)
+    finally:
+        del os.environ["ROC_SHMEM_REDUCE_LDS"]
+    try:
+        for n, wgs, wg_size, pe_size in (((1 << 20) + 4103, 4, 512, 8), (300001, 2, 1024, 8), (70000, 3, 256, 5),
+                                         (4099, 1, 64, 8)):
+            got, expect, _ = run_case(dtype, rs.SUM, 8, n, seed=31 + dtype, wgs=wgs, wg_size=wg_size,
+                                      pe_size=pe_size)
+            for p in range(8):
+                assert np.array_equal(got[p].view(np.uint8), expect[p].view(np.uint8)), (n, wgs, wg_size, p)
+        assert rs.take_status() == 0
+    finally:
+        rs.roc_shmem_finalize()
