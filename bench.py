@@ -484,7 +484,7 @@ def bench_granularities(rs, steps, n_pes):
     return res
 
 
-def bench_small_ops(rs, n_pes, n_ops, wgs_total, wg_size, slice_bytes, seed):
+def bench_small_ops(rs, n_pes, n_ops, wgs_total, wg_size, slice_bytes, seed, live_queue=True):
     """10 M 8-byte puts (unique targets, lower half) and int64 fetch-adds (upper half)."""
     rng = np.random.default_rng(seed)
     words = slice_bytes // 8
@@ -567,34 +567,35 @@ def bench_small_ops(rs, n_pes, n_ops, wgs_total, wg_size, slice_bytes, seed):
     ops["offset"] = np.where(is_put, (uniq % (words // 2)) * 8,
                              (words // 2 + rng.integers(0, words // 2, n_ops)) * 8) + mem.offset
     ops["value"] = rng.integers(-1000, 1000, n_ops)
-    dev = rs.device_array(ops)
-    stream = rs.Stream()
-    live_launch = rs.Launch(wgs_total // n_pes, wg_size, 0, stream)
-    rs.synchronize()
-    rs.sq_reset()
-    rs.sq_consumer_start()
-    try:
-        rs.roc_shmem_small_ops(dev, n_ops, None, live_launch)
-        stream.synchronize()
-        start, stop, reps = rs.Event(), rs.Event(), 3
-        start.record(stream)
-        for _ in range(reps):
+    if live_queue:
+        dev = rs.device_array(ops)
+        stream = rs.Stream()
+        live_launch = rs.Launch(wgs_total // n_pes, wg_size, 0, stream)
+        rs.synchronize()
+        rs.sq_reset()
+        rs.sq_consumer_start()
+        try:
             rs.roc_shmem_small_ops(dev, n_ops, None, live_launch)
-        stop.record(stream)
-        ms = start.elapsed_ms(stop) / reps
-        stream.synchronize()
-    finally:
-        totals = rs.sq_consumer_stop()
-    if totals["lost"] or totals["rejected"] or totals["retired"] != (reps + 1) * n_ops:
-        raise RuntimeError("live consumer: %r" % (totals,))
-    res["mixed_through_live_queues"] = {"Mops_per_s": n_ops / ms / 1e3, "ms": ms, "retired": totals["retired"],
-                                        "lost": 0, "rejected": 0,
-                                        "note": "1024-entry rings in queue mode, consumer kernel running beside the "
-                                                "producers, entries written through to memory"}
-    start.destroy()
-    stop.destroy()
-    stream.destroy()
-    dev.free()
+            stream.synchronize()
+            start, stop, reps = rs.Event(), rs.Event(), 3
+            start.record(stream)
+            for _ in range(reps):
+                rs.roc_shmem_small_ops(dev, n_ops, None, live_launch)
+            stop.record(stream)
+            ms = start.elapsed_ms(stop) / reps
+            stream.synchronize()
+        finally:
+            totals = rs.sq_consumer_stop()
+        if totals["lost"] or totals["rejected"] or totals["retired"] != (reps + 1) * n_ops:
+            raise RuntimeError("live consumer: %r" % (totals,))
+        res["mixed_through_live_queues"] = {"Mops_per_s": n_ops / ms / 1e3, "ms": ms, "retired": totals["retired"],
+                                            "lost": 0, "rejected": 0,
+                                            "note": "1024-entry rings in queue mode, consumer kernel running beside the "
+                                                    "producers, entries written through to memory"}
+        start.destroy()
+        stop.destroy()
+        stream.destroy()
+        dev.free()
     # The same stream once more with the rings as logs, for the consumer pass below.
     dev = rs.device_array(ops)
     rs.sq_reset()
@@ -813,6 +814,10 @@ def main():
                          "plain wg putmem copy of known size (2 GiB read + 2 GiB written), nothing else")
     ap.add_argument("--small-ops", action="store_true",
                     help="for rocprofv3 --pmc: the 10 M-operation streams and the consumer pass, nothing else")
+    ap.add_argument("--skip-live-queue", action="store_true",
+                    help="with --small-ops under rocprofv3 --pmc: leave out the stream through queues with a live "
+                         "consumer (counter collection runs one kernel at a time, and a consumer kernel cannot run "
+                         "beside the producers then)")
     ap.add_argument("--granularities", action="store_true",
                     help="putmem / getmem per wave and per thread, nothing else")
     ap.add_argument("--amo-kinds", action="store_true",
@@ -822,8 +827,8 @@ def main():
     ap.add_argument("--alignment", action="store_true",
                     help="large put / broadcast / reduction with shifted source and destination, nothing else")
     ap.add_argument("--pace-reduce", type=int, default=0, metavar="BYTES_PER_TICK",
-                    help="with --counter-pair: run the headline kernel paced at this rate (32 x 512 per PE), "
-                         "no tuner, for profiler runs of the paced kernel")
+                    help="run the headline kernel paced at this rate (32 x 512 lanes per PE) instead of asking "
+                         "the tuner, so that every launch of a profiler run is alike (also with --counter-pair)")
     ap.add_argument("--pacing-sweep", action="store_true",
                     help="the headline reduction and a sharded 64 MiB put, free and paced at fixed rates, nothing else")
     ap.add_argument("--reduce-lds", action="store_true",
@@ -868,7 +873,8 @@ def main():
         return
     if args.small_ops:
         rs.roc_shmem_init(16, 256 << 20, 64, 1024)
-        out = bench_small_ops(rs, 16, 10_000_000, 1024, 256, 64 << 20, seed=4)
+        out = bench_small_ops(rs, 16, 10_000_000, 1024, 256, 64 << 20, seed=4,
+                              live_queue=not args.skip_live_queue)
         rs.roc_shmem_finalize()
         print(json.dumps({"small_ops_16x64MiB_1024wg_x256": out}))
         return
@@ -908,8 +914,12 @@ def main():
         print(json.dumps({"to_all": out, "putmem_copy": put,
                           "copy_bytes_read": n_pes * (256 << 20), "copy_bytes_written": n_pes * (256 << 20)}))
         return
-    head = bench_to_all(rs, oracle, args.steps, args.warmup, rs.FLOAT, n_pes, n, seed=3, cpu=True,
-                        spread=True, tune=not args.no_pacing)
+    if args.pace_reduce:      # a fixed rate instead of the tuner (profiler runs: every launch alike)
+        head = bench_to_all(rs, oracle, args.steps, args.warmup, rs.FLOAT, n_pes, n, seed=3, cpu=True,
+                            spread=True, launch_shape=TUNE_SHAPES[1], pace=args.pace_reduce)
+    else:
+        head = bench_to_all(rs, oracle, args.steps, args.warmup, rs.FLOAT, n_pes, n, seed=3, cpu=True,
+                            spread=True, tune=not args.no_pacing)
     extra = {}
     if not args.quick:
         extra["to_all_float_sum_8x2^26_free_running"] = bench_to_all(
