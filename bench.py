@@ -35,7 +35,7 @@ KERNEL_SOURCES = ["roc_shmem_amd/csrc/rocshmem_device/reduce.hpp", "roc_shmem_am
 
 # Launch shapes chosen by measurement on MI355X (256 CUs).
 TO_ALL_LAUNCH = dict(wgs_per_pe=32, wg_size=1024)
-# Shapes the pacing tuner is tried with: running free, 32 x 1024 per PE is best; paced, 32 x 512.
+# Shapes the pacing tuner is tried with (256 workgroups either way: 128 KiB or 64 KiB per member per pass).
 TUNE_SHAPES = (dict(wgs_per_pe=32, wg_size=1024), dict(wgs_per_pe=32, wg_size=512))
 PUT_LAUNCH = dict(wgs_per_pe=32, wg_size=512)
 # one large message shared by the PE's workgroups (sharded extension): 1024-lane workgroups
@@ -160,11 +160,13 @@ def device_report():
 
 
 def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, cpu=False,
-                 spread=False, launch_shape=None, tune=False, pace=0):
+                 spread=False, launch_shape=None, tune=False, pace=None):
     """Returns a dict with ms_per_step, GB/s (algorithmic 2*P*N*s bytes) and optional CPU figures.
-    tune: let the library measure, outside the timed region, whether pacing its workgroups in
-    lockstep pays for this reduction on this card, with the launch shapes of TUNE_SHAPES; the
-    timed steps then run with the better shape and the rate the tuner set (0 = free running)."""
+    pace: None = the pacing rate the library holds (its default: reductions paced at 6.6 TB/s),
+    0 = workgroups run free, another value = that rate in bytes per tick.
+    tune: let the library measure, outside the timed region, which rate suits this reduction on
+    this card, with the launch shapes of TUNE_SHAPES; the timed steps then run with the better
+    shape and the rate the tuner set (0 = free running).  The library's rate is put back at the end."""
     npd = rs.NP_DTYPE[dtype]
     es = np.dtype(npd).itemsize
     src = rs.sym_array(n, npd)
@@ -187,17 +189,18 @@ def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, c
         rs.roc_shmem_to_all(dtype, rs.SUM, dst, src, n, 0, 0, n_pes, None, psync, launch)
 
     tuning = None
-    rs.set_pacing(0, pace)
+    pacing_before = rs.get_pacing()
+    if pace is not None:
+        rs.set_pacing(pacing_before[0], pace)
     if tune:
         tuning, best = {}, None
         for shape in TUNE_SHAPES:
-            rs.set_pacing(0, 0)
             res = rs.tune_reduce_pacing(dtype, rs.SUM, dst, src, n, 0, 0, n_pes, psync, rs.Launch(**shape))
             tuning["%dx%d" % (shape["wgs_per_pe"], shape["wg_size"])] = {k: round(v, 4) for k, v in res.items()}
             if best is None or res["paced_ms"] < best[1]["paced_ms"]:
                 best = (shape, res)
         launch = rs.Launch(**best[0])
-        rs.set_pacing(0, best[1]["rate"])
+        rs.set_pacing(pacing_before[0], best[1]["rate"])
     for _ in range(warmup):
         step()
     rs.synchronize()
@@ -218,6 +221,7 @@ def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, c
         out["ms_median"] = each[len(each) // 2]
         out["ms_min"] = each[0]
         out["ms_max"] = each[-1]
+    rs.set_pacing(*pacing_before)
 
     heap = None
     if check or cpu:
@@ -265,7 +269,6 @@ def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, c
                       "one_thread_per_pe": {"value": round(cpu_rate(min(n_pes, cores), 2), 2),
                                             "cores": min(n_pes, cores)},
                       "single_thread": {"value": round(cpu_rate(1, 1), 2), "cores": 1}}
-    rs.set_pacing(0, 0)
     src.free()
     dst.free()
     psync.free()
@@ -424,7 +427,8 @@ def bench_pacing_sweep(rs, n_pes):
     rng = np.random.default_rng(3)
     for p in range(n_pes):                     # N(0,1) like the headline's inputs, not zeros
         src.write(p, rng.standard_normal(n, dtype=np.float32))
-    rates = [0] + list(range(58000, 70001, 1000))
+    rates = [0] + list(range(58000, 70001, 1000)) + [75000, 80000, 90000]
+    pacing_before = rs.get_pacing()
     for shape in TUNE_SHAPES:
         launch = rs.Launch(**shape)
         key = "%dx%d" % (shape["wgs_per_pe"], shape["wg_size"])
@@ -444,7 +448,7 @@ def bench_pacing_sweep(rs, n_pes):
                 rs.synchronize()
                 row["free" if r == 0 else str(r)] = round(nbytes / (event_time_ms(rs, fn, 10) / 10) / 1e6, 1)
             out[name][key] = row
-    rs.set_pacing(0, 0)
+    rs.set_pacing(*pacing_before)
     if rs.take_status():
         raise RuntimeError("device status word raised")
     for a in (psync, dst, src):
@@ -827,15 +831,16 @@ def main():
     ap.add_argument("--alignment", action="store_true",
                     help="large put / broadcast / reduction with shifted source and destination, nothing else")
     ap.add_argument("--pace-reduce", type=int, default=0, metavar="BYTES_PER_TICK",
-                    help="run the headline kernel paced at this rate (32 x 512 lanes per PE) instead of asking "
-                         "the tuner, so that every launch of a profiler run is alike (also with --counter-pair)")
+                    help="run the headline kernel paced at this rate (32 x 1024 lanes per PE) instead of asking "
+                         "the tuner, so that every launch of a profiler run is alike (also with --counter-pair, "
+                         "which otherwise runs it at the library's default rate)")
     ap.add_argument("--pacing-sweep", action="store_true",
                     help="the headline reduction and a sharded 64 MiB put, free and paced at fixed rates, nothing else")
     ap.add_argument("--reduce-lds", action="store_true",
                     help="headline workload only, through the LDS-staged form of the reduction "
                          "(ROC_SHMEM_REDUCE_LDS=1), running free, for 32 x 512 and 32 x 1024 lanes per PE")
     ap.add_argument("--no-pacing", action="store_true",
-                    help="do not run the library's pacing tuner: every reduction runs free")
+                    help="pacing off: every reduction runs free (no schedule, no tuner)")
     ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="no GPU work: read the two rocprofv3 --pmc counter files of --counter-pair runs and "
                          "write the tracked traffic summary under profiles/")
@@ -857,7 +862,7 @@ def main():
             os.environ["ROC_SHMEM_REDUCE_LDS"] = str(staged)
             rs.roc_shmem_init(8, 1 << 30, 64, 1024)
             for shape in TUNE_SHAPES:
-                r = bench_to_all(rs, oracle, 10, 3, rs.FLOAT, 8, 1 << 26, seed=3, launch_shape=shape)
+                r = bench_to_all(rs, oracle, 10, 3, rs.FLOAT, 8, 1 << 26, seed=3, launch_shape=shape, pace=0)
                 out["%s_%dx%d" % ("lds_staged" if staged else "registers", shape["wgs_per_pe"], shape["wg_size"])] = \
                     {"GBps": round(r["GBps"], 1), "ms": round(r["ms_per_step"], 4),
                      "parity_checked_elements": r["parity_checked_elements"]}
@@ -908,7 +913,7 @@ def main():
     rs.roc_shmem_init(n_pes, 1 << 30, 64, 1024)
     if args.counter_pair:
         out = bench_to_all(rs, oracle, 3, 1, rs.FLOAT, n_pes, n, seed=3, check=False,
-                           launch_shape=TUNE_SHAPES[1] if args.pace_reduce else None, pace=args.pace_reduce)
+                           pace=0 if args.no_pacing else (args.pace_reduce or None))
         put = bench_putmem(rs, 3, n_pes, [64 << 20])
         rs.roc_shmem_finalize()
         print(json.dumps({"to_all": out, "putmem_copy": put,
@@ -916,17 +921,22 @@ def main():
         return
     if args.pace_reduce:      # a fixed rate instead of the tuner (profiler runs: every launch alike)
         head = bench_to_all(rs, oracle, args.steps, args.warmup, rs.FLOAT, n_pes, n, seed=3, cpu=True,
-                            spread=True, launch_shape=TUNE_SHAPES[1], pace=args.pace_reduce)
+                            spread=True, pace=args.pace_reduce)
+    elif args.no_pacing:
+        head = bench_to_all(rs, oracle, args.steps, args.warmup, rs.FLOAT, n_pes, n, seed=3, cpu=True,
+                            spread=True, pace=0)
     else:
         head = bench_to_all(rs, oracle, args.steps, args.warmup, rs.FLOAT, n_pes, n, seed=3, cpu=True,
-                            spread=True, tune=not args.no_pacing)
+                            spread=True, tune=True)
     extra = {}
     if not args.quick:
         extra["to_all_float_sum_8x2^26_free_running"] = bench_to_all(
+            rs, oracle, max(args.steps // 2, 3), 2, rs.FLOAT, n_pes, n, seed=3, check=False, pace=0)
+        extra["to_all_float_sum_8x2^26_library_defaults"] = bench_to_all(
             rs, oracle, max(args.steps // 2, 3), 2, rs.FLOAT, n_pes, n, seed=3, check=False)
         extra["to_all_bf16_sum_8x2^26"] = {k: v for k, v in bench_to_all(
             rs, oracle, max(args.steps // 2, 3), 2, rs.BF16, n_pes, n, seed=3,
-            tune=not args.no_pacing).items() if k != "cpu"}
+            tune=not args.no_pacing, pace=0 if args.no_pacing else None).items() if k != "cpu"}
         # every power of two from 8 B to 64 MiB (BASELINE configs[1]; the reference's own sweep,
         # clients/functional_tests/tester.cpp:503-563)
         extra["putmem_wg_8pe"] = bench_putmem(rs, 5, n_pes, [1 << k for k in range(3, 27)])

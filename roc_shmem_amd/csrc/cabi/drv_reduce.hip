@@ -399,16 +399,17 @@ int rsm_tune_reduce_pacing(int dtype, int op, void *dest, const void *source, si
   unsigned chosen = 0;
   float chosen_ms = free_ms;
   if (rc == 0 && best_rate != 0) {
-    // Just above the best rate the workgroups start to miss their slots, below it the time
-    // grows in proportion: stay 2 % below, and keep the pacing only if it still gains 1.5 %.
-    const unsigned safe = best_rate - best_rate / 50;
-    float safe_ms = 0, again_free = 0;
-    if (!measure(safe, &safe_ms) || !measure(0, &again_free)) {
+    // The best rate and running free once more, so that one lucky sample decides nothing; the
+    // schedule stays only if it still gains 1 %.  (No margin below the best rate is needed: a
+    // rate beyond what the card sustains costs a little, not the cliff a gate on slots has.)
+    float best_again = 0, again_free = 0;
+    if (!measure(best_rate, &best_again) || !measure(0, &again_free)) {
       rc = -1;
     } else {
       if (again_free < free_ms) free_ms = again_free;
+      if (best_again > best_ms) best_ms = best_again;
       chosen_ms = free_ms;
-      if (safe_ms < free_ms * 0.985f) { chosen = safe; chosen_ms = safe_ms; }
+      if (best_ms < free_ms * 0.99f) { chosen = best_rate; chosen_ms = best_ms; }
     }
   }
   if (!rt->set_pacing(copy_rate, rc == 0 ? chosen : 0) && rc == 0) rc = -1;

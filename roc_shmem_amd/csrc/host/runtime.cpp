@@ -272,6 +272,13 @@ std::string Runtime::init(const Options &opt) {
   state_.sq_queue_mode = opt_.sq_queue_mode ? 1u : 0u;
   state_.pace_copy_bytes_per_tick = opt_.pace_copy;
   state_.pace_reduce_bytes_per_tick = opt_.pace_reduce;
+  {
+    int dev = 0, cus = 0;
+    RT_HIP(hipGetDevice(&dev));
+    RT_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    state_.pace_max_grid_lanes = static_cast<uint32_t>(cus) * 1024u;
+    state_.pace_min_grid_workgroups = static_cast<uint32_t>(cus);
+  }
   state_.rebase_args = opt_.rebase_args ? 1u : 0u;
   state_.arena_bytes = stride_ * static_cast<uint64_t>(P);
   state_.stride_mask = (stride_ & (stride_ - 1)) == 0 ? stride_ - 1 : 0;

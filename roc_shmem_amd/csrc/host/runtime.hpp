@@ -65,9 +65,12 @@ struct Options {
   // calling PE's slice, so a kernel may pass roc_shmem_malloc's pointer straight through.
   bool rebase_args = true;
   // ROC_SHMEM_PACE_COPY / ROC_SHMEM_PACE_REDUCE: bytes per tick of the 100 MHz clock for the
-  // lockstep pacing of large sharded copies / reductions (device Pacer); 0 = off.
+  // lockstep pacing of large sharded copies / reductions (device Pacer); 0 = off.  Reductions
+  // are paced by default, at 6.6 TB/s: a little above what MI355X cards sustain, which is where
+  // the schedule gains most (it loses a quarter of its gain at 9 TB/s and none of the free rate).
+  // Copies run free by default: their short passes gain nothing from the schedule.
   uint32_t pace_copy = 0;
-  uint32_t pace_reduce = 0;
+  uint32_t pace_reduce = 66000;
   // ROC_SHMEM_REDUCE_LDS=1: rsm_to_all runs float / long / bfloat16 sums through the LDS-staged
   // form of the sharded reduction (a measured alternative, slower on MI355X; default 0).
   bool reduce_lds = false;

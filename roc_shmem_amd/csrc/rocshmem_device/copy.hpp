@@ -12,6 +12,7 @@
 #define ROCSHMEM_MI355X_DEVICE_COPY_HPP
 
 #include "state.hpp"
+#include "sync.hpp"
 #include "wave.hpp"
 
 namespace rocshmem {
@@ -198,26 +199,40 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t uniform_rsrc(const void *base,
 // which every workgroup can read: the workgroups on even XCDs issue the loads
 // of a pass in even slots and its stores in odd slots, those on odd XCDs the
 // other way round.  All of them then start each burst at the same instant,
-// half the chip reading while the other half writes, the bursts sweep one
-// compact window of every array, and when the period equals the time the
-// memory system needs for one slot's traffic the same copy runs at 6.4-6.5
-// TB/s.  A period that is too short is worse than none (workgroups miss their
-// slots and wait for the next), one that is too long costs in proportion, so
-// the rate the period is derived from is measured on the card (the library's
-// tuner), not assumed.  period == 0: no pacing.  The wait ends by itself: the
-// clock advances.
+// half the chip reading while the other half writes (of each pair of
+// neighbouring XCDs one reads while the other writes; pairing them any other
+// way measured worse), and the bursts sweep one compact window of every array.
+//
+// The slots are a schedule, not a gate: a wave keeps the start time of its
+// next burst, waits for it when it is early and goes at once when it is late.
+// With a rate the memory system can sustain everybody is on time and the
+// stream runs at that rate; with a rate beyond it everybody runs late, nobody
+// waits, and the stream keeps most of the gain of its aligned start (8 -> 8
+// fp32 reduction, bare kernel, one card: 6.00 TB/s free, 6.21 paced at 6.2,
+// 6.33 at 6.7, 6.22 at 7.0, 6.10 at 9.0 TB/s).  Gating on the slot's parity
+// instead (wait whenever the clock is in the other kind of slot) reaches the
+// same peak, but a wave that misses its slot then waits a whole slot for the
+// next, and 2 % beyond the best rate the stream falls to 4.9-5.4 TB/s.
+//
+// The schedule assumes that every workgroup of the grid is resident: those of
+// a grid larger than the chip would wait for slots sized for all of them while
+// only some run (half the rate for twice the chip).  make_pacer's callers
+// check that.  period == 0: no pacing.  Every wait ends by itself: the clock
+// advances.
 struct Pacer {
-  uint32_t period;   // ticks per slot
-  uint32_t parity;   // 0: loads in even slots; 1: loads in odd slots
-  __device__ __forceinline__ void wait_slot(uint32_t stores) const {
+  uint32_t period;   // ticks per slot; 0 = not paced
+  uint64_t next;     // clock value at which the next burst of this wave is due
+  __device__ __forceinline__ void wait_slot() {
     if (period == 0) return;
-    while (((static_cast<uint32_t>(wall_clock64()) / period) & 1u) != (stores ^ parity))
-      __builtin_amdgcn_s_sleep(2);
+    while (static_cast<int64_t>(wall_clock64() - next) < 0) __builtin_amdgcn_s_sleep(2);
+    next += period;
   }
 };
 
 // `slot_bytes`: what all workgroups of the grid move in one slot (loads of one
-// half plus stores of the other).  Too few or too many ticks per slot: no pacing.
+// half plus stores of the other).  Too few or too many ticks per slot: no
+// pacing.  The first burst (loads) is due at the start of the first slot of
+// this XCD's load parity that has not ended yet.
 __device__ __forceinline__ Pacer make_pacer(uint32_t bytes_per_tick, uint64_t slot_bytes) {
   Pacer p{0u, 0u};
   if (bytes_per_tick == 0) return p;
@@ -225,12 +240,23 @@ __device__ __forceinline__ Pacer make_pacer(uint32_t bytes_per_tick, uint64_t sl
   if (period < 64 || period > 50000) return p;
   p.period = static_cast<uint32_t>(period);
   // XCC_ID: the XCD this workgroup runs on
-  p.parity = __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 1u;
+  const uint32_t parity = __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 1u;
+  uint64_t slot = wall_clock64() / period;
+  slot += (static_cast<uint32_t>(slot) ^ parity) & 1u;
+  p.next = slot * period;
   return p;
 }
 
 __device__ __forceinline__ uint64_t grid_workgroups() {
   return static_cast<uint64_t>(gridDim.x) * gridDim.y * gridDim.z;
+}
+
+// This grid fills the chip and all of its workgroups run at the same time (what a
+// paced stream needs).
+__device__ __forceinline__ bool grid_is_resident() {
+  const uint64_t wgs = grid_workgroups();
+  return wgs >= g_state.pace_min_grid_workgroups &&
+         wgs * flat_block_size() <= g_state.pace_max_grid_lanes;
 }
 
 // Body of a group copy whose arguments are the same in every lane
@@ -257,14 +283,14 @@ __device__ __forceinline__ void stream_copy_uniform(char *d, const char *s, size
     __amdgpu_buffer_rsrc_t rs = uniform_rsrc(s + b, valid);
     __amdgpu_buffer_rsrc_t rd = uniform_rsrc(d + b, valid);
     u32x4 v[U];
-    pacer.wait_slot(0);
+    pacer.wait_slot();
 #pragma unroll
     for (int u = 0; u < U; ++u)
       v[u] = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * access_bytes, kAux);
     if (pacer.period) {
       // the data first, then the slot: stores leave together at the slot's start
       __builtin_amdgcn_s_waitcnt(0);
-      pacer.wait_slot(1);
+      pacer.wait_slot();
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -364,7 +390,7 @@ __device__ __forceinline__ void group_copy_dealt(void *dst, const void *src, siz
       // Paced when the library has a measured rate and every workgroup has enough
       // passes for the slots' start-up to disappear.
       Pacer pacer{0u, 0u};
-      if (pace_bytes_per_tick != 0 && body >= 16 * parts * pass_bytes)
+      if (pace_bytes_per_tick != 0 && body >= 16 * parts * pass_bytes && grid_is_resident())
         pacer = make_pacer(pace_bytes_per_tick, grid_workgroups() * pass_bytes);
       stream_copy_uniform<2 /* nt */, kStreamUnroll>(d + head, s + head, body, tid, nthr, part, parts,
                                                      pacer);

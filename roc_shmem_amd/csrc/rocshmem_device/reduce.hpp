@@ -203,7 +203,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
     const size_t left = byte_end - b;
     const int valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
     Acc acc[U][E];
-    pacer.wait_slot(0);
+    pacer.wait_slot();
     {
       __amdgpu_buffer_rsrc_t rs = uniform_rsrc(src0 + b, valid);
 #pragma unroll
@@ -248,7 +248,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
     for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int e = 0; e < E; ++e) out[u].e[e] = from_acc<T, Acc>(acc[u][e]);
-    pacer.wait_slot(1);
+    pacer.wait_slot();
     for (int m = 0; m < as.size; ++m) {
       __amdgpu_buffer_rsrc_t rd = uniform_rsrc(dst0 + m * member_step + b, valid);
 #pragma unroll
@@ -458,11 +458,13 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
       if (nvec < parts * static_cast<size_t>(kReduceUnroll) * nthr) {
         reduce_vectors<T, Op, 2, 4>(dest, source, 0, nvec, as, my_pe, tid, nthr, part, parts);
       } else {
-        // Paced (see Pacer) when the library has a measured rate and every workgroup has
-        // enough passes for the slots' start-up to disappear.
+        // Paced (see Pacer) when the library holds a rate, the grid fills the chip and
+        // every workgroup has at least four passes (with two, a 32 x 1024 launch measured
+        // 4 % slower paced than free; with four, 1-2 % faster; with eight, 5-7 %).
         const uint64_t pass_bytes = static_cast<uint64_t>(kReduceUnroll) * nthr * 16u;
         Pacer pacer{0u, 0u};
-        if (g_state.pace_reduce_bytes_per_tick != 0 && nvec * 16u >= 6 * parts * pass_bytes)
+        if (g_state.pace_reduce_bytes_per_tick != 0 && nvec * 16u >= 4 * parts * pass_bytes &&
+            grid_is_resident())
           pacer = make_pacer(g_state.pace_reduce_bytes_per_tick,
                              parts * pass_bytes * static_cast<uint64_t>(pe_size));
         if (lds_stage != nullptr) {

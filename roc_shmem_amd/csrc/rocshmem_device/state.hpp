@@ -122,6 +122,13 @@ struct DeviceState {
   // step; 0 = workgroups run free.
   uint32_t pace_copy_bytes_per_tick;
   uint32_t pace_reduce_bytes_per_tick;
+  // Grids that are paced: at most pace_max_grid_lanes lanes (compute units x 1024, what is
+  // resident together of the streaming kernels, which need 65-128 vector registers: the slots
+  // are sized for all workgroups of the grid running at once) and at least
+  // pace_min_grid_workgroups workgroups (one per compute unit: on half a chip the schedule
+  // measured 1-3 % slower than none).
+  uint32_t pace_max_grid_lanes;
+  uint32_t pace_min_grid_workgroups;
 };
 
 // Fingerprint of the structures device code and the host library share.  Device
@@ -132,8 +139,9 @@ struct DeviceState {
 // Bump kStateRevision when a layout changes without changing a size, or when
 // units must agree on how they use shared memory (3: the barrier pool holds
 // call counts, not flags that are reset; 4: live queues, cq_consumer;
-// 5: arguments rebased into the caller's slice; 6: pacing).
-constexpr uint32_t kStateRevision = 6;
+// 5: arguments rebased into the caller's slice; 6: pacing; 7: paced bursts follow a
+// schedule of start times).
+constexpr uint32_t kStateRevision = 7;
 constexpr uint32_t kStateLayout =
     (kStateRevision * 0x01000193u) ^
     static_cast<uint32_t>(sizeof(DeviceState) | (sizeof(DeviceCtx) << 8) | (sizeof(Team) << 16) |
