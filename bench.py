@@ -416,6 +416,40 @@ def bench_putmem(rs, steps, n_pes, msg_bytes_list):
     return res
 
 
+def bench_streams(rs, n_pes, steps=10):
+    """What this card's memory system gives plain streams (rsm_stream_probe: reads alone, writes
+    alone, every PE's workgroups over their own slice with the library's access pattern) and the
+    harmonic mean of the two, 2 / (1/read + 1/write): what a stream that reads and writes as much
+    would reach if mixing the two directions cost nothing."""
+    per_pe = 512 << 20          # 4 GiB per launch among 8 PEs, the headline's traffic
+    buf = rs.sym_array(per_pe, np.uint8)
+    chk = rs.sym_array(4, np.uint32, fill=0)
+    out = {}
+    for name, kind in (("read_only", rs.STREAM_READ), ("write_only", rs.STREAM_WRITE)):
+        best = None
+        for wgs in (32, 64):
+            launch = rs.Launch(wgs, 1024)
+
+            def fn():
+                rs.stream_probe(kind, buf, per_pe, chk, 7, launch)
+
+            fn()
+            rs.synchronize()
+            ms = event_time_ms(rs, fn, steps) / steps
+            rate = n_pes * per_pe / ms / 1e6
+            if best is None or rate > best["GBps"]:
+                best = {"GBps": round(rate, 1), "ms": round(ms, 4), "launch": {"wgs_per_pe": wgs, "wg_size": 1024}}
+        out[name] = best
+    r, w = out["read_only"]["GBps"], out["write_only"]["GBps"]
+    out["harmonic_mean_GBps"] = round(2.0 / (1.0 / r + 1.0 / w), 1)
+    out["bytes_per_launch"] = n_pes * per_pe
+    if rs.take_status():
+        raise RuntimeError("device status word raised")
+    chk.free()
+    buf.free()
+    return out
+
+
 def bench_pacing_sweep(rs, n_pes):
     """Rate of the headline reduction and of a sharded 64 MiB put, running free and paced at fixed
     rates (no tuner), for two launch shapes: GB/s by rate in bytes per tick of the 100 MHz clock."""
@@ -816,6 +850,8 @@ def main():
     ap.add_argument("--counter-pair", action="store_true",
                     help="for rocprofv3 --pmc: a few launches of the headline kernel and of a "
                          "plain wg putmem copy of known size (2 GiB read + 2 GiB written), nothing else")
+    ap.add_argument("--stream-probes", action="store_true",
+                    help="read-only and write-only streams over the heap (rsm_stream_probe), nothing else")
     ap.add_argument("--small-ops", action="store_true",
                     help="for rocprofv3 --pmc: the 10 M-operation streams and the consumer pass, nothing else")
     ap.add_argument("--skip-live-queue", action="store_true",
@@ -907,6 +943,12 @@ def main():
         rs.roc_shmem_finalize()
         print(json.dumps({"GBps_by_source_shift/destination_shift_8pe": out}))
         return
+    if args.stream_probes:
+        rs.roc_shmem_init(8, 1 << 30, 64, 1024)
+        out = bench_streams(rs, 8)
+        rs.roc_shmem_finalize()
+        print(json.dumps({"hbm_streams_on_this_card": out}))
+        return
     device = device_report() if not args.counter_pair else {}
     # ---- headline: fp32 sum_to_all, 8 slices x 2^26 elements (4 GiB algorithmic traffic) ----
     n_pes, n = 8, 1 << 26
@@ -929,6 +971,9 @@ def main():
         head = bench_to_all(rs, oracle, args.steps, args.warmup, rs.FLOAT, n_pes, n, seed=3, cpu=True,
                             spread=True, tune=True)
     extra = {}
+    streams = bench_streams(rs, n_pes)
+    streams["headline_over_harmonic_mean"] = round(head["GBps"] / streams["harmonic_mean_GBps"], 4)
+    extra["hbm_streams_on_this_card"] = streams
     if not args.quick:
         extra["to_all_float_sum_8x2^26_free_running"] = bench_to_all(
             rs, oracle, max(args.steps // 2, 3), 2, rs.FLOAT, n_pes, n, seed=3, check=False, pace=0)

@@ -154,6 +154,21 @@ int rsm_tune_reduce_pacing(int dtype, int op, void *dest, const void *source, si
                            const rsm_launch_t *launch, unsigned *rate_out, float *free_ms_out,
                            float *paced_ms_out);
 
+/* Plain streams over a symmetric buffer, to measure what the memory system of the card at
+ * hand delivers (no counterpart in the reference): the workgroups of every PE read
+ * (RSM_STREAM_READ) or write (RSM_STREAM_WRITE) `bytes_per_pe` bytes at `buf` in their own
+ * PE's slice, with the access pattern of the library's large transfers (128 KiB passes dealt
+ * round-robin to the PE's workgroups, 16 bytes per lane per access, non-temporal).  Reads
+ * alone and writes alone bound what a stream that does both can reach (the harmonic mean of
+ * the two rates for a 1:1 mix); cards differ by several per cent.  The caller times the
+ * launches.  READ folds all 16-byte vectors of a PE's buffer with XOR into the four 32-bit
+ * words at `checksum` (symmetric, 16 bytes, zeroed by the caller) of that PE's slice; WRITE
+ * stores {i mod 2^32, i >> 32, pe, seed} into vector i.  `buf` and `bytes_per_pe` must be
+ * multiples of 16. */
+enum rsm_stream_kind { RSM_STREAM_READ = 0, RSM_STREAM_WRITE = 1 };
+int rsm_stream_probe(int kind, void *buf, size_t bytes_per_pe, void *checksum, unsigned seed,
+                     const rsm_launch_t *launch);
+
 /* ---- teams (reference: roc_shmem.cpp:188-313, team.cpp:47-107) ------------ */
 
 uint64_t rsm_team_world(void);

@@ -60,6 +60,7 @@ SIGNATURES = {
     "rsm_to_all_noalloc": (i32, [i32, i32, vp, vp, sz, i32, i32, i32, LP]),
     "rsm_to_all_team": (i32, [i32, i32, u64, vp, vp, sz, LP]),
     "rsm_rma": (i32, [i32, i32, vp, vp, sz, sz, sz, sz, i32, LP]),
+    "rsm_stream_probe": (i32, [i32, vp, sz, vp, C.c_uint, LP]),
     "rsm_broadcast": (i32, [sz, vp, vp, sz, i32, i32, i32, i32, vp, LP]),
     "rsm_broadcast_team": (i32, [sz, u64, vp, vp, sz, i32, LP]),
     "rsm_alltoall": (i32, [sz, u64, vp, vp, sz, LP]),

@@ -24,7 +24,7 @@ __all__ = [
     "sq_consume", "sq_set_mode", "sq_consumer_state", "sq_consumer_start", "sq_consumer_stop",
     "sq_consumer_running", "cq_reader_state", "cq_image", "atomic_ret_image", "arena",
     "read_device", "write_device",
-    "kat_fetch_incr", "kat_coalesce", "take_status", "set_pacing", "get_pacing", "tune_reduce_pacing", "synchronize", "heap_bytes_in_use",
+    "kat_fetch_incr", "kat_coalesce", "take_status", "set_pacing", "get_pacing", "tune_reduce_pacing", "stream_probe", "STREAM_READ", "STREAM_WRITE", "synchronize", "heap_bytes_in_use",
     "sym_array", "Event", "device_array", "heap_base",
     "SHORT", "INT", "LONG", "LONGLONG", "FLOAT", "DOUBLE", "BF16",
     "SUM", "MAX", "MIN", "PROD", "AND", "OR", "XOR",
@@ -38,6 +38,7 @@ __all__ = [
 SHORT, INT, LONG, LONGLONG, FLOAT, DOUBLE, BF16 = range(7)
 SUM, MAX, MIN, PROD, AND, OR, XOR = range(7)
 PUT, GET, PUT_NBI, GET_NBI = range(4)
+STREAM_READ, STREAM_WRITE = range(2)
 THREAD, WAVE, WG, WG_SHARED = range(4)
 (OP_P64, OP_FADD64, OP_ADD64, OP_FINC64, OP_INC64, OP_CSWAP64, OP_FETCH64, OP_SET64, OP_SWAP64,
  OP_P32, OP_FADD32, OP_PUTMEM, OP_GETMEM, OP_FAND64, OP_FOR64, OP_FXOR64) = range(16)
@@ -348,6 +349,12 @@ def roc_shmem_rma(kind, granularity, dest, source, msg_bytes, n_msgs=1, dst_stri
     src_stride = msg_bytes if src_stride is None else src_stride
     _check(L.load().rsm_rma(kind, granularity, _addr(dest), _addr(source), msg_bytes, n_msgs,
                             dst_stride, src_stride, pe_shift, _launch(launch)))
+
+
+def stream_probe(kind, buf, bytes_per_pe, checksum=None, seed=0, launch=None):
+    """Plain read-only / write-only stream over `buf` in every PE's slice (rsm_stream_probe)."""
+    _check(L.load().rsm_stream_probe(kind, _addr(buf), bytes_per_pe, _addr(checksum) if checksum is not None else None,
+                                     seed, _launch(launch)))
 
 
 def roc_shmem_broadcast(elem_size, dest, source, nelem, PE_root, PE_start, logPE_stride, PE_size,
