@@ -291,6 +291,10 @@ int rsm_sq_state(int pe, int block, uint32_t *sq_counter, uint32_t *published,
 int rsm_sq_constants(int pe, int block, uint32_t *ctrl_qp_sq, uint64_t *ctrl_sig, uint32_t *lkey,
                      uint32_t *atomic_lkey, uint64_t *atomic_ret_base, uint32_t *max_nwqe);
 int rsm_sq_rkey(int dest_pe, uint32_t *rkey);
+/* What a fence's entry on a live queue is addressed to: PE `pe`'s flush word and the key it
+ * is named under (reference: hdp_address[] / hdp_rkey[], network_policy.cpp:114-180;
+ * QueuePair::fence, queue_pair.cpp:376-384). */
+int rsm_sq_flush_target(int pe, uint64_t *addr, uint32_t *rkey);
 
 /* ---- consumer pass, completion queues, queue mode -----------------------------------
  * What a NIC does with the rings in the reference: take published entries off
@@ -330,8 +334,12 @@ int rsm_sq_set_mode(int queue_mode);
  * rings publish (completion entries, `consumed`), and returns when all its waves are
  * resident.  Until rsm_sq_consumer_stop, producers (rsm_small_ops and any kernel that
  * posts) block in their post when their ring is full and go on when the consumer has freed
- * slots; roc_shmem_ctx_quiet collects the completions its queue has asked for (bounded
- * waits, status word on timeout).  Entries and completions are written through to
+ * slots; roc_shmem_ctx_quiet posts a zero-byte read (READ, DS = 2; QueuePair::zero_b_rd,
+ * queue_pair.cpp:318-325, as the reference's quiet does, thread_policy.cpp:35-108) and collects
+ * the completions its queue has asked for, that entry's included (bounded waits, status word
+ * on timeout); roc_shmem_ctx_fence posts the flush write of QueuePair::fence
+ * (queue_pair.cpp:376-384).  Without a live consumer neither posts anything: both are memory
+ * fences, and nothing would complete the entries.  Entries and completions are written through to
  * memory meanwhile.  rsm_sq_consumer_stop: call it when the producers' streams have been
  * synchronised (it synchronises the default stream itself); it lets the consumer drain the
  * rings, waits for it, restores the previous mode and returns what was retired.  Between

@@ -252,7 +252,7 @@ class WqeReq(C.Structure):
     _fields_ = [("opcode", C.c_uint8), ("size", C.c_uint32), ("raddr", C.c_uint64),
                 ("rkey", C.c_uint32), ("laddr", C.c_uint64), ("atomic_data", C.c_uint64),
                 ("atomic_cmp", C.c_uint64), ("inline_bytes", C.c_uint8 * 8),
-                ("atomic_pos", C.c_uint32), ("request_cqe", C.c_int)]
+                ("atomic_pos", C.c_uint32), ("request_cqe", C.c_int), ("form", C.c_int)]
 
 
 OP_WRITE, OP_READ, OP_ATOMIC_CS, OP_ATOMIC_FA = 0x08, 0x10, 0x11, 0x12
@@ -266,8 +266,11 @@ def requests_cqe(sq_counter, max_nwqe, closes_post):
     return bool(closes_post) or sq_counter % max_nwqe == max_nwqe - 2
 
 
+WQE_DATA, WQE_ZERO_BYTE_READ, WQE_FLUSH_WRITE = range(3)
+
+
 def wqe_build(slot, qp, sq_counter, opcode, size=0, raddr=0, rkey=0, laddr=0, atomic_data=0,
-              atomic_cmp=0, inline=b"", atomic_pos=0, request_cqe=False):
+              atomic_cmp=0, inline=b"", atomic_pos=0, request_cqe=False, form=WQE_DATA):
     """Write one entry into ``slot`` (a 64-byte uint8 array view), in place."""
     assert slot.dtype == np.uint8 and slot.size == 64 and slot.flags["C_CONTIGUOUS"]
     rq = WqeReq()
@@ -282,13 +285,15 @@ def wqe_build(slot, qp, sq_counter, opcode, size=0, raddr=0, rkey=0, laddr=0, at
         rq.inline_bytes[i] = b
     rq.atomic_pos = atomic_pos
     rq.request_cqe = 1 if request_cqe else 0
+    rq.form = form
     _lib.orc_wqe_build(slot.ctypes.data, C.byref(qp), sq_counter & 0xFFFFFFFF, C.byref(rq))
     return slot
 
 
 class Arena(C.Structure):
     _fields_ = [("heap_base0", C.c_uint64), ("slice_stride", C.c_uint64), ("heap_size", C.c_uint64),
-                ("num_pes", C.c_int), ("rkeys", C.c_void_p)]
+                ("num_pes", C.c_int), ("rkeys", C.c_void_p), ("flush_base", C.c_uint64),
+                ("flush_rkeys", C.c_void_p)]
 
 
 class ConsumeTotals(C.Structure):
@@ -300,14 +305,16 @@ class ConsumeTotals(C.Structure):
 
 
 def sq_consume(qp, ring, consumed, published, heap_base0, slice_stride, heap_size, rkeys, target,
-               sources, atomic_ret, cq, cq_producer=0, totals=None):
+               sources, atomic_ret, cq, cq_producer=0, totals=None, flush_base=0, flush_rkeys=None):
     """Retire entries [consumed, published) of one ring image (uint8, max_nwqe*64) in order.
 
     ``target`` / ``sources``: uint8 images laid out like the arena (``target`` may be None).
     ``atomic_ret``: uint64[4096]; ``cq``: uint8 image of the completion queue.  Returns
     (new cq_producer, ConsumeTotals)."""
     rk = np.ascontiguousarray(rkeys, dtype=np.uint32)
-    arena = Arena(heap_base0, slice_stride, heap_size, len(rk), rk.ctypes.data)
+    frk = None if flush_rkeys is None else np.ascontiguousarray(flush_rkeys, dtype=np.uint32)
+    arena = Arena(heap_base0, slice_stride, heap_size, len(rk), rk.ctypes.data, flush_base,
+                  None if frk is None else frk.ctypes.data)
     totals = totals if totals is not None else ConsumeTotals()
     prod = C.c_uint32(cq_producer)
     assert ring.dtype == np.uint8 and ring.flags["C_CONTIGUOUS"] and ring.size == qp.max_nwqe * 64
@@ -334,7 +341,7 @@ def sort_wqe_expect(expect):
 
 
 def ring_check(image, qp, first_counter, count, expect_sorted, heap_base0, slice_stride, heap_size,
-               rkeys, full_slot):
+               rkeys, full_slot, flush_base=0, flush_rkeys=None):
     """Entries first_counter .. first_counter+count-1 of a ring image (uint8, max_nwqe*64)
     against wqe_build (see ringcheck.c).  Returns a dict: ok, position / reason of the first
     wrong entry, used (which operations were matched), pos_count (uint32[4096] AMO return
@@ -342,7 +349,9 @@ def ring_check(image, qp, first_counter, count, expect_sorted, heap_base0, slice
     image = np.ascontiguousarray(image, dtype=np.uint8).reshape(-1)
     assert image.size == qp.max_nwqe * 64 and expect_sorted.dtype == WQE_EXPECT_DTYPE
     rk = np.ascontiguousarray(rkeys, dtype=np.uint32)
-    arena = Arena(heap_base0, slice_stride, heap_size, len(rk), rk.ctypes.data)
+    frk = None if flush_rkeys is None else np.ascontiguousarray(flush_rkeys, dtype=np.uint32)
+    arena = Arena(heap_base0, slice_stride, heap_size, len(rk), rk.ctypes.data, flush_base,
+                  None if frk is None else frk.ctypes.data)
     used = np.zeros(len(expect_sorted), dtype=np.uint8)
     pos_count = np.zeros(4096, dtype=np.uint32)
     n_atomic, n_cqe, why = C.c_uint32(0), C.c_uint32(0), C.c_int(0)

@@ -10,7 +10,13 @@
  * fourth segment), in queue order as on an RC queue pair, and the tail of the
  * completion entry the reference's quiet reads back (queue_pair.cpp:118-191:
  * op_own at byte 63 with the owner bit = bit cq_log_size of the consumer's
- * running number, opcode nibble 0; wqe_counter at bytes 60-61).
+ * running number, opcode nibble 0; wqe_counter at bytes 60-61).  The two
+ * entries that move no data are taken off the ring and completed like the
+ * others: quiet's zero-byte read (queue_pair.cpp:318-325: READ with DS = 2, the
+ * third segment is not part of the entry) and fence's flush write
+ * (queue_pair.cpp:376-384: a 4-byte inline write of the value 1 to the
+ * destination's flush word under the flush key); on this path there is nothing
+ * to flush, so executing them changes no memory.
  *
  * PARITY UNPINNED: the reference holds no vector for what a consumer does.
  * The tests pin this file by construction instead: entries built by
@@ -64,8 +70,9 @@ void orc_sq_consume(const orc_qp_t *qp, const uint8_t *ring, uint32_t consumed, 
     int is_atomic = opcode == 0x11 || opcode == 0x12;
     int is_write = opcode == 0x08, is_read = opcode == 0x10;
     int ok = s[0] == 0 && get_be16(s + 1) == (uint16_t)c &&
-             (get_le32(s + 4) & 0xffffffu) == qp->ctrl_qp_sq && (is_atomic || is_write || is_read) &&
-             s[7] == (is_atomic ? 4 : 3);
+             (get_le32(s + 4) & 0xffffffu) == qp->ctrl_qp_sq && (is_atomic || is_write || is_read);
+    const int zero_byte_read = is_read && s[7] == 2;
+    ok = ok && (zero_byte_read || s[7] == (is_atomic ? 4 : 3));
     uint64_t raddr = get_be64(s + 16);
     uint32_t rkey = get_le32(s + 24);
     uint32_t size = 0;
@@ -77,6 +84,8 @@ void orc_sq_consume(const orc_qp_t *qp, const uint8_t *ring, uint32_t consumed, 
       ok = ok && (raddr & 7) == 0 && get_be32(s + 48) == 8 && get_le32(s + 52) == qp->atomic_lkey &&
            (laddr & 7) == 0 && laddr >= qp->atomic_ret_base &&
            laddr < qp->atomic_ret_base + 8ull * 4096;
+    } else if (zero_byte_read) {
+      size = 0;           /* nothing beyond the second segment belongs to the entry */
     } else {
       uint32_t count = get_be32(s + 32);
       inl = (count >> 31) & 1;
@@ -90,14 +99,24 @@ void orc_sq_consume(const orc_qp_t *qp, const uint8_t *ring, uint32_t consumed, 
     }
     uint64_t roff = 0;
     int dest_pe = 0;
-    ok = ok && heap_offset(arena, raddr, size, &roff, &dest_pe) && rkey == arena->rkeys[dest_pe];
+    int flush_write = 0;
+    if (ok && is_write && inl && arena->flush_rkeys && raddr >= arena->flush_base &&
+        raddr - arena->flush_base < 64ull * (uint64_t)arena->num_pes) {
+      /* fence's entry: the flush word of one PE, its flush key, four bytes, the first one 1 */
+      uint64_t p = (raddr - arena->flush_base) / 64;
+      flush_write = 1;
+      ok = (raddr - arena->flush_base) % 64 == 0 && size == 4 && s[36] == 1 &&
+           rkey == arena->flush_rkeys[p];
+    } else {
+      ok = ok && heap_offset(arena, raddr, size, &roff, &dest_pe) && rkey == arena->rkeys[dest_pe];
+    }
 
     if (!ok) {
       t->rejected++;
     } else {
       t->bytes += size;
       if (is_atomic) t->atomics++; else if (is_write) t->writes++; else t->reads++;
-      if (target) {
+      if (target && !flush_write) {
         uint8_t *remote = target + roff;
         if (is_atomic) {
           uint64_t old, operand = get_be64(s + 32), compare = get_be64(s + 40);

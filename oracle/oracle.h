@@ -110,7 +110,15 @@ typedef struct orc_wqe_req {
   uint8_t inline_bytes[8];
   uint32_t atomic_pos;   /* return-slot index, already reduced modulo 4096 */
   int request_cqe;       /* completion flag byte <- 8 */
+  int form;              /* ORC_WQE_DATA, or one of the two entries that move no data */
 } orc_wqe_req_t;
+/* Forms of an entry.  ORC_WQE_ZERO_BYTE_READ: QueuePair::zero_b_rd (queue_pair.cpp:318-325),
+ * posted by quiet before it polls (thread_policy.cpp:35-108): opcode READ, DS = 2, remote
+ * address = base of the destination's heap, no data segment written.  ORC_WQE_FLUSH_WRITE:
+ * QueuePair::fence (queue_pair.cpp:376-384): a WRITE of size 0 is turned into a 4-byte inline
+ * write (queue_pair.cpp:230-233) whose first payload byte is 1 (segment_builder.cpp:110-116),
+ * addressed to the destination's flush word under the flush key (`raddr`, `rkey` as given). */
+enum { ORC_WQE_DATA = 0, ORC_WQE_ZERO_BYTE_READ = 1, ORC_WQE_FLUSH_WRITE = 2 };
 
 /* Overwrites, inside the 64-byte slot, exactly the bytes the reference writes. */
 void orc_wqe_build(uint8_t slot[64], const orc_qp_t *qp, uint32_t sq_counter,
@@ -123,6 +131,10 @@ typedef struct orc_arena {
   uint64_t heap_size;
   int num_pes;
   const uint32_t *rkeys; /* per destination PE, as stored in the entries */
+  /* Flush words (what the reference's hdp_address[] / hdp_rkey[] name, network_policy.cpp:114-180):
+   * PE p's at flush_base + 64 p under flush_rkeys[p]; flush_rkeys NULL: no flush writes expected. */
+  uint64_t flush_base;
+  const uint32_t *flush_rkeys;
 } orc_arena_t;
 
 typedef struct orc_consume_totals {

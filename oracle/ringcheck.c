@@ -14,6 +14,11 @@
  * position (bytes 56-63; counted per position so the caller can check that
  * positions are handed out densely, atomic_return.hpp:34-40).
  *
+ * The two entries that move no data are known to the checker too: a READ with
+ * DS = 2 is quiet's zero-byte read (expected as opcode 0x10, the remote address,
+ * data 0, size 0) and an inline WRITE to a flush word is fence's flush write
+ * (expected as opcode 0x08, the flush word's address, data 1, size 4); see wqe.c.
+ *
  * full_slot != 0: the ring never wrapped, bytes the builder leaves alone must
  * be zero (the ring's initial content).  full_slot == 0: the ring wrapped;
  * bytes the builder leaves alone hold what an older entry left there and are
@@ -58,8 +63,21 @@ long orc_ring_check(const uint8_t *image, const orc_qp_t *qp, uint32_t first_cou
     const uint64_t raddr = be_to_u64(slot + 16, 8);
     uint64_t data = 0, cmp = 0;
     uint32_t size = 8, pos = 0;
+    int form = ORC_WQE_DATA;
+    const int to_flush_word = arena->flush_rkeys && raddr >= arena->flush_base &&
+                              raddr - arena->flush_base < 64ull * (uint64_t)arena->num_pes;
     *why = 2; /* an opcode the stream cannot have produced */
-    if (is_atomic) {
+    if (opcode == 0x10 && slot[7] == 2) {
+      form = ORC_WQE_ZERO_BYTE_READ;
+      size = 0;
+    } else if (opcode == 0x08 && to_flush_word) {
+      const uint32_t bc = (uint32_t)be_to_u64(slot + 32, 4);
+      *why = 4;
+      if (bc != (0x80000000u | 4u) || (raddr - arena->flush_base) % 64) return 1 + (long)k;
+      form = ORC_WQE_FLUSH_WRITE;
+      size = 4;
+      data = slot[36];
+    } else if (is_atomic) {
       data = be_to_u64(slot + 32, 8);
       cmp = be_to_u64(slot + 40, 8);
       const uint64_t ret = be_to_u64(slot + 56, 8);
@@ -92,17 +110,24 @@ long orc_ring_check(const uint8_t *image, const orc_qp_t *qp, uint32_t first_cou
         expect[lo].size != size)
       return 1 + (long)k;
     used[lo] = 1;
-    /* destination slice -> the key the entry must carry */
+    /* destination slice (or flush word) -> the key the entry must carry */
     *why = 7;
-    if (raddr < arena->heap_base0) return 1 + (long)k;
-    const uint64_t pe = (raddr - arena->heap_base0) / arena->slice_stride;
-    if (pe >= (uint64_t)arena->num_pes) return 1 + (long)k;
+    uint32_t key;
+    if (form == ORC_WQE_FLUSH_WRITE) {
+      key = arena->flush_rkeys[(raddr - arena->flush_base) / 64];
+    } else {
+      if (raddr < arena->heap_base0) return 1 + (long)k;
+      const uint64_t pe = (raddr - arena->heap_base0) / arena->slice_stride;
+      if (pe >= (uint64_t)arena->num_pes) return 1 + (long)k;
+      key = arena->rkeys[pe];
+    }
     orc_wqe_req_t rq;
     memset(&rq, 0, sizeof rq);
     rq.opcode = opcode;
-    rq.size = size;
+    rq.size = form == ORC_WQE_DATA ? size : 0;
+    rq.form = form;
     rq.raddr = raddr;
-    rq.rkey = arena->rkeys[pe];
+    rq.rkey = key;
     rq.atomic_data = data;
     rq.atomic_cmp = cmp;
     for (uint32_t i = 0; i < 8; ++i) rq.inline_bytes[i] = (uint8_t)(data >> (8 * i));

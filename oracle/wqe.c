@@ -10,6 +10,8 @@
  *     (completion flag at byte 11, doorbell record and doorbell value)
  *   library/src/gpu_ib/connection_policy.cpp:45-79 (RC: one slot per operation,
  *     no address-vector segment)
+ *   library/src/gpu_ib/queue_pair.cpp:318-325,376-384 (the two entries that move
+ *     no data: quiet's zero-byte read and fence's flush write)
  * The segment layouts belong to rdma-core's <infiniband/mlx5dv.h>
  * (mlx5_wqe_ctrl_seg, mlx5_wqe_raddr_seg, mlx5_wqe_data_seg,
  * mlx5_wqe_atomic_seg, mlx5_wqe_inl_data_seg), a dependency the reference does
@@ -64,7 +66,9 @@ void orc_wqe_build(uint8_t slot[64], const orc_qp_t *qp, uint32_t sq_counter,
   slot[4] = (uint8_t)(qp->ctrl_qp_sq);
   slot[5] = (uint8_t)(qp->ctrl_qp_sq >> 8);
   slot[6] = (uint8_t)(qp->ctrl_qp_sq >> 16);
-  slot[7] = (uint8_t)(is_atomic ? 4 : 3);
+  /* DS: control + remote address (+ data) (+ atomic); a zero-byte read counts two
+   * (segment_builder.cpp:43-49). */
+  slot[7] = (uint8_t)(rq->form == ORC_WQE_ZERO_BYTE_READ ? 2 : is_atomic ? 4 : 3);
   slot[8] = (uint8_t)qp->ctrl_sig;                 /* signature */
   /* bytes 9-10 reserved: never written */
   slot[11] = (uint8_t)(qp->ctrl_sig >> 24);        /* fm_ce_se */
@@ -75,7 +79,16 @@ void orc_wqe_build(uint8_t slot[64], const orc_qp_t *qp, uint32_t sq_counter,
   put_le32(slot + 24, rq->rkey);                   /* key kept as harvested */
   /* bytes 28-31 reserved: never written */
 
-  if (is_atomic) {
+  if (rq->form == ORC_WQE_ZERO_BYTE_READ) {
+    /* zero_b_rd passes a null local address: update_data_seg returns before it
+     * writes anything (segment_builder.cpp:89-91), the third segment keeps what
+     * the slot held. */
+  } else if (rq->form == ORC_WQE_FLUSH_WRITE) {
+    /* size 0 became 4 (queue_pair.cpp:230-233); with a null local address the inline
+     * segment gets one payload byte, 1 (segment_builder.cpp:110-116). */
+    put_be32(slot + 32, 4u | 0x80000000u);
+    slot[36] = 1;
+  } else if (is_atomic) {
     /* Atomic segment (segment_builder.cpp:62-73) then a data segment that
      * names the 8-byte return slot (queue_pair.cpp:251-256). */
     put_be64(slot + 32, rq->atomic_data);

@@ -67,6 +67,7 @@ SIGNATURES = {
     "rsm_fcollect": (i32, [sz, u64, vp, vp, sz, LP]),
     "rsm_barrier_all": (i32, [i32, LP]),
     "rsm_small_ops": (i32, [vp, sz, vp, LP]),
+    "rsm_sq_flush_target": (i32, [i32, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32)]),
     "rsm_sq_reset": (i32, []),
     "rsm_sq_read": (i32, [i32, i32, C.c_uint, vp]),
     "rsm_sq_image": (i32, [i32, i32, vp, sz]),

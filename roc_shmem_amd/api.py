@@ -20,7 +20,7 @@ __all__ = [
     "roc_shmem_rma",
     "roc_shmem_broadcast", "roc_shmem_team_broadcast", "roc_shmem_alltoall",
     "roc_shmem_fcollect", "roc_shmem_wg_barrier_all", "roc_shmem_small_ops",
-    "sq_reset", "sq_read", "sq_image", "sq_state", "sq_constants", "sq_rkey",
+    "sq_reset", "sq_read", "sq_image", "sq_state", "sq_constants", "sq_rkey", "sq_flush_target",
     "sq_consume", "sq_set_mode", "sq_consumer_state", "sq_consumer_start", "sq_consumer_stop",
     "sq_consumer_running", "cq_reader_state", "cq_image", "atomic_ret_image", "arena",
     "read_device", "write_device",
@@ -428,6 +428,13 @@ def sq_rkey(dest_pe):
     k = C.c_uint32(0)
     _check(L.load().rsm_sq_rkey(dest_pe, C.byref(k)))
     return k.value
+
+
+def sq_flush_target(pe):
+    """(address, key) a fence's entry on a live queue names for PE ``pe`` (rsm_sq_flush_target)."""
+    a, k = C.c_uint64(0), C.c_uint32(0)
+    _check(L.load().rsm_sq_flush_target(pe, C.byref(a), C.byref(k)))
+    return a.value, k.value
 
 
 class ConsumeTotals(C.Structure):

@@ -468,6 +468,16 @@ int rsm_sq_rkey(int dest_pe, uint32_t *rkey) {
   return 0;
 }
 
+int rsm_sq_flush_target(int pe, uint64_t *addr, uint32_t *rkey) {
+  RSM_ENTRY;
+  RSM_NEED_RT(rt);
+  if (pe < 0 || pe >= rt->num_pes() || !addr || !rkey)
+    return rsm::fail("rsm_sq_flush_target: arguments out of range");
+  *addr = reinterpret_cast<uint64_t>(rt->flush_words()) + 64ull * static_cast<uint64_t>(pe);
+  *rkey = __builtin_bswap32(0x4000u + pe);
+  return 0;
+}
+
 // ---- host-logic hooks ------------------------------------------------------------
 
 int rsm_host_active_set_in_range(int pe_start, int log_pe_stride, int pe_size, int num_pes) {

@@ -207,10 +207,18 @@ std::string Runtime::init(const Options &opt) {
 
   // Synthetic queue-pair constants standing in for what the reference
   // harvests from a NIC-built template WQE (connection.cpp:379-391).
-  std::vector<uint32_t> rkeys(P);
-  for (int p = 0; p < P; ++p) rkeys[p] = bswap32(0x1000u + p);
-  RT_HIP(hipMalloc(reinterpret_cast<void **>(&rkeys_dev_), sizeof(uint32_t) * P));
-  RT_HIP(hipMemcpy(rkeys_dev_, rkeys.data(), sizeof(uint32_t) * P, hipMemcpyHostToDevice));
+  // Heap keys, then the flush keys (reference: hdp_rkey[], network_policy.cpp:114-180).
+  std::vector<uint32_t> rkeys(2 * static_cast<size_t>(P));
+  for (int p = 0; p < P; ++p) {
+    rkeys[p] = bswap32(0x1000u + p);
+    rkeys[P + p] = bswap32(0x4000u + p);
+  }
+  RT_HIP(hipMalloc(reinterpret_cast<void **>(&rkeys_dev_), sizeof(uint32_t) * rkeys.size()));
+  RT_HIP(hipMemcpy(rkeys_dev_, rkeys.data(), sizeof(uint32_t) * rkeys.size(), hipMemcpyHostToDevice));
+  // One 64-byte flush word per PE: what fence's entries are addressed to (the reference's
+  // hdp_address[]).  Nothing flushes through them on this path; they give the entries a target.
+  RT_HIP(hipMalloc(reinterpret_cast<void **>(&flush_words_dev_), 64 * static_cast<size_t>(P)));
+  RT_HIP(hipMemset(flush_words_dev_, 0, 64 * static_cast<size_t>(P)));
 
   ctx_images_.resize(rings);
   for (int p = 0; p < P; ++p) {
@@ -227,6 +235,8 @@ std::string Runtime::init(const Options &opt) {
       c.ring.atomic_ret_base =
           reinterpret_cast<uint64_t>(base + static_cast<size_t>(opt_.sq_size) * 64 + 64);
       c.ring.rkey_by_pe = rkeys_dev_;
+      c.ring.flush_rkey_by_pe = rkeys_dev_ + P;
+      c.ring.flush_base = reinterpret_cast<uint64_t>(flush_words_dev_);
       c.ring.ctrl_sig = 0;
       // Queue-pair number 0x000100 + ring index, laid out as the three
       // big-endian bytes that follow the opcode word of a WQE.
@@ -298,6 +308,7 @@ void Runtime::teardown() {
   if (status_dev_) (void)hipFree(status_dev_);
   if (ctx_table_dev_) (void)hipFree(ctx_table_dev_);
   if (rkeys_dev_) (void)hipFree(rkeys_dev_);
+  if (flush_words_dev_) (void)hipFree(flush_words_dev_);
   if (counters_dev_) (void)hipFree(counters_dev_);
   if (queue_mem_) (void)hipFree(queue_mem_);
   if (cq_mem_) (void)hipFree(cq_mem_);
@@ -307,6 +318,7 @@ void Runtime::teardown() {
   status_dev_ = nullptr;
   ctx_table_dev_ = nullptr;
   rkeys_dev_ = nullptr;
+  flush_words_dev_ = nullptr;
   counters_dev_ = nullptr;
   queue_mem_ = nullptr;
   cq_mem_ = nullptr;

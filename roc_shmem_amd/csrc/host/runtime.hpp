@@ -135,6 +135,7 @@ class Runtime {
   bool sq_queue_mode() const { return state_.sq_queue_mode != 0; }
   const detail::DeviceState &device_state() const { return state_; }
   char *arena() const { return arena_; }
+  char *flush_words() const { return flush_words_dev_; }
   // End (as a heap offset) of the live symmetric allocation that contains heap offset `offset`,
   // Pow2Allocator::kNoOffset when no allocation does.
   size_t allocation_end(size_t offset) const {
@@ -181,6 +182,7 @@ class Runtime {
   size_t cq_mem_bytes_ = 0;
   detail::SqCounters *counters_dev_ = nullptr;
   uint32_t *rkeys_dev_ = nullptr;
+  char *flush_words_dev_ = nullptr;
   uint32_t *status_dev_ = nullptr;
   detail::Team *teams_dev_ = nullptr;   // kMaxTeams objects
   std::vector<int> free_team_slots_;

@@ -170,18 +170,33 @@ __device__ inline T *roc_shmemx_my_addr(T *ptr) {
 // Ordering
 // ---------------------------------------------------------------------------
 
-__device__ inline void roc_shmem_ctx_fence(roc_shmem_ctx_t) { detail::fence_acq_rel_agent(); }
-__device__ inline void roc_shmem_ctx_fence(roc_shmem_ctx_t, int) { detail::fence_acq_rel_agent(); }
-__device__ inline void roc_shmem_fence() { detail::fence_acq_rel_agent(); }
-__device__ inline void roc_shmem_fence(int) { detail::fence_acq_rel_agent(); }
+// fence: what the calling PE has issued is ordered before what it issues next.
+// The operations are direct stores and atomics, which the memory fence orders.
+// On a queue with a live consumer the call also leaves the entry the
+// reference's fence posts (QueuePair::fence, queue_pair.cpp:376-384: an inline
+// write to the flush word), one per call, since a context has one queue for
+// all destinations.
+__device__ inline void roc_shmem_ctx_fence(roc_shmem_ctx_t ctx) {
+  detail::fence_acq_rel_agent();
+  if (detail::g_state.sq_queue_mode == detail::kSqLive)
+    detail::post_no_data_entry(detail::ctx_of(ctx), detail::kWqeFlushWrite);
+}
+__device__ inline void roc_shmem_ctx_fence(roc_shmem_ctx_t ctx, int) { roc_shmem_ctx_fence(ctx); }
+__device__ inline void roc_shmem_fence() { roc_shmem_ctx_fence(ROC_SHMEM_CTX_DEFAULT); }
+__device__ inline void roc_shmem_fence(int) { roc_shmem_ctx_fence(ROC_SHMEM_CTX_DEFAULT); }
 // quiet: everything the calling PE has issued is complete and visible.  The
 // operations themselves are direct stores and atomics, which the fence
 // completes.  With a live consumer on the send queues the call also collects
-// the completions its queue has asked for, as the reference's quiet does
+// the completions its queue has asked for, as the reference's quiet does: a
+// zero-byte read that asks for a completion (quiet_heavy, thread_policy.cpp:
+// 35-108; QueuePair::zero_b_rd, queue_pair.cpp:318-325), then the poll
 // (QueuePair::quiet_internal, queue_pair.cpp:118-191).
 __device__ inline void roc_shmem_ctx_quiet(roc_shmem_ctx_t ctx) {
   detail::fence_acq_rel_agent();
-  if (detail::g_state.sq_queue_mode == detail::kSqLive) detail::quiet_live(detail::ctx_of(ctx));
+  if (detail::g_state.sq_queue_mode == detail::kSqLive) {
+    detail::post_no_data_entry(detail::ctx_of(ctx), detail::kWqeZeroByteRead);
+    detail::quiet_live(detail::ctx_of(ctx));
+  }
 }
 __device__ inline void roc_shmem_quiet() { roc_shmem_ctx_quiet(ROC_SHMEM_CTX_DEFAULT); }
 __device__ inline void roc_shmem_ctx_threadfence_system(roc_shmem_ctx_t) {

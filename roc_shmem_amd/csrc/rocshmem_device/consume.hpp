@@ -10,7 +10,10 @@
 //   * checks that it is well-formed: the index field equals the slot's
 //     position in the stream, the queue number is the ring's, the remote
 //     address lies in a PE slice whose key the entry carries, atomics are
-//     8-byte aligned and name a return slot inside the ring's own window;
+//     8-byte aligned and name a return slot inside the ring's own window; the
+//     two entries that move no data (quiet's zero-byte read: READ with DS = 2;
+//     fence's flush write: 4 inline bytes, the first one 1, to a PE's flush
+//     word under its flush key) are recognised, completed and change nothing;
 //   * optionally executes it against a *target arena* laid out like the
 //     symmetric heap (RDMA WRITE, inline WRITE, RDMA READ, fetch-add,
 //     compare-and-swap, with the old value of an atomic stored to the return
@@ -75,7 +78,7 @@ __device__ __forceinline__ uint64_t heap_offset(uint64_t addr, uint64_t size, in
 // What one 64-byte entry says, and whether it is well formed.  `c` is the
 // entry's running number in its ring; w0..w7 are its eight 64-bit words.
 struct DecodedEntry {
-  bool ok, is_atomic, is_write, is_read, inl, wants_completion;
+  bool ok, is_atomic, is_write, is_read, inl, wants_completion, no_data;
   uint32_t head, opcode, size;
   uint64_t laddr, roff;
 };
@@ -97,9 +100,10 @@ __device__ __forceinline__ DecodedEntry decode_entry(const SqRing &ring, uint32_
   const bool is_atomic = opcode == kOpcodeAtomicFa || opcode == kOpcodeAtomicCs;
   const bool is_write = opcode == kOpcodeRdmaWrite;
   const bool is_read = opcode == kOpcodeRdmaRead;
+  const bool zero_byte_read = is_read && ds == 2u;
   bool ok = (head & 0xffu) == 0 && index == (c & 0xffffu) &&
             (qpn_ds & 0xffffffu) == ring.ctrl_qp_sq && (is_atomic || is_write || is_read) &&
-            ds == (is_atomic ? 4u : 3u);
+            (zero_byte_read || ds == (is_atomic ? 4u : 3u));
 
   uint32_t size = 0;
   bool inl = false;
@@ -110,6 +114,8 @@ __device__ __forceinline__ DecodedEntry decode_entry(const SqRing &ring, uint32_
          static_cast<uint32_t>(w6 >> 32) == ring.atomic_lkey;
     laddr = __builtin_bswap64(w7);
     ok = ok && (laddr & 7u) == 0 && laddr >= ret_lo && laddr < ret_hi;
+  } else if (zero_byte_read) {
+    size = 0;   // nothing beyond the second segment belongs to the entry
   } else {
     const uint32_t count = __builtin_bswap32(static_cast<uint32_t>(w4));
     inl = (count & 0x80000000u) != 0;
@@ -122,9 +128,21 @@ __device__ __forceinline__ DecodedEntry decode_entry(const SqRing &ring, uint32_
     }
   }
   int dest_pe = 0;
-  const uint64_t roff = ok ? heap_offset(raddr, size, &dest_pe) : ~0ull;
-  ok = ok && roff != ~0ull && rkey == ring.rkey_by_pe[dest_pe];
+  uint64_t roff = ~0ull;
+  bool flush_write = false;
+  if (ok && is_write && inl && raddr >= ring.flush_base &&
+      raddr - ring.flush_base < 64ull * static_cast<uint64_t>(g_state.num_pes)) {
+    const uint64_t p = (raddr - ring.flush_base) / 64u;
+    flush_write = true;
+    ok = (raddr - ring.flush_base) % 64u == 0 && size == 4u &&
+         (static_cast<uint32_t>(w4 >> 32) & 0xffu) == 1u && rkey == ring.flush_rkey_by_pe[p];
+    roff = 0;
+  } else {
+    roff = ok ? heap_offset(raddr, size, &dest_pe) : ~0ull;
+    ok = ok && roff != ~0ull && rkey == ring.rkey_by_pe[dest_pe];
+  }
   DecodedEntry d;
+  d.no_data = flush_write || zero_byte_read;
   d.ok = ok;
   d.is_atomic = is_atomic;
   d.is_write = is_write;
@@ -275,7 +293,7 @@ __device__ __forceinline__ void consume_ring(const DeviceCtx *ctx, char *target,
       } else {
         ++t.reads;
       }
-      if (target != nullptr) {
+      if (target != nullptr && !d.no_data) {
         char *remote = target + roff;
         if (is_atomic) {
           if (lane == 0) {

@@ -68,6 +68,11 @@ struct SqRing {
   uint64_t *cq;
   uint32_t cq_size;
   uint32_t cq_log_size;
+  // Flush words (reference: hdp_address[] / hdp_rkey[], network_policy.cpp:114-180; what a
+  // fence's entry is addressed to, queue_pair.cpp:376-384): PE p's at flush_base + 64 p
+  // under flush_rkey_by_pe[p].  Named by entries, never written.
+  const uint32_t *flush_rkey_by_pe;
+  uint64_t flush_base;
 };
 
 // Mutable producer indices of a ring, on their own cache line.
@@ -140,8 +145,8 @@ struct DeviceState {
 // units must agree on how they use shared memory (3: the barrier pool holds
 // call counts, not flags that are reset; 4: live queues, cq_consumer;
 // 5: arguments rebased into the caller's slice; 6: pacing; 7: paced bursts follow a
-// schedule of start times).
-constexpr uint32_t kStateRevision = 7;
+// schedule of start times; 8: quiet and fence post on live queues).
+constexpr uint32_t kStateRevision = 8;
 constexpr uint32_t kStateLayout =
     (kStateRevision * 0x01000193u) ^
     static_cast<uint32_t>(sizeof(DeviceState) | (sizeof(DeviceCtx) << 8) | (sizeof(Team) << 16) |

@@ -13,7 +13,14 @@
 //     atomic    : BE64 swap_add | BE64 compare
 //   3 atomic only: BE32 8 | atomic_lkey | BE64 &atomic_ret[pos]
 // Bytes the reference never writes (inline padding, segment 3 of non-atomic
-// entries) are left as the ring holds them.
+// entries) are left as the ring holds them.  Two entries move no data: the
+// zero-byte read that quiet posts before it polls (QueuePair::zero_b_rd,
+// queue_pair.cpp:318-325; thread_policy.cpp:35-108): opcode READ, DS = 2, remote
+// address = the destination's heap base, third segment not written; and the
+// flush write that fence posts (QueuePair::fence, queue_pair.cpp:376-384): a
+// WRITE of size 0 becomes a 4-byte inline write (queue_pair.cpp:230-233) whose
+// first payload byte is 1 (segment_builder.cpp:110-116), addressed to the
+// destination's flush word under the flush key.
 //
 // What differs from the reference is how lanes get their slots.  The
 // reference serialises waves with a per-queue spin lock and lets every lane
@@ -61,6 +68,8 @@ __device__ __forceinline__ uint32_t be64_second(uint64_t v) {
   return __builtin_bswap32(static_cast<uint32_t>(v));
 }
 
+enum WqeForm : uint8_t { kWqeData = 0, kWqeZeroByteRead = 1, kWqeFlushWrite = 2 };
+
 struct WqeRequest {
   uint8_t opcode;
   uint32_t size;         // bytes the entry covers (already merged by the coalescer)
@@ -70,6 +79,7 @@ struct WqeRequest {
   uint64_t atomic_cmp;   // compare operand (0 for fetch-add)
   uint64_t inline_data;  // payload bytes, little-endian packed, when size <= 8 and WRITE
   int pe;
+  WqeForm form = kWqeData;
 };
 
 // Post one entry per lane that passes `sends == true`.  Called by every lane
@@ -144,7 +154,7 @@ __device__ __forceinline__ void wave_post_with(DeviceCtx *ctx, bool sends, const
     const bool inl = rq.opcode == kOpcodeRdmaWrite && rq.size <= kInlineThreshold;
 
     // Segment 0: control.
-    const uint32_t ds = is_atomic ? 4u : 3u;
+    const uint32_t ds = rq.form == kWqeZeroByteRead ? 2u : is_atomic ? 4u : 3u;
     u32x4 c;
     c.x = (static_cast<uint32_t>(rq.opcode) << 24) |
           (static_cast<uint32_t>(__builtin_bswap16(idx16)) << 8);
@@ -161,11 +171,16 @@ __device__ __forceinline__ void wave_post_with(DeviceCtx *ctx, bool sends, const
     u32x4 r;
     r.x = be64_first(rq.raddr);
       r.y = be64_second(rq.raddr);
-    r.z = ring.rkey_by_pe[rq.pe];
+    r.z = rq.form == kWqeFlushWrite ? ring.flush_rkey_by_pe[rq.pe] : ring.rkey_by_pe[rq.pe];
     r.w = 0;
     __builtin_amdgcn_raw_buffer_store_b128(r, ring_mem, at + 16u, 0, kThrough);
 
-    if (is_atomic) {
+    if (rq.form == kWqeZeroByteRead) {
+      // no third segment
+    } else if (rq.form == kWqeFlushWrite) {
+      __builtin_amdgcn_raw_buffer_store_b32(be32(4u | 0x80000000u), ring_mem, at + 32u, 0, kThrough);
+      __builtin_amdgcn_raw_buffer_store_b8(static_cast<uint8_t>(1), ring_mem, at + 36u, 0, kThrough);
+    } else if (is_atomic) {
       u32x4 a;
       a.x = be64_first(rq.atomic_data);
       a.y = be64_second(rq.atomic_data);
@@ -273,6 +288,31 @@ __device__ __forceinline__ void quiet_live(DeviceCtx *ctx) {
   __hip_atomic_store(reinterpret_cast<unsigned long long *>(&ring.mailbox[2]),
                      static_cast<unsigned long long>(be32(number + 1)), __ATOMIC_RELAXED,
                      __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ void wave_post(DeviceCtx *ctx, bool sends, const WqeRequest &rq);
+
+// The entries quiet and fence leave on a queue with a live consumer, posted by
+// the lowest active lane of the calling wave (the reference's multi-thread
+// policy picks one lane per wave the same way, thread_policy.cpp:40-71).  The
+// reference posts one per destination queue pair; a context here has one queue
+// for all destinations, so it posts one, addressed to the calling PE.
+__device__ __forceinline__ void post_no_data_entry(DeviceCtx *ctx, WqeForm form) {
+  const uint64_t active = __ballot(true);
+  WqeRequest rq;
+  rq.opcode = form == kWqeZeroByteRead ? kOpcodeRdmaRead : kOpcodeRdmaWrite;
+  rq.size = 0;
+  rq.raddr = form == kWqeZeroByteRead
+                 ? reinterpret_cast<uint64_t>(g_state.heap_base0) +
+                       static_cast<uint64_t>(ctx->my_pe) * g_state.slice_stride
+                 : ctx->ring.flush_base + 64ull * static_cast<uint64_t>(ctx->my_pe);
+  rq.laddr = 0;
+  rq.atomic_data = 0;
+  rq.atomic_cmp = 0;
+  rq.inline_data = 0;
+  rq.pe = ctx->my_pe;
+  rq.form = form;
+  wave_post(ctx, lane_id() == static_cast<uint32_t>(__builtin_ctzll(active)), rq);
 }
 
 // A ring that only one workgroup feeds (at most ROC_SHMEM_NUM_BLOCKS

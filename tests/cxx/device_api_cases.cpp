@@ -15,6 +15,7 @@
 #include <vector>
 
 #include "roc_shmem.hpp"
+#include "rocshmem_mi355x.h"
 
 using namespace rocshmem;
 
@@ -1225,6 +1226,83 @@ static void put_quiet_flag() {
   roc_shmem_free(s_buf);
 }
 
+// ---- fence and quiet on queues with a live consumer -----------------------------------------
+// Reference: roc_shmem_ctx_fence posts an inline write to the destination's flush word
+// (QueuePair::fence, queue_pair.cpp:376-384) and roc_shmem_ctx_quiet a zero-byte read before it
+// polls for completions (quiet_heavy, thread_policy.cpp:35-108; zero_b_rd, queue_pair.cpp:318-325).
+// With a consumer running beside the kernel the same entries appear on the context's queue, in
+// program order between the puts, and quiet returns with every completion collected.
+__global__ void FenceQuietLiveTest(long *word) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  const int me = roc_shmem_ctx_my_pe(ctx), right = (me + 1) % roc_shmem_ctx_n_pes(ctx);
+  if (threadIdx.x == 0) {
+    roc_shmem_ctx_long_p(ctx, word, 100 + me, right);
+    roc_shmem_ctx_fence(ctx);
+    roc_shmem_ctx_long_p(ctx, word + 1, 200 + me, right);
+    roc_shmem_ctx_quiet(ctx);
+  }
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+static uint64_t be64_of(uint64_t le_word) { return __builtin_bswap64(le_word); }
+
+static void fence_quiet_live() {
+  current_case = "fence and quiet on live queues";
+  long *word = static_cast<long *>(roc_shmem_malloc(2 * sizeof(long)));
+  for (int pe = 0; pe < npes; ++pe) fill(word, 2, 0L, pe);
+  roc_shmem_barrier_all();
+  hipStream_t stream;
+  EXPECT(hipStreamCreate(&stream) == hipSuccess, "hipStreamCreate");
+  EXPECT(rsm_sq_reset() == 0, "rsm_sq_reset: %s", rsm_last_error());
+  EXPECT(rsm_sq_consumer_start() == 0, "rsm_sq_consumer_start: %s", rsm_last_error());
+  FenceQuietLiveTest<<<npes, 64, 0, stream>>>(word);
+  EXPECT(hipStreamSynchronize(stream) == hipSuccess, "hipStreamSynchronize");
+  rsm_consume_totals_t t;
+  EXPECT(rsm_sq_consumer_stop(&t) == 0, "rsm_sq_consumer_stop: %s", rsm_last_error());
+  finish_kernel("FenceQuietLiveTest");
+  EXPECT(t.retired == 4ull * npes && t.writes == 3ull * npes && t.reads == 1ull * npes && t.atomics == 0 &&
+             t.rejected == 0 && t.lost == 0 && t.bytes == (8ull + 4 + 8) * npes,
+         "totals: retired %llu writes %llu reads %llu rejected %llu lost %llu bytes %llu",
+         (unsigned long long)t.retired, (unsigned long long)t.writes, (unsigned long long)t.reads,
+         (unsigned long long)t.rejected, (unsigned long long)t.lost, (unsigned long long)t.bytes);
+  for (int pe = 0; pe < npes; ++pe) {
+    const int left = (pe + npes - 1) % npes;
+    auto got = load(word, 2, pe);
+    EXPECT(got[0] == 100 + left && got[1] == 200 + left, "PE %d holds %ld %ld", pe, got[0], got[1]);
+    uint32_t sq_counter = 0, published = 0, atomic_counter = 0, cq_consumer = 0, quiet_counter = 9, cq_db = 0;
+    uint64_t mailbox[2];
+    EXPECT(rsm_sq_state(pe, 0, &sq_counter, &published, &atomic_counter, mailbox) == 0, "rsm_sq_state");
+    EXPECT(sq_counter == 4 && published == 4, "PE %d: %u entries posted, %u published", pe, sq_counter, published);
+    EXPECT(rsm_cq_reader_state(pe, 0, &cq_consumer, &quiet_counter, &cq_db) == 0, "rsm_cq_reader_state");
+    EXPECT(quiet_counter == 0 && cq_consumer == 4, "PE %d: quiet left %u completions, took %u", pe,
+           quiet_counter, cq_consumer);
+    uint64_t flush_addr = 0;
+    uint32_t flush_key = 0, heap_key = 0;
+    EXPECT(rsm_sq_flush_target(pe, &flush_addr, &flush_key) == 0 && rsm_sq_rkey(pe, &heap_key) == 0, "keys");
+    uint64_t e[8];
+    // entry 1: fence's flush write
+    EXPECT(rsm_sq_read(pe, 0, 1, e) == 0, "rsm_sq_read");
+    const uint8_t *b = reinterpret_cast<const uint8_t *>(e);
+    EXPECT(b[3] == 0x08 && b[7] == 3 && b[1] == 0 && b[2] == 1 && b[11] == 8, "PE %d fence entry: control %02x ds %u",
+           pe, b[3], b[7]);
+    EXPECT(be64_of(e[2]) == flush_addr && static_cast<uint32_t>(e[3]) == flush_key,
+           "PE %d fence entry: address %llx key %x", pe, (unsigned long long)be64_of(e[2]),
+           static_cast<uint32_t>(e[3]));
+    EXPECT(b[32] == 0x80 && b[33] == 0 && b[34] == 0 && b[35] == 4 && b[36] == 1, "PE %d fence entry: inline segment", pe);
+    // entry 3: quiet's zero-byte read, addressed to the PE's own heap
+    EXPECT(rsm_sq_read(pe, 0, 3, e) == 0, "rsm_sq_read");
+    EXPECT(b[3] == 0x10 && b[7] == 2 && b[2] == 3 && b[11] == 8, "PE %d quiet entry: opcode %02x ds %u", pe, b[3], b[7]);
+    EXPECT(be64_of(e[2]) == reinterpret_cast<uint64_t>(rsm_heap_base(pe)) && static_cast<uint32_t>(e[3]) == heap_key,
+           "PE %d quiet entry: address %llx", pe, (unsigned long long)be64_of(e[2]));
+    EXPECT(e[4] == 0 && e[5] == 0 && e[6] == 0 && e[7] == 0, "PE %d quiet entry wrote beyond its two segments", pe);
+  }
+  EXPECT(hipStreamDestroy(stream) == hipSuccess, "hipStreamDestroy");
+  roc_shmem_free(word);
+}
+
 int main() {
   if (!getenv("ROC_SHMEM_NUM_PES")) setenv("ROC_SHMEM_NUM_PES", "4", 1);
   setenv("ROC_SHMEM_HEAP_SIZE", "67108864", 0);
@@ -1244,7 +1322,8 @@ int main() {
                {"primitive_amo", primitive_amo},
                {"back_to_back_collectives", back_to_back_collectives},
                {"reference_kernels_unchanged", reference_kernels_unchanged},
-               {"put_quiet_flag", put_quiet_flag}};
+               {"put_quiet_flag", put_quiet_flag},
+               {"fence_quiet_live", fence_quiet_live}};
   for (auto &c : cases) {
     const int before = failures;
     c.run();

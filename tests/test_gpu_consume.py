@@ -330,8 +330,10 @@ def test_live_consumer_retires_entries_while_producers_post(wgs, wg_size, num_bl
             totals = rs.sq_consumer_stop()
         assert not rs.sq_consumer_running()
         assert rs.take_status() == 0, "a producer's wait for queue space or a quiet gave up"
-        assert totals["retired"] == 2 * n_ops and totals["lost"] == 0 and totals["rejected"] == 0
-        assert totals["bytes"] == 16 * n_ops
+        # besides the operations, every workgroup's closing quiet posts one zero-byte read per launch
+        quiets = 2 * n_pes * wgs
+        assert totals["retired"] == 2 * n_ops + quiets and totals["lost"] == 0 and totals["rejected"] == 0
+        assert totals["bytes"] == 16 * n_ops and totals["reads"] == quiets
         for p in range(n_pes):
             assert np.array_equal(mem.read(p), heap.view(p, 0, words, np.int64)), "heap of PE %d" % p
         for pe in range(n_pes):

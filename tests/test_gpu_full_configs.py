@@ -150,10 +150,12 @@ class Config4:
         for p in range(self.n_pes):
             assert np.array_equal(mem.read(p), heap.view(p, 0, self.words, np.int64)), "heap of PE %d" % p
 
-    def check_rings(self, shifted, sq):
+    def check_rings(self, shifted, sq, live=False):
         """Every entry the rings hold against the CPU builder, byte for byte: all entries when no
         ring wrapped (then every operation must also be found exactly once), else the newest `sq`
-        of every ring."""
+        of every ring.  live: the rings were queues with a live consumer, where the quiet that ends
+        each workgroup's part of the kernel posts a zero-byte read (one workgroup per ring here:
+        one more entry per ring, its newest)."""
         n_pes, num_blocks = self.n_pes, self.num_blocks
         base0, stride = rs.heap_base(0), rs.heap_base(1) - rs.heap_base(0)
         expect = np.zeros(self.n_ops, oracle.WQE_EXPECT_DTYPE)
@@ -162,6 +164,7 @@ class Config4:
                            shifted["offset"].astype(np.int64)).astype(np.uint64)
         expect["data"] = shifted["value"].astype(np.int64).view(np.uint64)
         expect["size"] = 8
+        flush = [rs.sq_flush_target(p) for p in range(n_pes)]
         order = np.argsort(self.ring, kind="stable")
         bounds = np.searchsorted(self.ring[order], np.arange(n_pes * num_blocks + 1))
         rkeys = [rs.sq_rkey(p) for p in range(n_pes)]
@@ -172,7 +175,7 @@ class Config4:
                 mine = order[bounds[r]:bounds[r + 1]]
                 st = rs.sq_state(pe, block)
                 count = int(st["sq_counter"])
-                assert count == st["published"] == len(mine), (pe, block)
+                assert count == st["published"] == len(mine) + (1 if live else 0), (pe, block)
                 assert st["atomic_counter"] == int((~self.is_put[mine]).sum())
                 wrapped = count > sq
                 first = count - sq if wrapped else 0
@@ -181,12 +184,21 @@ class Config4:
                 qp = oracle.Qp()
                 qp.ctrl_qp_sq, qp.ctrl_sig, qp.lkey = c["ctrl_qp_sq"], c["ctrl_sig"], c["lkey"]
                 qp.atomic_lkey, qp.atomic_ret_base, qp.max_nwqe = c["atomic_lkey"], c["atomic_ret_base"], sq
-                res = oracle.ring_check(image, qp, first, count - first, oracle.sort_wqe_expect(expect[mine]),
-                                        base0, stride, self.slice_bytes * 4, rkeys, full_slot=not wrapped)
+                mine_expect = expect[mine]
+                if live:
+                    quiet_entry = np.zeros(1, oracle.WQE_EXPECT_DTYPE)
+                    quiet_entry["opcode"], quiet_entry["raddr"] = oracle.OP_READ, base0 + pe * stride
+                    mine_expect = np.concatenate([mine_expect, quiet_entry])
+                res = oracle.ring_check(image, qp, first, count - first, oracle.sort_wqe_expect(mine_expect),
+                                        base0, stride, self.slice_bytes * 4, rkeys, full_slot=not wrapped,
+                                        flush_base=flush[0][0], flush_rkeys=[k for _, k in flush])
                 assert res["ok"], "ring %d/%d entry %d: %s" % (pe, block, first + res["position"], res["reason"])
                 checked += count - first
                 newest = image[(count - 1) % sq]
                 assert newest[11] == 8, "the entry that closes the last post asks for a completion"
+                if live:    # READ, two segments, addressed to the issuing PE's heap
+                    assert newest[3] == oracle.OP_READ and newest[7] == 2
+                    assert int.from_bytes(bytes(newest[16:24]), "big") == base0 + pe * stride
                 assert np.array_equal(st["mailbox"], oracle.doorbell(newest, count))
                 if not wrapped:
                     assert res["used"].all(), "an operation of ring %d/%d left no entry" % (pe, block)
@@ -244,11 +256,13 @@ def test_config4_through_queues_with_a_live_consumer_nothing_lost():
         finally:
             totals = rs.sq_consumer_stop()
         assert totals["lost"] == 0 and totals["rejected"] == 0, totals
-        assert totals["retired"] == cfg.n_ops and totals["bytes"] == 8 * cfg.n_ops
+        # every workgroup's closing quiet posts one zero-byte read before it collects completions
+        assert totals["retired"] == cfg.n_ops + cfg.wgs_total and totals["bytes"] == 8 * cfg.n_ops
         assert totals["writes"] == cfg.n_ops // 2 and totals["atomics"] == cfg.n_ops // 2
+        assert totals["reads"] == cfg.wgs_total
         assert rs.take_status() == 0
         cfg.check_heap(mem)
-        assert cfg.check_rings(shifted, 1024) == cfg.n_pes * cfg.num_blocks * 1024
+        assert cfg.check_rings(shifted, 1024, live=True) == cfg.n_pes * cfg.num_blocks * 1024
         completions = 0
         for pe in range(cfg.n_pes):
             for block in range(cfg.num_blocks):

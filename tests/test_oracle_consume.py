@@ -281,3 +281,91 @@ def test_replay_agrees_with_the_small_operation_model():
     for i, pos in slots.items():
         if int(ops["kind"][i]) in (oracle.OP_FADD64, oracle.OP_FINC64, oracle.OP_CSWAP64, oracle.OP_FETCH64):
             assert int(ret[pos]) == u64(fetched[i]), i
+
+
+# ---- the two entries that move no data: quiet's zero-byte read, fence's flush write -------------
+
+FLUSH_BASE = 0x7F77_0000_0400
+FLUSH_RKEYS = np.array([int.from_bytes((0x4000 + p).to_bytes(4, "big"), "little") for p in range(P)],
+                       dtype=np.uint32)
+
+
+def consume_with_flush(ring, target, sources):
+    cq = np.zeros(ring.qp.max_nwqe * 64, np.uint8)
+    ret = np.zeros(4096, np.uint64)
+    prod, totals = oracle.sq_consume(ring.qp, ring.image, 0, ring.count, BASE, STRIDE, HEAP, RKEYS, target,
+                                     sources, ret, cq, 0, flush_base=FLUSH_BASE, flush_rkeys=FLUSH_RKEYS)
+    return prod, totals.as_dict(), cq.reshape(-1, 64)
+
+
+def post_raw(ring, opcode, raddr, rkey, cqe=False, **kw):
+    oracle.wqe_build(ring.slot(ring.count), ring.qp, ring.count, opcode, raddr=raddr, rkey=rkey,
+                     request_cqe=cqe, **kw)
+    ring.count += 1
+
+
+def test_zero_byte_read_and_flush_write_are_completed_and_change_nothing():
+    ring = Ring(make_qp())
+    ring.image[:] = 0xEE                        # what older entries may have left in the slots
+    src = fresh_arena(3)
+    tgt = src.copy()
+    ring.post(oracle.OP_WRITE, 1, 64, size=8, inline=b"ABCDEFGH")
+    post_raw(ring, oracle.OP_WRITE, FLUSH_BASE + 64 * 2, int(FLUSH_RKEYS[2]), cqe=True, form=oracle.WQE_FLUSH_WRITE)
+    post_raw(ring, oracle.OP_READ, addr(1, 0), int(RKEYS[1]), cqe=True, form=oracle.WQE_ZERO_BYTE_READ)
+    prod, totals, cq = consume_with_flush(ring, tgt, src)
+    expect = src.copy()
+    expect[STRIDE + 64:STRIDE + 72] = np.frombuffer(b"ABCDEFGH", np.uint8)
+    assert np.array_equal(tgt, expect)
+    assert totals == {"retired": 3, "writes": 2, "reads": 1, "atomics": 0, "bytes": 8 + 4 + 0,
+                      "completions": 2, "lost": 0, "rejected": 0, "local_skipped": 0}
+    assert prod == 2 and [int(cq[i][61]) for i in range(2)] == [1, 2]
+    # the zero-byte read's third and fourth segments are whatever the slot held
+    assert (ring.slot(2)[32:] == 0xEE).all() and ring.slot(2)[7] == 2
+
+
+def test_malformed_no_data_entries_are_rejected():
+    def one(build):
+        ring = Ring(make_qp())
+        build(ring)
+        _, totals, _ = consume_with_flush(ring, None, None)
+        return totals["rejected"], totals["retired"]
+
+    good = [
+        lambda r: post_raw(r, oracle.OP_READ, addr(2, 0), int(RKEYS[2]), form=oracle.WQE_ZERO_BYTE_READ),
+        lambda r: post_raw(r, oracle.OP_WRITE, FLUSH_BASE, int(FLUSH_RKEYS[0]), form=oracle.WQE_FLUSH_WRITE),
+    ]
+    for g in good:
+        assert one(g) == (0, 1)
+
+    def ds2_write(r):        # DS = 2 on anything but a read
+        post_raw(r, oracle.OP_WRITE, addr(0, 0), int(RKEYS[0]), size=4, inline=b"abcd")
+        r.slot(0)[7] = 2
+
+    def read_wrong_key(r):
+        post_raw(r, oracle.OP_READ, addr(2, 0), int(RKEYS[1]), form=oracle.WQE_ZERO_BYTE_READ)
+
+    def read_outside(r):
+        post_raw(r, oracle.OP_READ, BASE + P * STRIDE, int(RKEYS[0]), form=oracle.WQE_ZERO_BYTE_READ)
+
+    def flush_heap_key(r):   # a flush word named under a heap key
+        post_raw(r, oracle.OP_WRITE, FLUSH_BASE + 64, int(RKEYS[1]), form=oracle.WQE_FLUSH_WRITE)
+
+    def flush_other_pe_key(r):
+        post_raw(r, oracle.OP_WRITE, FLUSH_BASE + 64, int(FLUSH_RKEYS[2]), form=oracle.WQE_FLUSH_WRITE)
+
+    def flush_misaligned(r):
+        post_raw(r, oracle.OP_WRITE, FLUSH_BASE + 68, int(FLUSH_RKEYS[1]), form=oracle.WQE_FLUSH_WRITE)
+
+    def flush_wrong_payload(r):
+        post_raw(r, oracle.OP_WRITE, FLUSH_BASE, int(FLUSH_RKEYS[0]), form=oracle.WQE_FLUSH_WRITE)
+        r.slot(0)[36] = 0
+
+    def flush_wrong_size(r):
+        post_raw(r, oracle.OP_WRITE, FLUSH_BASE, int(FLUSH_RKEYS[0]), size=8, inline=b"\x01" + bytes(7))
+
+    def flush_beyond_the_last_pe(r):
+        post_raw(r, oracle.OP_WRITE, FLUSH_BASE + 64 * P, int(FLUSH_RKEYS[0]), form=oracle.WQE_FLUSH_WRITE)
+
+    for bad in (ds2_write, read_wrong_key, read_outside, flush_heap_key, flush_other_pe_key, flush_misaligned,
+                flush_wrong_payload, flush_wrong_size, flush_beyond_the_last_pe):
+        assert one(bad) == (1, 1), bad.__name__

@@ -36,14 +36,14 @@ def test_hand_assembled_entries():
     q = g["queue"]
     queue = qp(num(q["ctrl_qp_sq"]), num(q["ctrl_sig"]), num(q["lkey"]), num(q["atomic_lkey"]),
                num(q["atomic_ret_base"]), num(q["max_nwqe"]))
-    assert len(g["entries"]) >= 4
+    assert len(g["entries"]) >= 6 and {e.get("form", 0) for e in g["entries"]} == {0, 1, 2}
     for e in g["entries"]:
         slot = np.full(64, int(e["background"], 16), np.uint8)
         oracle.wqe_build(slot, queue, num(e["counter"]), num(e["opcode"]), size=e["size"],
                          raddr=num(e["raddr"]), rkey=num(e["rkey"]), laddr=num(e.get("laddr", 0)),
                          atomic_data=num(e.get("atomic_data", 0)), atomic_cmp=num(e.get("atomic_cmp", 0)),
                          inline=bytes.fromhex(e.get("inline", "")), atomic_pos=e.get("atomic_pos", 0),
-                         request_cqe=e["cqe"])
+                         request_cqe=e["cqe"], form=e.get("form", oracle.WQE_DATA))
         want = bytes.fromhex("".join(e["bytes"]).replace(" ", ""))
         assert len(want) == 64
         assert bytes(slot) == want, e["name"]
@@ -295,6 +295,44 @@ def test_ring_check_catches_each_kind_of_damage():
     assert not r["ok"]
     r = run_check(q, good, 0, 255, expect_of(ops[:100] + ops[101:]), True)
     assert r["reason"].startswith("no operation") and r["position"] == 100
+
+
+def test_ring_check_knows_the_two_entries_that_move_no_data():
+    # quiet's zero-byte read and fence's flush write among ordinary entries, on a ring that has
+    # wrapped (leftover bytes in the segments those entries do not write)
+    flush_base = 0x7F2000000400
+    flush_rkeys = [oracle.bswap32(0x4000 + p) for p in range(N_PES)]
+    rng = np.random.default_rng(23)
+    q = qp(n=64)
+    ops = random_ops(rng, 40)
+    ring = ring_of(q, ops, background=0xEE)
+    zero_read = (oracle.OP_READ, BASE0 + 2 * STRIDE, 0, 0, 0)
+    flush = (oracle.OP_WRITE, flush_base + 64 * 3, 1, 0, 4)
+    oracle.wqe_build(ring[40], q, 40, oracle.OP_WRITE, raddr=flush[1], rkey=flush_rkeys[3],
+                     form=oracle.WQE_FLUSH_WRITE, request_cqe=True)
+    oracle.wqe_build(ring[41], q, 41, oracle.OP_READ, raddr=zero_read[1], rkey=RKEYS[2],
+                     form=oracle.WQE_ZERO_BYTE_READ, request_cqe=True)
+    expect = expect_of(ops + [flush, zero_read])
+
+    def check(image, exp=expect, **kw):
+        return oracle.ring_check(image, q, 0, 42, exp, BASE0, STRIDE, STRIDE, RKEYS, full_slot=False,
+                                 flush_base=flush_base, flush_rkeys=flush_rkeys, **kw)
+
+    res = check(ring)
+    assert res["ok"] and res["used"].all(), res
+    assert not check(ring, expect_of(ops + [flush]))["ok"]                      # an entry nobody posted
+    for slot, byte, value, reason in ((41, 7, 3, "opcode"),                     # a read that moves data
+                                      (41, 24, 0x55, "bytes differ from the builder's"),   # its key
+                                      (40, 36, 0, "no operation"),              # the flush value
+                                      (40, 35, 8, "not an inline write of 1..8 bytes"),    # its size
+                                      (40, 27, 0x10, "bytes differ from the builder's")):  # heap key, not flush key
+        bad = ring.copy()
+        bad[slot, byte] = value
+        r = check(bad)
+        assert not r["ok"] and r["reason"].startswith(reason) and r["position"] == slot, (slot, byte, r)
+    # without the flush words declared, a write to one of them is outside every heap
+    r = oracle.ring_check(ring, q, 0, 42, expect, BASE0, STRIDE, STRIDE, RKEYS, full_slot=False)
+    assert not r["ok"] and r["position"] == 40
 
 
 def test_bulk_builder_and_threaded_small_ops_agree_with_the_scalar_forms():
