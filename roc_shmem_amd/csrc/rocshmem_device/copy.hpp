@@ -175,6 +175,11 @@ __device__ __forceinline__ void group_copy(void *dst, const void *src, size_t n,
 
 constexpr int kStreamUnroll = 8;          // 16-byte accesses per lane per pass
 constexpr int kRawBufferFlags = 0x00020000;  // untyped 32-bit data, no swizzle
+// Cache-policy bit of a raw-buffer access: sc1.  A store that carries it is
+// written through this XCD's L2 to memory (visible to the other XCDs once the
+// storing wave's s_waitcnt vmcnt(0) has passed); streaming stores run as fast
+// with it as without (write-only probe: plain, sc0, sc1, nt within 2 %).
+constexpr int kWriteThrough = 16;
 
 // Descriptor over [base, base + bytes) for a group whose lanes all pass the
 // same `base` and `bytes`.  Both go through readfirstlane here even though the

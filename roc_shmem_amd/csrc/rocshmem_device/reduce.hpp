@@ -176,6 +176,9 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
   using V = VecOf<T>;
   constexpr int E = V::kElems;
   constexpr int kNt = 2;                       // cache policy: non-temporal
+  // Results are written through to memory (kWriteThrough), so that the barrier
+  // that ends the collective need not write this XCD's L2 back (wg_flag_barrier).
+  constexpr int kStore = kNt | kWriteThrough;
 
   const int64_t stride = static_cast<int64_t>(g_state.slice_stride);
   char *src0 = const_cast<char *>(reinterpret_cast<const char *>(src)) +
@@ -253,9 +256,11 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
       __amdgpu_buffer_rsrc_t rd = uniform_rsrc(dst0 + m * member_step + b, valid);
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        __builtin_amdgcn_raw_buffer_store_b128(out[u].raw, rd, lane_off, u * access_bytes, kNt);
+        __builtin_amdgcn_raw_buffer_store_b128(out[u].raw, rd, lane_off, u * access_bytes, kStore);
     }
   }
+  // every wave has its own stores in memory before it meets the others
+  __builtin_amdgcn_s_waitcnt(0);
 }
 
 // The same reduction with the loads staged through LDS: every lane's 16-byte
@@ -279,6 +284,7 @@ __device__ __forceinline__ void reduce_vectors_lds(T *dst, const T *src, size_t 
   using V = VecOf<T>;
   constexpr int E = V::kElems;
   constexpr int kNt = 2;
+  constexpr int kStore = kNt | kWriteThrough;   // as in reduce_vectors
   const int64_t stride = static_cast<int64_t>(g_state.slice_stride);
   char *src0 = const_cast<char *>(reinterpret_cast<const char *>(src)) +
                (static_cast<int64_t>(as.pe_start) - my_pe) * stride;
@@ -330,9 +336,10 @@ __device__ __forceinline__ void reduce_vectors_lds(T *dst, const T *src, size_t 
       __amdgpu_buffer_rsrc_t rd = uniform_rsrc(dst0 + m * member_step + b, static_cast<int>(pass_bytes));
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        __builtin_amdgcn_raw_buffer_store_b128(out[u].raw, rd, lane_off, u * access_bytes, kNt);
+        __builtin_amdgcn_raw_buffer_store_b128(out[u].raw, rd, lane_off, u * access_bytes, kStore);
     }
   }
+  __builtin_amdgcn_s_waitcnt(0);
 }
 
 // Scalar path for element range [e_begin, e_end): unaligned arrays and tails.
@@ -403,6 +410,9 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
   wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, pe_stride, pe_size, psync_pe_step);
 
   constexpr size_t E = VecOf<T>::kElems;
+  // Whether this workgroup stores anything that is not written through (the
+  // element path's plain stores): decides how the closing barrier releases.
+  bool plain_stores = false;
   // The vector path stores 16-byte aligned and loads at any 4-byte alignment,
   // so it takes every pair of arrays that agree modulo 4 (all pairs of 4- and
   // 8-byte elements; 2-byte elements an even number of elements apart): the
@@ -485,8 +495,10 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
       if (lead) reduce_elements<T, Op>(all_dest, all_source, 0, lead, as, my_pe, tid, nthr);
       if (lead + nvec * E < n)
         reduce_elements<T, Op>(all_dest, all_source, lead + nvec * E, n, as, my_pe, tid, nthr);
+      plain_stores = lead != 0 || lead + nvec * E < n;
     }
   } else {
+    plain_stores = true;
     const size_t share = (n + parts - 1) / parts;
     size_t e0 = share * part;
     size_t e1 = e0 + share;
@@ -495,7 +507,8 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
     reduce_elements<T, Op>(dest, source, e0, e1, as, my_pe, tid, nthr);
   }
 
-  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size, psync_pe_step);
+  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size, psync_pe_step,
+                  !plain_stores);
 }
 
 }  // namespace detail

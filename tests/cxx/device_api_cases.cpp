@@ -1226,6 +1226,61 @@ static void put_quiet_flag() {
   roc_shmem_free(s_buf);
 }
 
+// ---- a collective's result is there when the call returns ---------------------------------------
+// Every workgroup reduces a tile of its own, round after round, writing new inputs before each
+// call and reading its whole tile of the result right after it: what the other PEs' workgroups
+// (on other XCDs) stored must be visible once the closing barrier has passed, with no help from
+// the end of a kernel.  256 KiB tiles take the streaming path (results written through to
+// memory, closing barrier without an L2 write-back); the ragged tiles take the element path for
+// their ends (plain stores, closing barrier with the write-back).
+__global__ void ResultVisibleTest(int rounds, int *src, int *dst, int *pWrk, long *pSync, int tile, int n_valid,
+                                  int *errors) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  const int me = roc_shmem_ctx_my_pe(ctx), np = roc_shmem_ctx_n_pes(ctx), w = wg_index();
+  int *my_src = roc_shmemx_my_addr(src) + static_cast<size_t>(w) * tile;    // dereferenced below
+  int *my_dst = roc_shmemx_my_addr(dst) + static_cast<size_t>(w) * tile;
+  int bad = 0;
+  for (int r = 0; r < rounds; ++r) {
+    for (int k = threadIdx.x; k < n_valid; k += blockDim.x) my_src[k] = (me + 1) * (k % 1021 + r) + w;
+    roc_shmem_ctx_int_sum_wg_to_all(ctx, dst + static_cast<size_t>(w) * tile, src + static_cast<size_t>(w) * tile,
+                                    n_valid, 0, 0, np, pWrk, pSync + w * ROC_SHMEM_REDUCE_SYNC_SIZE);
+    const int pes_sum = np * (np + 1) / 2;
+    for (int k = threadIdx.x; k < n_valid; k += blockDim.x)
+      if (my_dst[k] != pes_sum * (k % 1021 + r) + np * w) ++bad;
+  }
+  if (bad) atomicAdd(errors, bad);
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+static void result_visible_after_collective() {
+  current_case = "collective result visible on return";
+  const int wgs = 8, tile = 64 << 10, rounds = 60;
+  int *src = static_cast<int *>(roc_shmem_malloc(sizeof(int) * wgs * tile));
+  int *dst = static_cast<int *>(roc_shmem_malloc(sizeof(int) * wgs * tile));
+  int *pWrk = static_cast<int *>(roc_shmem_malloc(sizeof(int) * ROC_SHMEM_REDUCE_MIN_WRKDATA_SIZE));
+  long *pSync = static_cast<long *>(roc_shmem_malloc(sizeof(long) * wgs * ROC_SHMEM_REDUCE_SYNC_SIZE));
+  int *errors;
+  EXPECT(hipMalloc(&errors, sizeof(int)) == hipSuccess, "hipMalloc");
+  for (int pe = 0; pe < npes; ++pe) fill(pSync, wgs * ROC_SHMEM_REDUCE_SYNC_SIZE, 0L, pe);
+  for (int n_valid : {tile, tile - 3}) {          // aligned tiles; tiles with a ragged end
+    EXPECT(hipMemset(errors, 0, sizeof(int)) == hipSuccess, "hipMemset");
+    roc_shmem_barrier_all();
+    ResultVisibleTest<<<npes * wgs, 512>>>(rounds, src, dst, pWrk, pSync, tile, n_valid, errors);
+    finish_kernel("ResultVisibleTest");
+    int bad = -1;
+    EXPECT(hipMemcpy(&bad, errors, sizeof(int), hipMemcpyDeviceToHost) == hipSuccess, "copy");
+    EXPECT(bad == 0, "%d elements of a result were not there when the call returned (n = %d)", bad, n_valid);
+  }
+  EXPECT(hipFree(errors) == hipSuccess, "hipFree");
+  roc_shmem_free(pSync);
+  roc_shmem_free(pWrk);
+  roc_shmem_free(dst);
+  roc_shmem_free(src);
+}
+
 // ---- fence and quiet on queues with a live consumer -----------------------------------------
 // Reference: roc_shmem_ctx_fence posts an inline write to the destination's flush word
 // (QueuePair::fence, queue_pair.cpp:376-384) and roc_shmem_ctx_quiet a zero-byte read before it
@@ -1323,6 +1378,7 @@ int main() {
                {"back_to_back_collectives", back_to_back_collectives},
                {"reference_kernels_unchanged", reference_kernels_unchanged},
                {"put_quiet_flag", put_quiet_flag},
+               {"result_visible_after_collective", result_visible_after_collective},
                {"fence_quiet_live", fence_quiet_live}};
   for (auto &c : cases) {
     const int before = failures;
