@@ -47,6 +47,9 @@ __device__ __forceinline__ void copy_passes_to_members(char *dst0, const char *s
                                                        uint32_t tid, uint32_t nthr,
                                                        size_t first_pass, size_t pass_step) {
   constexpr int kNt = 2;
+  // written through to memory, and waited for below, so that the collective's closing
+  // barrier need not write this XCD's L2 back (wg_flag_barrier, written_through)
+  constexpr int kStore = kNt | kWriteThrough;
   const uint32_t lane_off = tid * 16u;
   const uint32_t access_bytes = nthr * 16u;
   const uint32_t pass_bytes = access_bytes * U;
@@ -89,9 +92,10 @@ __device__ __forceinline__ void copy_passes_to_members(char *dst0, const char *s
       __amdgpu_buffer_rsrc_t rd = uniform_rsrc(dst0 + m * member_step + b, valid);
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        __builtin_amdgcn_raw_buffer_store_b128(v[u], rd, lane_off, u * access_bytes, kNt);
+        __builtin_amdgcn_raw_buffer_store_b128(v[u], rd, lane_off, u * access_bytes, kStore);
     }
   }
+  __builtin_amdgcn_s_waitcnt(0);
 }
 
 // Copy `n` bytes from `src` into the same symmetric address `dst_mine` of
@@ -103,13 +107,15 @@ __device__ __forceinline__ void copy_passes_to_members(char *dst0, const char *s
 // `first_pass` / `pass_step` (vector path only; the caller checks alignment
 // and size first) restrict the call to passes first_pass, first_pass +
 // pass_step, ... of the vector body, and `edges` says whether this caller
-// moves the unaligned head and tail bytes.
-__device__ __forceinline__ void wg_copy_to_members(char *dst_mine, const char *src, size_t n,
+// moves the unaligned head and tail bytes.  Returns whether everything this
+// caller stored was written through to memory and waited for (the vector
+// body is; head, tail and payloads under 256 bytes are plain stores).
+__device__ __forceinline__ bool wg_copy_to_members(char *dst_mine, const char *src, size_t n,
                                                    const ActiveSet &as, int my_pe, int skip_idx,
                                                    uint32_t tid, uint32_t nthr,
                                                    size_t first_pass = 0, size_t pass_step = 1,
                                                    bool edges = true) {
-  if (n == 0) return;
+  if (n == 0) return true;
   const int64_t stride = static_cast<int64_t>(g_state.slice_stride);
   char *dst0 = dst_mine + (static_cast<int64_t>(as.pe_start) - my_pe) * stride;
   const int64_t member_step = stride * as.pe_stride;
@@ -123,7 +129,7 @@ __device__ __forceinline__ void wg_copy_to_members(char *dst_mine, const char *s
       if (m == skip_idx) continue;
       group_copy_uniform(dst0 + m * member_step, src, n, tid, nthr);
     }
-    return;
+    return false;
   }
   const size_t head = stream_head(dst_mine, n);
   const size_t body = (n - head) & ~static_cast<size_t>(15);
@@ -149,6 +155,7 @@ __device__ __forceinline__ void wg_copy_to_members(char *dst_mine, const char *s
     copy_passes_to_members<false>(dst0 + head, src + head, body, member_step, ndst, skip_at, tid, nthr,
                                   first_pass, pass_step);
   }
+  return !(edges && head + tail != 0);
 }
 
 // Broadcast `nbytes` from the root member's `source` to every other member's
@@ -194,17 +201,18 @@ __device__ __forceinline__ void wg_broadcast_bytes(int my_pe, void *dest, const 
 
   const char *root_src = translate(static_cast<const char *>(source), my_pe, as.pe_at(root_idx));
   const size_t pass_bytes = static_cast<size_t>(nthr) * 16u * kStreamUnroll;
+  bool through;
   if (nbytes >= 2 * parts * pass_bytes) {
-    wg_copy_to_members(static_cast<char *>(dest), root_src, nbytes, as, my_pe, root_idx, tid, nthr,
-                       part, parts, part == 0);
+    through = wg_copy_to_members(static_cast<char *>(dest), root_src, nbytes, as, my_pe, root_idx, tid,
+                                 nthr, part, parts, part == 0);
   } else {
     size_t b, e;
     split_range(nbytes, static_cast<int>(parts), static_cast<int>(part), 256, b, e);
-    wg_copy_to_members(static_cast<char *>(dest) + b, root_src + b, e - b, as, my_pe, root_idx,
-                       tid, nthr);
+    through = wg_copy_to_members(static_cast<char *>(dest) + b, root_src + b, e - b, as, my_pe,
+                                 root_idx, tid, nthr);
   }
 
-  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size);
+  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size, 0, through);
 }
 
 // Alltoall block exchange: member i's block j goes to member j's block i,
@@ -246,7 +254,20 @@ __device__ __forceinline__ void wg_alltoall_bytes(int my_pe, void *dest, const v
   const size_t len = e - b;
   const uintptr_t alike = reinterpret_cast<uintptr_t>(dst_mine + b) |
                           reinterpret_cast<uintptr_t>(src + b) | block_bytes | len;
-  if (len != 0 && len <= static_cast<size_t>(nthr) * 16u && (alike & 15u) == 0) {
+  bool through = false;
+  if (len >= kNonTemporalBytes && (alike & 15u) == 0 && stream_head(dst_mine + b, len) == 0) {
+    // Large ranges between aligned blocks: the streaming loop itself, its stores written
+    // through and waited for, so that the closing barrier skips the L2 write-back.
+    for (int jj = 0; jj < pe_size; ++jj) {
+      int j = my_idx + jj;      // start at the own index: concurrent members hit different slices
+      if (j >= pe_size) j -= pe_size;
+      stream_copy_uniform<2 /* nt */ | kWriteThrough, kStreamUnroll>(
+          translate(dst_mine, my_pe, as.pe_at(j)) + b, src + static_cast<size_t>(j) * block_bytes + b,
+          len, tid, nthr);
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    through = true;
+  } else if (len != 0 && len <= static_cast<size_t>(nthr) * 16u && (alike & 15u) == 0) {
     // Blocks that one access of the workgroup covers: one copy after the other
     // would be a chain of pe_size load latencies; here eight blocks' loads are in
     // flight before the first store (4 KiB or 32 KiB among 8 PEs: 9.2 -> 6.8 us per call).
@@ -287,7 +308,7 @@ __device__ __forceinline__ void wg_alltoall_bytes(int my_pe, void *dest, const v
     }
   }
 
-  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size);
+  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size, 0, through);
 }
 
 // Fcollect: member i's `block_bytes` land in block i of every member's dest
@@ -325,9 +346,9 @@ __device__ __forceinline__ void wg_fcollect_bytes(int my_pe, void *dest, const v
   const char *src = static_cast<const char *>(source);
   size_t b, e;
   split_range(block_bytes, nshards, shard, 256, b, e);
-  wg_copy_to_members(dst_mine + b, src + b, e - b, as, my_pe, -1, tid, nthr);
+  const bool through = wg_copy_to_members(dst_mine + b, src + b, e - b, as, my_pe, -1, tid, nthr);
 
-  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size);
+  wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size, 0, through);
 }
 
 // Barrier among the member workgroups (reference: internal_sync,
