@@ -132,14 +132,14 @@ int rsm_take_status(void);                      /* sticky device status word, cl
 
 /* Lockstep pacing of large sharded transfers and reductions (no counterpart in the
  * reference).  Rates are bytes of memory traffic per tick of the GPU's 100 MHz constant
- * clock; 0 switches pacing off.  Defaults: reductions 66000 (6.6 TB/s), copies 0; also
+ * clock; 0 switches pacing off.  Defaults: reductions 68000 (6.8 TB/s), copies 0; also
  * settable through ROC_SHMEM_PACE_REDUCE / ROC_SHMEM_PACE_COPY.  With a rate set, the
  * workgroups of sharded reductions and of rsm_rma(..., RSM_WG_SHARED) transfers
  * (roc_shmemx_ctx_{put,get}mem_wg_shard) that fill the chip issue their loads and stores
  * by a common schedule of time slots derived from the rate (a wave that is early waits for
  * its slot, one that is late goes at once) instead of drifting apart; results are the
  * same, only the timing changes.  A rate somewhat above what the card sustains is best
- * (fp32 sum over 8 x 2^26: 5.80 TB/s free, 6.22 at 66000, 6.03 at 90000, 5.70 at 58000);
+ * (fp32 sum over 8 x 2^26: 6.05 TB/s free, 6.37 at 68000, 6.20 at 90000, 5.78 at 58000);
  * rsm_tune_reduce_pacing measures it for one reduction on this card. */
 int rsm_set_pacing(unsigned copy_bytes_per_tick, unsigned reduce_bytes_per_tick);
 int rsm_get_pacing(unsigned *copy_bytes_per_tick, unsigned *reduce_bytes_per_tick);
@@ -155,15 +155,16 @@ int rsm_tune_reduce_pacing(int dtype, int op, void *dest, const void *source, si
                            float *paced_ms_out);
 
 /* Plain streams over a symmetric buffer, to measure what the memory system of the card at
- * hand delivers (no counterpart in the reference): the workgroups of every PE read
- * (RSM_STREAM_READ) or write (RSM_STREAM_WRITE) `bytes_per_pe` bytes at `buf` in their own
- * PE's slice, with the access pattern of the library's large transfers (128 KiB passes dealt
- * round-robin to the PE's workgroups, 16 bytes per lane per access, non-temporal).  Reads
- * alone and writes alone bound what a stream that does both can reach (the harmonic mean of
- * the two rates for a 1:1 mix); cards differ by several per cent.  The caller times the
- * launches.  READ folds all 16-byte vectors of a PE's buffer with XOR into the four 32-bit
- * words at `checksum` (symmetric, 16 bytes, zeroed by the caller) of that PE's slice; WRITE
- * stores {i mod 2^32, i >> 32, pe, seed} into vector i.  `buf` and `bytes_per_pe` must be
+ * hand delivers (no counterpart in the reference): the grid's workgroups read
+ * (RSM_STREAM_READ) or write (RSM_STREAM_WRITE) the `bytes_per_pe` bytes at `buf` of every
+ * PE's slice, one PE's after the other, with the access pattern of the library's large
+ * collectives (128 KiB passes dealt round-robin to the workgroups, all of them inside one
+ * compact window at any moment, 16 bytes per lane per access, non-temporal).  Reads alone and
+ * writes alone bound what a stream that does both can reach (the harmonic mean of the two
+ * rates for a 1:1 mix); cards differ by several per cent.  The caller times the launches.
+ * READ folds all 16-byte vectors of a PE's buffer with XOR into the four 32-bit words at
+ * `checksum` (symmetric, 16 bytes, zeroed by the caller) of that PE's slice; WRITE stores
+ * {i mod 2^32, i >> 32, pe, seed} into vector i.  `buf` and `bytes_per_pe` must be
  * multiples of 16. */
 enum rsm_stream_kind { RSM_STREAM_READ = 0, RSM_STREAM_WRITE = 1 };
 int rsm_stream_probe(int kind, void *buf, size_t bytes_per_pe, void *checksum, unsigned seed,

@@ -66,11 +66,12 @@ struct Options {
   bool rebase_args = true;
   // ROC_SHMEM_PACE_COPY / ROC_SHMEM_PACE_REDUCE: bytes per tick of the 100 MHz clock for the
   // lockstep pacing of large sharded copies / reductions (device Pacer); 0 = off.  Reductions
-  // are paced by default, at 6.6 TB/s: a little above what MI355X cards sustain, which is where
-  // the schedule gains most (it loses a quarter of its gain at 9 TB/s and none of the free rate).
+  // are paced by default, at 6.8 TB/s: a little above what MI355X cards sustain, which is where
+  // the schedule gains most (fp32 sum over 8 x 2^26, one card: 6046 GB/s free, 6190 at 62000,
+  // 6316 at 66000, 6374 at 68000, 6255 at 70000, 6196 at 90000).
   // Copies run free by default: their short passes gain nothing from the schedule.
   uint32_t pace_copy = 0;
-  uint32_t pace_reduce = 66000;
+  uint32_t pace_reduce = 68000;
   // ROC_SHMEM_REDUCE_LDS=1: rsm_to_all runs float / long / bfloat16 sums through the LDS-staged
   // form of the sharded reduction (a measured alternative, slower on MI355X; default 0).
   bool reduce_lds = false;
