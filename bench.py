@@ -411,6 +411,19 @@ def bench_putmem(rs, steps, n_pes, msg_bytes_list):
     res["getmem_67108864_shared"] = {"GBps": 2.0 * n_pes * total / ms / 1e6, "ms": ms, "calls_per_pe": total // msg,
                                      "bytes_per_call": msg, "note": "roc_shmemx_ctx_getmem_wg_shard",
                                      "launch": PUT_SHARED_LAUNCH}
+    # the reference's own launch model (driver.sh: one workgroup per PE issues the whole message with
+    # one roc_shmemx_ctx_putmem_wg call): what one compute unit moves
+    one = {}
+    launch = rs.Launch(1, 1024)
+    for m in (64 << 10, 1 << 20, 64 << 20):
+        def one_call():
+            rs.roc_shmem_rma(rs.PUT, rs.WG, dst, src, m, 1, m, m, 1, launch)
+
+        one_call()
+        rs.synchronize()
+        ms = event_time_ms(rs, one_call, steps) / steps
+        one[str(m)] = {"GBps": 2.0 * n_pes * m / ms / 1e6, "us": ms * 1e3}
+    res["one_workgroup_per_pe_one_call_per_message"] = one
     src.free()
     dst.free()
     return res
