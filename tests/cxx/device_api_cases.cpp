@@ -1281,6 +1281,66 @@ static void result_visible_after_collective() {
   roc_shmem_free(src);
 }
 
+// The same for the copying collectives: alltoall, fcollect and broadcast over the world team, each
+// checked by every PE right after it returns, with new inputs every round.  Blocks of 64 KiB take
+// the streaming path (written through, closing barrier without a write-back), blocks of 100
+// bytes the plain-store path.
+__global__ void CopiesVisibleTest(int rounds, roc_shmem_team_t team, int *src, int *dst, int nelem, int *errors) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  const int me = roc_shmem_ctx_my_pe(ctx), np = roc_shmem_ctx_n_pes(ctx);
+  int *my_src = roc_shmemx_my_addr(src), *my_dst = roc_shmemx_my_addr(dst);   // dereferenced below
+  int bad = 0;
+  for (int r = 0; r < rounds; ++r) {
+    // alltoall: my block j goes to PE j's block `me`
+    for (int k = threadIdx.x; k < np * nelem; k += blockDim.x) my_src[k] = (me << 20) + k * 7 + r;
+    roc_shmem_ctx_int_wg_alltoall(ctx, team, dst, src, nelem);
+    for (int k = threadIdx.x; k < np * nelem; k += blockDim.x) {
+      const int from = k / nelem, at = me * nelem + k % nelem;
+      if (my_dst[k] != (from << 20) + at * 7 + r) ++bad;
+    }
+    roc_shmem_ctx_wg_team_sync(ctx, team);      // everybody has checked before dst is written again
+    // fcollect: my first block lands in block `me` of everybody
+    for (int k = threadIdx.x; k < nelem; k += blockDim.x) my_src[k] = (me << 20) - k * 3 - r;
+    roc_shmem_ctx_int_wg_fcollect(ctx, team, dst, src, nelem);
+    for (int k = threadIdx.x; k < np * nelem; k += blockDim.x)
+      if (my_dst[k] != ((k / nelem) << 20) - (k % nelem) * 3 - r) ++bad;
+    roc_shmem_ctx_wg_team_sync(ctx, team);
+    // broadcast from a moving root: everybody but the root receives its first block
+    const int root = r % np;
+    for (int k = threadIdx.x; k < nelem; k += blockDim.x) my_src[k] = (me << 20) ^ (k * 5 + r);
+    roc_shmem_ctx_int_wg_broadcast(ctx, team, dst, src, nelem, root);
+    if (me != root)
+      for (int k = threadIdx.x; k < nelem; k += blockDim.x)
+        if (my_dst[k] != ((root << 20) ^ (k * 5 + r))) ++bad;
+    roc_shmem_ctx_wg_team_sync(ctx, team);
+  }
+  if (bad) atomicAdd(errors, bad);
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+static void copies_visible_after_collective() {
+  current_case = "alltoall / fcollect / broadcast results visible on return";
+  int *errors;
+  EXPECT(hipMalloc(&errors, sizeof(int)) == hipSuccess, "hipMalloc");
+  for (int nelem : {16 << 10, 25}) {
+    int *src = static_cast<int *>(roc_shmem_malloc(sizeof(int) * npes * nelem));
+    int *dst = static_cast<int *>(roc_shmem_malloc(sizeof(int) * npes * nelem));
+    EXPECT(hipMemset(errors, 0, sizeof(int)) == hipSuccess, "hipMemset");
+    roc_shmem_barrier_all();
+    CopiesVisibleTest<<<npes, 512>>>(40, ROC_SHMEM_TEAM_WORLD, src, dst, nelem, errors);
+    finish_kernel("CopiesVisibleTest");
+    int bad = -1;
+    EXPECT(hipMemcpy(&bad, errors, sizeof(int), hipMemcpyDeviceToHost) == hipSuccess, "copy");
+    EXPECT(bad == 0, "%d elements were not there when a collective returned (blocks of %d ints)", bad, nelem);
+    roc_shmem_free(dst);
+    roc_shmem_free(src);
+  }
+  EXPECT(hipFree(errors) == hipSuccess, "hipFree");
+}
+
 // ---- fence and quiet on queues with a live consumer -----------------------------------------
 // Reference: roc_shmem_ctx_fence posts an inline write to the destination's flush word
 // (QueuePair::fence, queue_pair.cpp:376-384) and roc_shmem_ctx_quiet a zero-byte read before it
@@ -1379,6 +1439,7 @@ int main() {
                {"reference_kernels_unchanged", reference_kernels_unchanged},
                {"put_quiet_flag", put_quiet_flag},
                {"result_visible_after_collective", result_visible_after_collective},
+               {"copies_visible_after_collective", copies_visible_after_collective},
                {"fence_quiet_live", fence_quiet_live}};
   for (auto &c : cases) {
     const int before = failures;
