@@ -51,7 +51,9 @@ enum rsm_op {
 
 enum rsm_rma_kind { RSM_PUT = 0, RSM_GET = 1, RSM_PUT_NBI = 2, RSM_GET_NBI = 3 };
 /* RSM_WG_SHARED: every message is moved by all workgroups of the PE together
- * (roc_shmemx_ctx_{put,get}mem_wg_shard, an extension). */
+ * (roc_shmemx_ctx_{put,get}mem_wg_shard, an extension); it is complete when the launch is
+ * (stream order): the kernel issues no quiet of its own, since a message is complete only
+ * when every workgroup that shares it has returned. */
 enum rsm_granularity { RSM_THREAD = 0, RSM_WAVE = 1, RSM_WG = 2, RSM_WG_SHARED = 3 };
 
 /* Kinds of the small-operation stream executed by rsm_small_ops(). */
