@@ -342,8 +342,10 @@ int rsm_sq_set_mode(int queue_mode);
  * the completions its queue has asked for, that entry's included (bounded waits, status word
  * on timeout); roc_shmem_ctx_fence posts the flush write of QueuePair::fence
  * (queue_pair.cpp:376-384).  Without a live consumer neither posts anything: both are memory
- * fences, and nothing would complete the entries.  Entries and completions are written through to
- * memory meanwhile.  rsm_sq_consumer_stop: call it when the producers' streams have been
+ * fences, and nothing would complete the entries.  Entries and completions are written
+ * through to memory meanwhile, and the pacing of large reductions and copies rests (rates 0;
+ * restored by rsm_sq_consumer_stop): a paced grid counts on all its workgroups being
+ * resident, which the consumer's waves may prevent.  rsm_sq_consumer_stop: call it when the producers' streams have been
  * synchronised (it synchronises the default stream itself); it lets the consumer drain the
  * rings, waits for it, restores the previous mode and returns what was retired.  Between
  * the two calls synchronise streams, not the device: entry points that synchronise the

@@ -41,6 +41,9 @@ struct LiveConsumer {
   detail::LiveControl *control = nullptr;   // host memory the device can address
   bool running = false;
   uint32_t mode_before = detail::kSqLog;
+  // pacing rates that were set when the consumer started: a paced grid assumes that all of its
+  // workgroups are resident, which the consumer's waves may prevent, so pacing rests meanwhile
+  uint32_t pace_copy_before = 0, pace_reduce_before = 0;
 };
 LiveConsumer g_live;
 
@@ -114,7 +117,9 @@ int rsm_sq_consumer_start(void) {
   // Everything launched so far has finished before the rings change hands.
   CONSUME_HIP(hipDeviceSynchronize());
   g_live.mode_before = rt->device_state().sq_queue_mode;
-  if (!rt->set_sq_mode(detail::kSqLive))
+  g_live.pace_copy_before = rt->device_state().pace_copy_bytes_per_tick;
+  g_live.pace_reduce_before = rt->device_state().pace_reduce_bytes_per_tick;
+  if (!rt->set_sq_mode(detail::kSqLive) || !rt->set_pacing(0, 0))
     return rsm::fail("rsm_sq_consumer_start: could not update the device state");
   *g_live.control = detail::LiveControl{};
   detail::ConsumeTotals *totals = static_cast<detail::ConsumeTotals *>(rt->result_scratch());
@@ -131,6 +136,7 @@ int rsm_sq_consumer_start(void) {
   hipError_t launched = hipGetLastError();
   if (launched != hipSuccess) {
     (void)rt->set_sq_mode(g_live.mode_before);
+    (void)rt->set_pacing(g_live.pace_copy_before, g_live.pace_reduce_before);
     return rsm::fail(std::string("rsm_sq_consumer_start: ") + hipGetErrorString(launched));
   }
   g_live.running = true;
@@ -158,7 +164,8 @@ int rsm_sq_consumer_stop(rsm_consume_totals_t *totals) {
   hipError_t waited = hipStreamSynchronize(g_live.stream);
   g_live.running = false;
   const bool expired = __atomic_load_n(&g_live.control->expired, __ATOMIC_ACQUIRE) != 0;
-  const bool mode_ok = rt->set_sq_mode(g_live.mode_before);
+  const bool mode_ok = rt->set_sq_mode(g_live.mode_before) &&
+                       rt->set_pacing(g_live.pace_copy_before, g_live.pace_reduce_before);
   if (waited != hipSuccess)
     return rsm::fail(std::string("rsm_sq_consumer_stop: ") + hipGetErrorString(waited));
   rsm_consume_totals_t host = {};

@@ -309,8 +309,10 @@ def test_live_consumer_retires_entries_while_producers_post(wgs, wg_size, num_bl
         heap = oracle.Heap(n_pes, words * 8)
         stream = rs.Stream()
         rs.sq_reset()
+        pacing = rs.get_pacing()
         rs.sq_consumer_start()
         assert rs.sq_consumer_running()
+        assert rs.get_pacing() == (0, 0), "pacing rests while consumer waves hold compute units"
         devs = []
         try:
             with pytest.raises(rs.RocShmemError, match="live send-queue consumer"):
@@ -329,6 +331,7 @@ def test_live_consumer_retires_entries_while_producers_post(wgs, wg_size, num_bl
         finally:
             totals = rs.sq_consumer_stop()
         assert not rs.sq_consumer_running()
+        assert rs.get_pacing() == pacing and pacing[1] != 0
         assert rs.take_status() == 0, "a producer's wait for queue space or a quiet gave up"
         # besides the operations, every workgroup's closing quiet posts one zero-byte read per launch
         quiets = 2 * n_pes * wgs
