@@ -158,17 +158,33 @@ int rsm_tune_reduce_pacing(int dtype, int op, void *dest, const void *source, si
 
 /* Plain streams over a symmetric buffer, to measure what the memory system of the card at
  * hand delivers (no counterpart in the reference): the grid's workgroups read
- * (RSM_STREAM_READ) or write (RSM_STREAM_WRITE) the `bytes_per_pe` bytes at `buf` of every
- * PE's slice, one PE's after the other, with the access pattern of the library's large
- * collectives (128 KiB passes dealt round-robin to the workgroups, all of them inside one
- * compact window at any moment, 16 bytes per lane per access, non-temporal).  Reads alone and
- * writes alone bound what a stream that does both can reach (the harmonic mean of the two
- * rates for a 1:1 mix); cards differ by several per cent.  The caller times the launches.
+ * (RSM_STREAM_READ), write (RSM_STREAM_WRITE) or copy (RSM_STREAM_COPY: the first half onto
+ * the second half) the `bytes_per_pe` bytes at `buf` of every PE's slice, one PE's after
+ * the other, in passes dealt round-robin to the workgroups, all of them inside one compact
+ * window at any moment, 16 bytes per lane per access, loads non-temporal, stores with the
+ * policy of the collectives' results.  launch->tile is the size of a pass in bytes,
+ * wg_size * 16 * {1, 2, 4, 8} (0 = 8 accesses, the 128 KiB passes of the library's large
+ * collectives at 1024 lanes).  The shape of the launch matters more than the card: workgroups
+ * that stay and take pass after pass, as a device-side collective's do, reach 6.3-6.9 TB/s
+ * one way; a grid of as many small workgroups as passes (wgs_per_pe = passes per PE, 256
+ * lanes, one access each), which the hardware hands out in address order, 7.1-7.6 TB/s;
+ * copies stay at 6.1-6.7 TB/s either way.  The caller times the launches.
  * READ folds all 16-byte vectors of a PE's buffer with XOR into the four 32-bit words at
- * `checksum` (symmetric, 16 bytes, zeroed by the caller) of that PE's slice; WRITE stores
+ * `checksum` (symmetric, 16 bytes, zeroed by the caller; NULL: the loads are performed and
+ * nothing is folded, as a timed run of many small workgroups wants) of that PE's slice; WRITE stores
  * {i mod 2^32, i >> 32, pe, seed} into vector i.  `buf` and `bytes_per_pe` must be
- * multiples of 16. */
-enum rsm_stream_kind { RSM_STREAM_READ = 0, RSM_STREAM_WRITE = 1 };
+ * multiples of 16 (32 for the copies).  For comparison, RSM_STREAM_RUNTIME_FILL and
+ * RSM_STREAM_RUNTIME_COPY run the HIP runtime's own kernels over the same buffers, one call
+ * per PE on the launch's stream (the launch's shape is not used): hipMemsetAsync of every
+ * byte to `seed` & 0xff, and hipMemcpyAsync of each buffer's first half onto its second
+ * half.  Those two are not for a stream under graph capture. */
+enum rsm_stream_kind {
+  RSM_STREAM_READ = 0,
+  RSM_STREAM_WRITE = 1,
+  RSM_STREAM_RUNTIME_FILL = 2,
+  RSM_STREAM_RUNTIME_COPY = 3,
+  RSM_STREAM_COPY = 4
+};
 int rsm_stream_probe(int kind, void *buf, size_t bytes_per_pe, void *checksum, unsigned seed,
                      const rsm_launch_t *launch);
 

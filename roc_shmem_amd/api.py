@@ -24,7 +24,7 @@ __all__ = [
     "sq_consume", "sq_set_mode", "sq_consumer_state", "sq_consumer_start", "sq_consumer_stop",
     "sq_consumer_running", "cq_reader_state", "cq_image", "atomic_ret_image", "arena",
     "read_device", "write_device",
-    "kat_fetch_incr", "kat_coalesce", "take_status", "set_pacing", "get_pacing", "tune_reduce_pacing", "stream_probe", "STREAM_READ", "STREAM_WRITE", "synchronize", "heap_bytes_in_use",
+    "kat_fetch_incr", "kat_coalesce", "take_status", "set_pacing", "get_pacing", "tune_reduce_pacing", "stream_probe", "STREAM_READ", "STREAM_WRITE", "STREAM_RUNTIME_FILL", "STREAM_RUNTIME_COPY", "STREAM_COPY", "synchronize", "heap_bytes_in_use",
     "sym_array", "Event", "device_array", "heap_base",
     "SHORT", "INT", "LONG", "LONGLONG", "FLOAT", "DOUBLE", "BF16",
     "SUM", "MAX", "MIN", "PROD", "AND", "OR", "XOR",
@@ -38,7 +38,7 @@ __all__ = [
 SHORT, INT, LONG, LONGLONG, FLOAT, DOUBLE, BF16 = range(7)
 SUM, MAX, MIN, PROD, AND, OR, XOR = range(7)
 PUT, GET, PUT_NBI, GET_NBI = range(4)
-STREAM_READ, STREAM_WRITE = range(2)
+STREAM_READ, STREAM_WRITE, STREAM_RUNTIME_FILL, STREAM_RUNTIME_COPY, STREAM_COPY = range(5)
 THREAD, WAVE, WG, WG_SHARED = range(4)
 (OP_P64, OP_FADD64, OP_ADD64, OP_FINC64, OP_INC64, OP_CSWAP64, OP_FETCH64, OP_SET64, OP_SWAP64,
  OP_P32, OP_FADD32, OP_PUTMEM, OP_GETMEM, OP_FAND64, OP_FOR64, OP_FXOR64) = range(16)
