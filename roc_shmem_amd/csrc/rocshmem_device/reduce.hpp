@@ -202,11 +202,36 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
   if (byte_begin < byte_end && byte_end - byte_begin < pass_bytes &&
       uniform((tid & ~63u) * 16u) >= byte_end - byte_begin)
     return;
-  for (size_t b = byte_begin; b < byte_end; b += step_bytes) {
-    const size_t left = byte_end - b;
-    const int valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
+  // A workgroup that fills the edges of the schedule (Pacer::fill_edges; it has two passes
+  // or more, so its first one is whole) takes the first half of its first pass, then its
+  // other passes, then the second half of the first: a half pass is the same code over a
+  // window of half the size (the descriptor clips the other accesses), at half the slot.
+  const bool halves = pacer.period != 0 && pacer.fill_edges && byte_begin + step_bytes < byte_end;
+  const uint32_t half_bytes = pass_bytes / 2;
+  int edge = halves ? 0 : 1;   // 0: first half of the first pass, 1: whole passes, 2: its second half
+  size_t next_b = byte_begin;
+  for (;;) {
+    size_t b;
+    int valid;
+    uint32_t slot = pacer.period;
+    if (edge == 1) {
+      if (next_b >= byte_end) {
+        if (!halves) break;
+        edge = 2;
+      } else {
+        b = next_b;
+        next_b += step_bytes;
+        const size_t left = byte_end - b;
+        valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
+      }
+    }
+    if (edge != 1) {
+      b = byte_begin + (edge == 0 ? 0u : half_bytes);
+      valid = static_cast<int>(half_bytes);
+      slot = pacer.period / 2;
+    }
     Acc acc[U][E];
-    pacer.wait_slot();
+    pacer.wait(slot);
     {
       __amdgpu_buffer_rsrc_t rs = uniform_rsrc(src0 + b, valid);
 #pragma unroll
@@ -251,12 +276,17 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
     for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int e = 0; e < E; ++e) out[u].e[e] = from_acc<T, Acc>(acc[u][e]);
-    pacer.wait_slot();
+    pacer.wait(slot);
     for (int m = 0; m < as.size; ++m) {
       __amdgpu_buffer_rsrc_t rd = uniform_rsrc(dst0 + m * member_step + b, valid);
 #pragma unroll
       for (int u = 0; u < U; ++u)
         __builtin_amdgcn_raw_buffer_store_b128(out[u].raw, rd, lane_off, u * access_bytes, kStore);
+    }
+    if (edge == 2) break;
+    if (edge == 0) {
+      edge = 1;
+      next_b = byte_begin + step_bytes;
     }
   }
   // every wave has its own stores in memory before it meets the others
@@ -475,8 +505,8 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
         Pacer pacer{0u, 0u};
         if (g_state.pace_reduce_bytes_per_tick != 0 && nvec * 16u >= 4 * parts * pass_bytes &&
             grid_is_resident())
-          pacer = make_pacer(g_state.pace_reduce_bytes_per_tick,
-                             parts * pass_bytes * static_cast<uint64_t>(pe_size));
+          pacer = make_edge_filling_pacer(g_state.pace_reduce_bytes_per_tick,
+                                          parts * pass_bytes * static_cast<uint64_t>(pe_size));
         if (lds_stage != nullptr) {
           // whole passes through LDS, two vectors per lane per member; what is left of the
           // range goes the usual way, to whoever's turn it would have been
