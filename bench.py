@@ -104,10 +104,13 @@ def record_traffic(fetch_csv, write_csv):
     import csv
 
     def mean_kib(path, counter, kernel_prefix):
+        # only launches that fill the chip: the copy of known size is issued by 256 workgroups, the
+        # same kernel's one-workgroup-per-PE rows of the put sweep move other amounts
         vals = []
         with open(path, newline="") as f:
             for row in csv.DictReader(f):
-                if row["Counter_Name"] == counter and row["Kernel_Name"].startswith(kernel_prefix):
+                if row["Counter_Name"] == counter and row["Kernel_Name"].startswith(kernel_prefix) and \
+                        int(row["Grid_Size"]) // int(row["Workgroup_Size"]) >= 256:
                     vals.append(float(row["Counter_Value"]))
         if not vals:
             raise SystemExit("%s: no %s rows for %s" % (path, counter, kernel_prefix))
@@ -162,7 +165,7 @@ def device_report():
 def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, cpu=False,
                  spread=False, launch_shape=None, tune=False, pace=None):
     """Returns a dict with ms_per_step, GB/s (algorithmic 2*P*N*s bytes) and optional CPU figures.
-    pace: None = the pacing rate the library holds (its default: reductions paced at 6.6 TB/s),
+    pace: None = the pacing rate the library holds (its default: reductions paced at 6.8 TB/s),
     0 = workgroups run free, another value = that rate in bytes per tick.
     tune: let the library measure, outside the timed region, which rate suits this reduction on
     this card, with the launch shapes of TUNE_SHAPES; the timed steps then run with the better

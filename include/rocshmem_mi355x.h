@@ -141,7 +141,7 @@ int rsm_take_status(void);                      /* sticky device status word, cl
  * by a common schedule of time slots derived from the rate (a wave that is early waits for
  * its slot, one that is late goes at once) instead of drifting apart; results are the
  * same, only the timing changes.  A rate somewhat above what the card sustains is best
- * (fp32 sum over 8 x 2^26: 6.05 TB/s free, 6.37 at 68000, 6.20 at 90000, 5.78 at 58000);
+ * (fp32 sum over 8 x 2^26: 6.02 TB/s free, 6.41 at 68000, 6.21 at 90000, 5.74 at 58000);
  * rsm_tune_reduce_pacing measures it for one reduction on this card. */
 int rsm_set_pacing(unsigned copy_bytes_per_tick, unsigned reduce_bytes_per_tick);
 int rsm_get_pacing(unsigned *copy_bytes_per_tick, unsigned *reduce_bytes_per_tick);
