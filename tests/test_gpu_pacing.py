@@ -42,6 +42,31 @@ def test_paced_reduction_matches_the_oracle(rate):
                 a.free()
 
 
+def test_paced_reduction_in_place_with_half_passes_at_the_edges():
+    """dest == source at the default rate and the headline's launch shape: the workgroups on odd
+    XCDs reduce the first half of their first pass first and its second half last, each byte
+    range read and then overwritten by the same lanes."""
+    n_pes, wgs, wg_size = 8, 32, 1024       # 256 workgroups, 128 KiB per member per pass
+    with runtime(n_pes, heap_size=512 << 20, num_blocks=32):
+        n = (160 << 20) // 4 + 13            # five passes per workgroup and a ragged end
+        buf = rs.sym_array(n, np.float32)
+        psync = rs.sym_array(wgs * rs.ROC_SHMEM_REDUCE_SYNC_SIZE, np.int64, fill=0)
+        heap = oracle.Heap(n_pes, n * 4)
+        for p in range(n_pes):
+            vals = random_values(rs.FLOAT, n, 70 + p)
+            buf.write(p, vals)
+            heap.view(p, 0, n, np.float32)[:] = vals
+        assert rs.get_pacing()[1] != 0       # the library's default rate is in force
+        rs.roc_shmem_to_all(rs.FLOAT, rs.SUM, buf, buf, n, 0, 0, n_pes, None, psync, rs.Launch(wgs, wg_size))
+        rs.synchronize()
+        oracle.to_all_rounded_once(heap, rs.FLOAT, rs.SUM, 0, 0, n)
+        for p in range(n_pes):
+            assert np.array_equal(buf.read(p).view(np.uint32), heap.view(p, 0, n, np.float32).view(np.uint32)), p
+        assert rs.take_status() == 0
+        psync.free()
+        buf.free()
+
+
 @pytest.mark.parametrize("rate", [40000, 66000, 90000])
 def test_paced_shared_put_and_get_are_exact(rate):
     n_pes, nbytes = 8, (40 << 20) + 4099        # 32 x 512 per PE: 20 passes per workgroup
