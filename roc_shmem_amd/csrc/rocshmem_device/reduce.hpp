@@ -499,11 +499,12 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
         reduce_vectors<T, Op, 2, 4>(dest, source, 0, nvec, as, my_pe, tid, nthr, part, parts);
       } else {
         // Paced (see Pacer) when the library holds a rate, the grid fills the chip and
-        // every workgroup has at least four passes (with two, a 32 x 1024 launch measured
-        // 4 % slower paced than free; with four, 1-2 % faster; with eight, 5-7 %).
+        // every workgroup has at least two passes (8 PEs, fp32, paced against free at the
+        // default rate: with two passes +1 % at 32 x 1024 lanes per PE, +5 % at 32 x 512,
+        // +8 % at 64 x 512; with four +2 to +6 %; with eight +6 %).
         const uint64_t pass_bytes = static_cast<uint64_t>(kReduceUnroll) * nthr * 16u;
         Pacer pacer{0u, 0u};
-        if (g_state.pace_reduce_bytes_per_tick != 0 && nvec * 16u >= 4 * parts * pass_bytes &&
+        if (g_state.pace_reduce_bytes_per_tick != 0 && nvec * 16u >= 2 * parts * pass_bytes &&
             grid_is_resident())
           pacer = make_edge_filling_pacer(g_state.pace_reduce_bytes_per_tick,
                                           parts * pass_bytes * static_cast<uint64_t>(pe_size));

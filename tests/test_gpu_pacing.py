@@ -2,8 +2,8 @@
 their loads and stores, never what they compute: results with pacing on are bit-identical to
 the oracle's, whatever the rate (too low and too high rates only cost time).  The library
 paces a call only when its grid fills the chip (at least one workgroup per compute unit, all
-of them resident) and every workgroup has several passes, so the cases below are that large:
-256 workgroups of 512 lanes, 64 MiB and more per PE."""
+of them resident) and every workgroup has two passes or more, so the cases below are that large:
+256 workgroups of 512 lanes, 32 MiB and more per PE."""
 import numpy as np
 import pytest
 
@@ -14,14 +14,14 @@ from helpers import random_values, runtime
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("rate", [40000, 64000, 90000])
-def test_paced_reduction_matches_the_oracle(rate):
+@pytest.mark.parametrize("rate,mib", [(40000, 80), (64000, 32), (90000, 80)])
+def test_paced_reduction_matches_the_oracle(rate, mib):
     n_pes, wgs, wg_size = 8, 32, 512        # 256 workgroups, 64 KiB per member per pass
     with runtime(n_pes, heap_size=512 << 20, num_blocks=32):   # power-of-two blocks: 2 x 128 MiB
         for dtype, op in ((rs.FLOAT, rs.SUM), (rs.LONG, rs.XOR), (rs.BF16, rs.MAX)):
             npd = rs.NP_DTYPE[dtype]
             es = np.dtype(npd).itemsize
-            n = (80 << 20) // es + 77          # five passes per workgroup and a ragged end
+            n = (mib << 20) // es + 77         # five (two) passes per workgroup and a ragged end
             src = rs.sym_array(n, npd)
             dst = rs.sym_array(n, npd, fill=0x5A)
             psync = rs.sym_array(wgs * rs.ROC_SHMEM_REDUCE_SYNC_SIZE, np.int64, fill=0)
