@@ -42,6 +42,30 @@ def test_paced_reduction_matches_the_oracle(rate, mib):
                 a.free()
 
 
+@pytest.mark.parametrize("n_pes,wgs,wg_size,mib", [(16, 16, 1024, 80), (4, 64, 512, 40), (2, 128, 1024, 72)])
+def test_paced_reduction_with_other_numbers_of_pes(n_pes, wgs, wg_size, mib):
+    """256 workgroups in all, two to five passes each, a ragged end, the library's default rate:
+    2, 4 and 16 members (with 2 and 4 PEs the workgroups of a PE are spread over several XCDs)."""
+    with runtime(n_pes, heap_size=512 << 20, num_blocks=wgs):   # two power-of-two blocks of 128 MiB
+        n = (mib << 20) // 4 + 41
+        src = rs.sym_array(n, np.float32)
+        dst = rs.sym_array(n, np.float32, fill=0x5A)
+        psync = rs.sym_array(wgs * rs.ROC_SHMEM_REDUCE_SYNC_SIZE, np.int64, fill=0)
+        heap = oracle.Heap(n_pes, 2 * n * 4)
+        for p in range(n_pes):
+            vals = random_values(rs.FLOAT, n, 90 + p)
+            src.write(p, vals)
+            heap.view(p, 0, n, np.float32)[:] = vals
+        assert rs.get_pacing()[1] != 0
+        rs.roc_shmem_to_all(rs.FLOAT, rs.SUM, dst, src, n, 0, 0, n_pes, None, psync, rs.Launch(wgs, wg_size))
+        rs.synchronize()
+        oracle.to_all_rounded_once(heap, rs.FLOAT, rs.SUM, n * 4, 0, n)
+        for p in range(n_pes):
+            assert np.array_equal(dst.read(p).view(np.uint32), heap.view(p, n * 4, n, np.float32).view(np.uint32)), p
+        for a in (psync, dst, src):
+            a.free()
+
+
 def test_paced_reduction_in_place_with_half_passes_at_the_edges():
     """dest == source at the default rate and the headline's launch shape: the workgroups on odd
     XCDs reduce the first half of their first pass first and its second half last, each byte
