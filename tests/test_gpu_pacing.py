@@ -66,6 +66,31 @@ def test_paced_reduction_with_other_numbers_of_pes(n_pes, wgs, wg_size, mib):
             a.free()
 
 
+def test_paced_reduction_of_arrays_that_start_off_a_vector_boundary():
+    """Source and destination three elements into their allocations: the elements in front of the
+    first 1 KiB boundary and behind the last whole vector go one by one, the rest is paced."""
+    n_pes, wgs, wg_size, shift = 8, 32, 512, 3
+    with runtime(n_pes, heap_size=256 << 20, num_blocks=wgs):
+        n = (40 << 20) // 4 + 5
+        src = rs.sym_array(n + 16, np.float32)
+        dst = rs.sym_array(n + 16, np.float32, fill=0x5A)
+        psync = rs.sym_array(wgs * rs.ROC_SHMEM_REDUCE_SYNC_SIZE, np.int64, fill=0)
+        heap = oracle.Heap(n_pes, 2 * (n + 16) * 4)
+        for p in range(n_pes):
+            vals = random_values(rs.FLOAT, n + 16, 110 + p)
+            src.write(p, vals)
+            heap.view(p, 0, n + 16, np.float32)[:] = vals
+            heap.view(p, (n + 16) * 4, n + 16, np.uint32)[:] = 0x5A5A5A5A
+        rs.roc_shmem_to_all(rs.FLOAT, rs.SUM, dst.addr + 4 * shift, src.addr + 4 * shift, n, 0, 0, n_pes, None, psync,
+                            rs.Launch(wgs, wg_size))
+        rs.synchronize()
+        oracle.to_all_rounded_once(heap, rs.FLOAT, rs.SUM, (n + 16 + shift) * 4, shift * 4, n)
+        for p in range(n_pes):     # the whole allocation: nothing in front of or behind the range is touched
+            assert np.array_equal(dst.read(p).view(np.uint32), heap.view(p, (n + 16) * 4, n + 16, np.uint32)), p
+        for a in (psync, dst, src):
+            a.free()
+
+
 def test_paced_reduction_in_place_with_half_passes_at_the_edges():
     """dest == source at the default rate and the headline's launch shape: the workgroups on odd
     XCDs reduce the first half of their first pass first and its second half last, each byte
