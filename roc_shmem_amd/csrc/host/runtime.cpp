@@ -254,7 +254,8 @@ std::string Runtime::init(const Options &opt) {
   RT_HIP(hipMemcpy(ctx_table_dev_, ctx_images_.data(), sizeof(detail::DeviceCtx) * rings,
                    hipMemcpyHostToDevice));
 
-  // status word (first 64 bytes) and, 256 bytes in, a scratch area for small kernel results
+  // status word (first 64 bytes), the count of workgroups inside large standard reductions (next
+  // 64 bytes) and, 256 bytes in, a scratch area for small kernel results
   RT_HIP(hipMalloc(reinterpret_cast<void **>(&status_dev_), 512));
   RT_HIP(hipMemset(status_dev_, 0, 512));
 
@@ -494,7 +495,8 @@ uint32_t Runtime::take_status() {
     // between the members that got through and those that did not.  Nothing is running
     // (the device was synchronised above), so put every library-owned pool back to zero.
     reset_sync_pools();
-    (void)hipMemset(status_dev_, 0, sizeof(v));
+    // (and the count of streaming workgroups, which calls that gave up may not have left)
+    (void)hipMemset(status_dev_, 0, 128);
   }
   return v;
 }

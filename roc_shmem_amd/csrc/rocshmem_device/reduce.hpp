@@ -171,7 +171,8 @@ template <typename T, ROC_SHMEM_OP Op, int U = kReduceUnroll, int C = kReducePeC
 __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_begin,
                                                size_t v_end, const ActiveSet &as, int my_pe,
                                                uint32_t tid, uint32_t nthr, size_t first_pass = 0,
-                                               size_t pass_step = 1, Pacer pacer = Pacer{0u, 0u}) {
+                                               size_t pass_step = 1, Pacer pacer = Pacer{0u, 0u},
+                                               uint32_t start_at = 0) {
   using Acc = typename AccOf<T, Op>::type;
   using V = VecOf<T>;
   constexpr int E = V::kElems;
@@ -192,41 +193,47 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
   const uint32_t pass_bytes = access_bytes * U;   // at most 128 KiB
   const size_t byte_end = v_end * 16;
 
-  // This workgroup takes passes first_pass, first_pass + pass_step, ... of the range.
+  // This workgroup takes passes first_pass, first_pass + pass_step, ... of the range: `mine` of
+  // them, visited in the order start_at, start_at + 1, ..., mine - 1, 0, ..., start_at - 1.
   const size_t step_bytes = pass_step * pass_bytes;
   const size_t byte_begin = v_begin * 16 + first_pass * pass_bytes;
+  if (byte_begin >= byte_end) return;
   // A short first pass is the only one, and a wave whose every lane lies past
   // its end has nothing to do in it.  Its accesses would be clipped, but a
   // clipped access still costs its issue slots: a 4 KiB reduction by one
   // workgroup of 1024 lanes took 10.4 us against 7.1 us by one of 256, now 8.0.
-  if (byte_begin < byte_end && byte_end - byte_begin < pass_bytes &&
-      uniform((tid & ~63u) * 16u) >= byte_end - byte_begin)
+  if (byte_end - byte_begin < pass_bytes && uniform((tid & ~63u) * 16u) >= byte_end - byte_begin)
     return;
+  const uint32_t mine = static_cast<uint32_t>((byte_end - byte_begin + step_bytes - 1) / step_bytes);
+  if (start_at >= mine) start_at %= mine;
   // A workgroup that fills the edges of the schedule (Pacer::fill_edges; it has two passes
   // or more, so its first one is whole) takes the first half of its first pass, then its
   // other passes, then the second half of the first: a half pass is the same code over a
   // window of half the size (the descriptor clips the other accesses), at half the slot.
-  const bool halves = pacer.period != 0 && pacer.fill_edges && byte_begin + step_bytes < byte_end;
+  const bool halves = pacer.period != 0 && pacer.fill_edges && mine > 1 &&
+                      byte_begin + start_at * step_bytes + pass_bytes <= byte_end;
   const uint32_t half_bytes = pass_bytes / 2;
   int edge = halves ? 0 : 1;   // 0: first half of the first pass, 1: whole passes, 2: its second half
-  size_t next_b = byte_begin;
+  uint32_t turn = 0;           // passes taken so far
   for (;;) {
     size_t b;
     int valid;
     uint32_t slot = pacer.period;
     if (edge == 1) {
-      if (next_b >= byte_end) {
+      if (turn >= mine) {
         if (!halves) break;
         edge = 2;
       } else {
-        b = next_b;
-        next_b += step_bytes;
+        uint32_t p = turn + start_at;
+        if (p >= mine) p -= mine;
+        ++turn;
+        b = byte_begin + p * step_bytes;
         const size_t left = byte_end - b;
         valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
       }
     }
     if (edge != 1) {
-      b = byte_begin + (edge == 0 ? 0u : half_bytes);
+      b = byte_begin + start_at * step_bytes + (edge == 0 ? 0u : half_bytes);
       valid = static_cast<int>(half_bytes);
       slot = pacer.period / 2;
     }
@@ -286,7 +293,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
     if (edge == 2) break;
     if (edge == 0) {
       edge = 1;
-      next_b = byte_begin + step_bytes;
+      turn = 1;
     }
   }
   // every wave has its own stores in memory before it meets the others
@@ -437,12 +444,7 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
   const size_t parts = static_cast<size_t>(pe_size) * nshards;
   const size_t part = static_cast<size_t>(shard) * pe_size + my_idx;
 
-  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, pe_stride, pe_size, psync_pe_step);
-
   constexpr size_t E = VecOf<T>::kElems;
-  // Whether this workgroup stores anything that is not written through (the
-  // element path's plain stores): decides how the closing barrier releases.
-  bool plain_stores = false;
   // The vector path stores 16-byte aligned and loads at any 4-byte alignment,
   // so it takes every pair of arrays that agree modulo 4 (all pairs of 4- and
   // 8-byte elements; 2-byte elements an even number of elements apart): the
@@ -455,77 +457,120 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
   const uintptr_t dest_at = reinterpret_cast<uintptr_t>(dest);
   const uintptr_t differ = dest_at ^ reinterpret_cast<uintptr_t>(source);
   const bool coaligned = (differ & 3u) == 0 && dest_at % sizeof(typename Storage<T>::elem) == 0;
+  size_t lead = 0, nvec = 0;
   if (coaligned) {
     const size_t bytes = n * sizeof(typename Storage<T>::elem);
     const uintptr_t boundary = bytes >= 65536 ? kStoreChunkBytes : bytes >= 4096 ? 128u : 16u;
-    size_t lead = ((boundary - (dest_at & (boundary - 1))) & (boundary - 1)) /
-                  sizeof(typename Storage<T>::elem);
+    lead = ((boundary - (dest_at & (boundary - 1))) & (boundary - 1)) / sizeof(typename Storage<T>::elem);
     if (lead > n) lead = n;
-    T *const all_dest = dest;
-    const T *const all_source = source;
-    dest += lead;
-    source += lead;
-    const size_t nvec = (n - lead) / E;
-    if (nshards == 1) {
-      // One workgroup per member: member k takes the k-th contiguous share.
+    nvec = (n - lead) / E;
+  }
+  const size_t full_pass_vecs = static_cast<size_t>(kReduceUnroll) * nthr;
+  // A stream: every workgroup of the call has two full passes or more.  Its passes are dealt
+  // round-robin over the call's workgroups, and it may follow the schedule (Pacer).
+  const bool stream = nvec >= 2 * parts * full_pass_vecs;
+  // A standard (unsharded) call knows its own members only, and the schedule is sized for all
+  // the workgroups that stream at the same time.  Such a call therefore counts itself in while
+  // it runs and follows the schedule only when (nearly) every workgroup of the grid is inside
+  // a call like it - a grid that tiles one large reduction over its workgroups; a lone large
+  // call in a grid that does other things runs free.
+  const bool counted = stream && nshards == 1 && g_state.pace_reduce_bytes_per_tick != 0 &&
+                       grid_is_resident();
+  if (counted && tid == 0)
+    __hip_atomic_fetch_add(streaming_workgroups(), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+  wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, pe_stride, pe_size, psync_pe_step);
+
+  // Whether this workgroup stores anything that is not written through (the
+  // element path's plain stores): decides how the closing barrier releases.
+  bool plain_stores = false;
+  if (coaligned) {
+    T *const vec_dest = dest + lead;
+    const T *const vec_source = source + lead;
+    // Vectors [v0, v1) in passes first_pass, first_pass + pass_step, ... of this workgroup.
+    size_t v0 = 0, v1 = nvec, first_pass = part, pass_step = parts;
+    bool short_passes = nvec < parts * full_pass_vecs;
+    Pacer pacer{0u, 0u, false};
+    uint32_t start_at = 0;
+    if (nshards == 1 && !stream) {
+      // One workgroup per member and less than two full passes each: member k takes the k-th
+      // contiguous share (dealing a single pass or two would leave members without work).
       const size_t share = (nvec + pe_size - 1) / pe_size;
-      size_t v0 = share * my_idx;
-      size_t v1 = v0 + share;
+      v0 = share * my_idx;
+      v1 = v0 + share;
       if (v0 > nvec) v0 = nvec;
       if (v1 > nvec) v1 = nvec;
-      if (v1 - v0 < static_cast<size_t>(kReduceUnroll) * nthr) {
-        // A share of less than one full pass costs the chain of load latencies:
-        // passes of two vectors per lane with four members' loads issued together
-        // (a 4096-element int64 reduction among 4 PEs: 9.1 -> 6.1 us per call).
-        reduce_vectors<T, Op, 2, 4>(dest, source, v0, v1, as, my_pe, tid, nthr);
-      } else {
-        reduce_vectors<T, Op>(dest, source, v0, v1, as, my_pe, tid, nthr);
+      first_pass = 0;
+      pass_step = 1;
+      short_passes = v1 - v0 < full_pass_vecs;
+    }
+    if (stream) {
+      // Passes are dealt round-robin over all workgroups of the call, so that the workgroups
+      // running at one moment sweep one compact window of every array.  Measured on MI355X
+      // (8 -> 8 fp32 reduction, no barriers): 6.06 TB/s against 5.86 TB/s when every
+      // workgroup walks a region of its own; giving each member a contiguous share and
+      // striding only within it was no better and less even across launch shapes.
+      // Paced (see Pacer) when the library holds a rate and the grid fills the chip (8 PEs,
+      // fp32, paced against free at the default rate: with two passes per workgroup +1 % at
+      // 32 x 1024 lanes per PE, +5 % at 32 x 512, +8 % at 64 x 512; with four +2 to +6 %;
+      // with eight +6 %).
+      const uint64_t pass_bytes = static_cast<uint64_t>(full_pass_vecs) * 16u;
+      const uint64_t wgs = grid_workgroups();
+      // A grid that tiles one large array over standard calls: each call deals its own tile,
+      // so the workgroups of different calls move through their tiles in step, and when every
+      // one of them starts at its tile's first passes, all windows in flight agree in the
+      // address bits that count passes within a tile and differ only in the bits that number
+      // the tiles; the memory system serves that badly (8 PEs, 32 x 1024 lanes per PE, one
+      // call per workgroup over a tile of 2^21 floats: 4600 GB/s, against 5800 when every
+      // member walks a contiguous share of the tile).  A call therefore starts its round-robin
+      // at the turn given by the address bits above one grid's worth of passes, which differ
+      // between the tiles that would otherwise collide: the windows in flight then differ in
+      // every address bit between a pass and a grid's worth of passes, as those of one sharded
+      // call do (6215 GB/s, the sharded form on the same card 6325).
+      // (32-bit arithmetic in KiB: the offset into the arena and a pass are multiples of it.)
+      if (nshards == 1 && nvec / full_pass_vecs < wgs) {
+        const uint64_t into_arena = reinterpret_cast<uintptr_t>(vec_dest) -
+                                    reinterpret_cast<uintptr_t>(g_state.heap_base0);
+        start_at = static_cast<uint32_t>(into_arena >> 10) / static_cast<uint32_t>(pass_bytes >> 10) /
+                   static_cast<uint32_t>(wgs);
       }
-    } else {
-      // Several workgroups per member: passes are dealt round-robin over all
-      // of them, so that the workgroups running at one moment sweep one
-      // compact window of every array.  Measured on MI355X (8 -> 8 fp32
-      // reduction, no barriers): 6.06 TB/s against 5.86 TB/s when every
-      // workgroup walks a region of its own; giving each member a contiguous
-      // share and striding only within it was no better and less even across
-      // launch shapes.
-      // With less than one full pass per workgroup, full passes would leave most
-      // workgroups idle while a few walk eight members' loads one after the other:
-      // short passes with four members' loads in flight spread the same vectors
-      // over four times as many workgroups (fp32 sum among 8 PEs: 1 MiB per PE
-      // with 16 workgroups of 512 lanes each 16.5 -> 13.0 us, 256 KiB with 4
-      // workgroups of 1024 lanes 21.9 -> 11.3 us).
-      if (nvec < parts * static_cast<size_t>(kReduceUnroll) * nthr) {
-        reduce_vectors<T, Op, 2, 4>(dest, source, 0, nvec, as, my_pe, tid, nthr, part, parts);
-      } else {
-        // Paced (see Pacer) when the library holds a rate, the grid fills the chip and
-        // every workgroup has at least two passes (8 PEs, fp32, paced against free at the
-        // default rate: with two passes +1 % at 32 x 1024 lanes per PE, +5 % at 32 x 512,
-        // +8 % at 64 x 512; with four +2 to +6 %; with eight +6 %).
-        const uint64_t pass_bytes = static_cast<uint64_t>(kReduceUnroll) * nthr * 16u;
-        Pacer pacer{0u, 0u};
-        if (g_state.pace_reduce_bytes_per_tick != 0 && nvec * 16u >= 2 * parts * pass_bytes &&
-            grid_is_resident())
+      if (nshards > 1) {
+        if (g_state.pace_reduce_bytes_per_tick != 0 && grid_is_resident())
           pacer = make_edge_filling_pacer(g_state.pace_reduce_bytes_per_tick,
                                           parts * pass_bytes * static_cast<uint64_t>(pe_size));
-        if (lds_stage != nullptr) {
-          // whole passes through LDS, two vectors per lane per member; what is left of the
-          // range goes the usual way, to whoever's turn it would have been
-          const size_t lds_pass_vecs = 2u * nthr;
-          const size_t whole = nvec / lds_pass_vecs;
-          reduce_vectors_lds<T, Op, 2>(dest, source, whole, as, my_pe, tid, nthr, part, parts, lds_stage,
-                                       uniform(lds_stage_bytes));
-          if (whole * lds_pass_vecs < nvec && whole % parts == part)
-            reduce_vectors<T, Op, 2, 1>(dest, source, whole * lds_pass_vecs, nvec, as, my_pe, tid, nthr);
-        } else {
-          reduce_vectors<T, Op>(dest, source, 0, nvec, as, my_pe, tid, nthr, part, parts, pacer);
-        }
+      } else if (counted) {
+        const uint32_t inside = uniform(__hip_atomic_load(streaming_workgroups(), __ATOMIC_RELAXED,
+                                                          __HIP_MEMORY_SCOPE_AGENT));
+        if (static_cast<uint64_t>(inside) * 4u >= wgs * 3u)
+          pacer = make_edge_filling_pacer(g_state.pace_reduce_bytes_per_tick,
+                                          wgs * pass_bytes * static_cast<uint64_t>(pe_size));
       }
     }
+    if (lds_stage != nullptr && stream && nshards > 1) {
+      // whole passes through LDS, two vectors per lane per member; what is left of the
+      // range goes the usual way, to whoever's turn it would have been
+      const size_t lds_pass_vecs = 2u * nthr;
+      const size_t whole = nvec / lds_pass_vecs;
+      reduce_vectors_lds<T, Op, 2>(vec_dest, vec_source, whole, as, my_pe, tid, nthr, part, parts, lds_stage,
+                                   uniform(lds_stage_bytes));
+      if (whole * lds_pass_vecs < nvec && whole % parts == part)
+        reduce_vectors<T, Op, 2, 1>(vec_dest, vec_source, whole * lds_pass_vecs, nvec, as, my_pe, tid, nthr);
+    } else if (short_passes) {
+      // Less than one full pass per workgroup costs the chain of load latencies, and full
+      // passes would leave most workgroups idle while a few walk eight members' loads one
+      // after the other: passes of two vectors per lane with four members' loads issued
+      // together (a 4096-element int64 reduction among 4 PEs: 9.1 -> 6.1 us per call; fp32
+      // sum among 8 PEs, 1 MiB per PE with 16 workgroups of 512 lanes each 16.5 -> 13.0 us,
+      // 256 KiB with 4 workgroups of 1024 lanes 21.9 -> 11.3 us).
+      reduce_vectors<T, Op, 2, 4>(vec_dest, vec_source, v0, v1, as, my_pe, tid, nthr, first_pass, pass_step);
+    } else {
+      reduce_vectors<T, Op>(vec_dest, vec_source, v0, v1, as, my_pe, tid, nthr, first_pass, pass_step, pacer,
+                            start_at);
+    }
     if (part == parts - 1) {
-      if (lead) reduce_elements<T, Op>(all_dest, all_source, 0, lead, as, my_pe, tid, nthr);
+      if (lead) reduce_elements<T, Op>(dest, source, 0, lead, as, my_pe, tid, nthr);
       if (lead + nvec * E < n)
-        reduce_elements<T, Op>(all_dest, all_source, lead + nvec * E, n, as, my_pe, tid, nthr);
+        reduce_elements<T, Op>(dest, source, lead + nvec * E, n, as, my_pe, tid, nthr);
       plain_stores = lead != 0 || lead + nvec * E < n;
     }
   } else {
@@ -540,6 +585,8 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
 
   wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size, psync_pe_step,
                   !plain_stores);
+  if (counted && tid == 0)
+    __hip_atomic_fetch_sub(streaming_workgroups(), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace detail

@@ -145,8 +145,9 @@ struct DeviceState {
 // units must agree on how they use shared memory (3: the barrier pool holds
 // call counts, not flags that are reset; 4: live queues, cq_consumer;
 // 5: arguments rebased into the caller's slice; 6: pacing; 7: paced bursts follow a
-// schedule of start times; 8: quiet and fence post on live queues).
-constexpr uint32_t kStateRevision = 8;
+// schedule of start times; 8: quiet and fence post on live queues; 9: word 16 of the status block
+// counts the workgroups inside large standard reductions).
+constexpr uint32_t kStateRevision = 9;
 constexpr uint32_t kStateLayout =
     (kStateRevision * 0x01000193u) ^
     static_cast<uint32_t>(sizeof(DeviceState) | (sizeof(DeviceCtx) << 8) | (sizeof(Team) << 16) |

@@ -40,6 +40,15 @@ __device__ __forceinline__ void status_raise(uint32_t code) {
                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// How many workgroups are inside a large standard (unsharded) reduction at this moment: a word
+// of its own cache line in the status block, counted up and down by those calls themselves
+// (wg_all_reduce), which is how a call that knows only its own members learns whether the
+// whole grid streams with it.
+constexpr int kStreamingWorkgroupsWord = 16;
+__device__ __forceinline__ uint32_t *streaming_workgroups() {
+  return g_state.status + kStreamingWorkgroupsWord;
+}
+
 // Translate a symmetric address of PE `from_pe` into the slice of PE `to_pe`.
 template <typename T>
 __device__ __forceinline__ T *translate(T *ptr, int from_pe, int to_pe) {

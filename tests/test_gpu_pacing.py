@@ -116,6 +116,41 @@ def test_paced_reduction_in_place_with_half_passes_at_the_edges():
         buf.free()
 
 
+@pytest.mark.parametrize("rate,wgs,wg_size,tiles_per_wg", [(68000, 32, 1024, 1), (40000, 32, 512, 1),
+                                                           (90000, 64, 512, 2), (68000, 32, 1024, 2)])
+def test_paced_standard_calls_tiled_over_the_grid_match_the_oracle(rate, wgs, wg_size, tiles_per_wg):
+    """The unchanged roc_shmem_ctx_<T>_<op>_wg_to_all, one call per tile, 256 or 512 workgroups in
+    the grid and two passes or more per member and call: every call deals its tile's passes to
+    its members, starts at the turn its address gives, counts itself among the streaming
+    workgroups and follows the schedule.  Bit-identical to the oracle whatever the rate, with a
+    ragged last tile, in place too."""
+    n_pes = 8
+    with runtime(n_pes, heap_size=1 << 30, num_blocks=64):
+        for dtype, op, in_place in ((rs.FLOAT, rs.SUM, False), (rs.LONG, rs.SUM, True), (rs.BF16, rs.MIN, False)):
+            npd = rs.NP_DTYPE[dtype]
+            es = np.dtype(npd).itemsize
+            tile = 3 * n_pes * wg_size * 128 // es          # three passes per member and call
+            n = tile * wgs * tiles_per_wg - tile // 2 + 5    # the last tile is half a tile and ragged
+            src = rs.sym_array(n, npd)
+            dst = src if in_place else rs.sym_array(n, npd, fill=0x5A)
+            psync = rs.sym_array(wgs * rs.ROC_SHMEM_REDUCE_SYNC_SIZE, np.int64, fill=0)
+            heap = oracle.Heap(n_pes, 2 * n * es)
+            for p in range(n_pes):
+                vals = random_values(dtype, n, 130 + p)
+                src.write(p, vals)
+                heap.view(p, 0, n, npd)[:] = vals
+            rs.set_pacing(0, rate)
+            rs.roc_shmem_to_all(dtype, op, dst, src, n, 0, 0, n_pes, None, psync, rs.Launch(wgs, wg_size, tile))
+            rs.synchronize()
+            rs.set_pacing(0, 0)
+            oracle.to_all_rounded_once(heap, dtype, op, 0 if in_place else n * es, 0, n)
+            for p in range(n_pes):
+                assert np.array_equal(dst.read(p), heap.view(p, 0 if in_place else n * es, n, npd)), (dtype, op, p)
+            assert rs.take_status() == 0
+            for a in ((psync, src) if in_place else (psync, dst, src)):
+                a.free()
+
+
 @pytest.mark.parametrize("rate", [40000, 66000, 90000])
 def test_paced_shared_put_and_get_are_exact(rate):
     n_pes, nbytes = 8, (40 << 20) + 4099        # 32 x 512 per PE: 20 passes per workgroup
