@@ -139,6 +139,38 @@ def record_traffic(fetch_csv, write_csv):
     print(json.dumps(out))
 
 
+def timeline_summary(path):
+    """Summary of the clock readings a timeline build of the library leaves in ROC_SHMEM_TIMELINE_FILE
+    (csrc/Makefile: EXTRA=-DROCSHMEM_TIMELINE; the readings of the last large reduction before the
+    runtime went): microseconds after the first wave entered the call, per mark, for the waves on
+    even and on odd XCDs - first wave, median, last wave - and the same for wave 0 and the last
+    wave of every workgroup."""
+    raw = np.fromfile(path, dtype=np.uint64).reshape(-1, 8)
+    rows = raw[raw[:, 0] != 0]
+    if not len(rows):
+        return {"waves": 0}
+    t0 = rows[:, 0].min()
+    us = (rows[:, :6].astype(np.int64) - np.int64(t0)) / 100.0      # 100 MHz clock
+    xcd = (rows[:, 6] & 15).astype(int)
+    wave_of_wg = np.nonzero(raw[:, 0] != 0)[0] % 16
+    names = ["entered", "entry_barrier_done", "first_burst_stored", "last_whole_pass_stored", "own_stores_landed",
+             "closing_barrier_done"]
+    out = {"waves": int(len(rows)), "period_ticks": int(rows[0, 6] >> 16),
+           "edge_filling_waves": int(((rows[:, 6] >> 8) & 1).sum())}
+    for label, sel in (("even_xcds", xcd % 2 == 0), ("odd_xcds", xcd % 2 == 1),
+                       ("first_wave_of_each_workgroup", wave_of_wg == 0),
+                       ("last_wave_of_each_workgroup", wave_of_wg == wave_of_wg.max())):
+        if not sel.any():
+            continue
+        out[label] = {n: [round(float(np.min(us[sel, i])), 1), round(float(np.median(us[sel, i])), 1),
+                          round(float(np.max(us[sel, i])), 1)] for i, n in enumerate(names)}
+    # how many waves are still streaming (own stores not landed) at 10 us steps before the end
+    end = us[:, 4].max()
+    out["waves_still_streaming_at_us_before_end"] = {str(d): int((us[:, 4] > end - d).sum()) for d in (5, 10, 20, 30, 40, 60, 80)}
+    out["per_xcd_last_store_landed_us"] = {str(x): round(float(us[xcd == x, 4].max()), 1) for x in sorted(set(xcd))}
+    return out
+
+
 def host_threads():
     """Threads for the CPU legs: the cores this process may run on, capped by the box's
     per-GPU share of host cores where the environment states one (OMP_NUM_THREADS)."""
@@ -165,7 +197,7 @@ def device_report():
 def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, cpu=False,
                  spread=False, launch_shape=None, tune=False, pace=None):
     """Returns a dict with ms_per_step, GB/s (algorithmic 2*P*N*s bytes) and optional CPU figures.
-    pace: None = the pacing rate the library holds (its default: reductions paced at 6.8 TB/s),
+    pace: None = the pacing rates the library holds (its defaults: 6.7 TB/s, 6.5 with short passes),
     0 = workgroups run free, another value = that rate in bytes per tick.
     tune: let the library measure, outside the timed region, which rate suits this reduction on
     this card, with the launch shapes of TUNE_SHAPES; the timed steps then run with the better
@@ -924,7 +956,13 @@ def main():
     ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="no GPU work: read the two rocprofv3 --pmc counter files of --counter-pair runs and "
                          "write the tracked traffic summary under profiles/")
+    ap.add_argument("--timeline", metavar="FILE",
+                    help="no GPU work: summarise the clock readings a timeline build of the library wrote "
+                         "(ROC_SHMEM_TIMELINE_FILE)")
     args = ap.parse_args()
+    if args.timeline:
+        print(json.dumps(timeline_summary(args.timeline)))
+        return
     if args.record_traffic:
         record_traffic(*args.record_traffic)
         return

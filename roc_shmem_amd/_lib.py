@@ -104,9 +104,11 @@ def load():
     global _lib
     if _lib is not None:
         return _lib
-    if not os.path.exists(LIB_PATH):
+    # ROC_SHMEM_LIBRARY names a variant build of the same sources (csrc/Makefile: EXTRA=, LIB=)
+    path = os.environ.get("ROC_SHMEM_LIBRARY") or LIB_PATH
+    if path == LIB_PATH and not os.path.exists(LIB_PATH):
         build()
-    lib = C.CDLL(LIB_PATH)
+    lib = C.CDLL(path)
     for name, (restype, argtypes) in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError if the symbol is missing
         fn.restype = restype

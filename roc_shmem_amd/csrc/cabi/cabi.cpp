@@ -98,6 +98,21 @@ bool active_set_in_range(int pe_start, int log_pe_stride, int pe_size, int num_p
   return last < num_pes;
 }
 
+bool device_idle(const char *who) {
+  rocshmem::host::Runtime *rt = rocshmem::host::Runtime::get();
+  if (rt && rt->persistent_kernel_running()) {
+    fail(std::string(who) + ": a live send-queue consumer is running (rsm_sq_consumer_stop first; "
+                            "rsm_stream_synchronize waits for one stream)");
+    return false;
+  }
+  const bool idle = rt ? rt->wait_for_device() : hipStreamSynchronize(nullptr) == hipSuccess;
+  if (!idle) {
+    fail(std::string(who) + ": waiting for the device failed: " + hipGetErrorString(hipGetLastError()));
+    return false;
+  }
+  return true;
+}
+
 int after_launch(const char *what) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(std::string(what) + ": " + hipGetErrorString(e));
@@ -183,7 +198,7 @@ void *rsm_malloc(size_t bytes) {
 int rsm_free(void *ptr) {
   RSM_ENTRY;
   RSM_NEED_RT(rt);
-  (void)hipDeviceSynchronize();
+  if (!rsm::device_idle("rsm_free")) return -1;
   return rt->sym_free(ptr) ? 0 : rsm::fail("rsm_free: not an outstanding symmetric allocation");
 }
 
@@ -249,7 +264,7 @@ int rsm_team_split_strided(uint64_t parent, int start, int stride, int size, uin
 int rsm_team_destroy(uint64_t team) {
   RSM_ENTRY;
   RSM_NEED_RT(rt);
-  (void)hipDeviceSynchronize();
+  if (!rsm::device_idle("rsm_team_destroy")) return -1;
   rt->team_destroy(reinterpret_cast<detail::Team *>(team));
   return 0;
 }
@@ -284,11 +299,7 @@ int rsm_fill(void *dst, int byte_value, size_t bytes) {
 }
 int rsm_synchronize(void) {
   RSM_ENTRY;
-  if (rsm::live_consumer_running())
-    return rsm::fail("rsm_synchronize: a live send-queue consumer is running; synchronise streams "
-                     "(rsm_stream_synchronize) until rsm_sq_consumer_stop");
-  RSM_HIP(hipDeviceSynchronize());
-  return 0;
+  return rsm::device_idle("rsm_synchronize") ? 0 : -1;
 }
 int rsm_stream_synchronize(void *stream) {
   RSM_ENTRY;
@@ -399,12 +410,9 @@ static bool sq_args_ok(Runtime *rt, int pe, int block) {
 int rsm_sq_reset(void) {
   RSM_ENTRY;
   RSM_NEED_RT(rt);
-  if (rsm::live_consumer_running())
-    return rsm::fail("rsm_sq_reset: a live send-queue consumer is running (rsm_sq_consumer_stop first)");
-  RSM_HIP(hipDeviceSynchronize());
+  if (!rsm::device_idle("rsm_sq_reset")) return -1;
   rt->reset_queues(nullptr);
-  RSM_HIP(hipDeviceSynchronize());
-  return 0;
+  return rsm::device_idle("rsm_sq_reset") ? 0 : -1;
 }
 
 int rsm_sq_read(int pe, int block, unsigned index, uint64_t out_words[8]) {
@@ -412,7 +420,7 @@ int rsm_sq_read(int pe, int block, unsigned index, uint64_t out_words[8]) {
   RSM_NEED_RT(rt);
   if (!sq_args_ok(rt, pe, block) || index >= rt->options().sq_size)
     return rsm::fail("rsm_sq_read: arguments out of range");
-  RSM_HIP(hipDeviceSynchronize());
+  if (!rsm::device_idle("rsm_sq_read")) return -1;
   RSM_HIP(hipMemcpy(out_words, rt->ctx_image(pe, block).ring.sq + 8ull * index, 64,
                     hipMemcpyDeviceToHost));
   return 0;
@@ -423,7 +431,7 @@ int rsm_sq_image(int pe, int block, void *host_out, size_t bytes) {
   RSM_NEED_RT(rt);
   if (!sq_args_ok(rt, pe, block) || bytes > 64ull * rt->options().sq_size)
     return rsm::fail("rsm_sq_image: arguments out of range");
-  RSM_HIP(hipDeviceSynchronize());
+  if (!rsm::device_idle("rsm_sq_image")) return -1;
   RSM_HIP(hipMemcpy(host_out, rt->ctx_image(pe, block).ring.sq, bytes, hipMemcpyDeviceToHost));
   return 0;
 }
@@ -433,7 +441,7 @@ int rsm_sq_state(int pe, int block, uint32_t *sq_counter, uint32_t *published,
   RSM_ENTRY;
   RSM_NEED_RT(rt);
   if (!sq_args_ok(rt, pe, block)) return rsm::fail("rsm_sq_state: arguments out of range");
-  RSM_HIP(hipDeviceSynchronize());
+  if (!rsm::device_idle("rsm_sq_state")) return -1;
   detail::SqCounters c;
   const detail::DeviceCtx &ctx = rt->ctx_image(pe, block);
   RSM_HIP(hipMemcpy(&c, ctx.counters, sizeof(c), hipMemcpyDeviceToHost));

@@ -53,10 +53,16 @@ long *noalloc_flags();
 // Stops a live send-queue consumer, if one is running, and releases its stream and control
 // block (drv_consume.hip); rsm_finalize calls it before the runtime is destroyed.
 void consumer_shutdown();
+void consumer_stop_for_teardown();   // the same stop, in the form the runtime's teardown calls
 // True between rsm_sq_consumer_start and rsm_sq_consumer_stop.  A device-wide synchronisation
 // would then wait for the consumer kernel, which runs until it is told to stop: entry points
 // that synchronise the device refuse to run meanwhile (use rsm_stream_synchronize).
 bool live_consumer_running();
+
+// Waits until the device is idle, for entry points that read or change what kernels use.  With
+// a live consumer running the wait would only end when the consumer gave up by itself (and the
+// queues would be left without one): the call is refused instead, false with the error set.
+bool device_idle(const char *who);
 
 // hipGetLastError() after a launch, folded into the error convention.
 int after_launch(const char *what);

@@ -58,6 +58,15 @@ bool ring_args_ok(Runtime *rt, int pe, int block) {
 namespace rsm {
 bool live_consumer_running() { return g_live.running; }
 
+// What the runtime calls when it is torn down with the consumer still up (a finalize through
+// the host interface, which knows nothing of this file).
+void consumer_stop_for_teardown() {
+  if (g_live.running) {
+    rsm_consume_totals_t ignored;
+    (void)rsm_sq_consumer_stop(&ignored);
+  }
+}
+
 // Called by rsm_finalize before the runtime goes away: a consumer that is still running is
 // told to stop and waited for, and what start allocated is released.
 void consumer_shutdown() {
@@ -84,8 +93,7 @@ int rsm_sq_consume(int pe, int block, void *target_arena, rsm_consume_totals_t *
   RSM_ENTRY;
   Runtime *rt = Runtime::get();
   if (!rt) return rsm::fail("rsm_init has not been called");
-  if (g_live.running)
-    return rsm::fail("rsm_sq_consume: a live consumer is running (rsm_sq_consumer_stop first)");
+  if (!rsm::device_idle("rsm_sq_consume")) return -1;
   if ((pe != -1 && (pe < 0 || pe >= rt->num_pes())) ||
       (block != -1 && (block < 0 || block >= rt->options().num_blocks)))
     return rsm::fail("rsm_sq_consume: pe / block out of range (-1 selects all)");
@@ -97,7 +105,7 @@ int rsm_sq_consume(int pe, int block, void *target_arena, rsm_consume_totals_t *
   hipLaunchKernelGGL(consume_kernel, dim3(rings), dim3(64), 0, nullptr, pe, block,
                      static_cast<char *>(target_arena), dev);
   CONSUME_HIP(hipGetLastError());
-  CONSUME_HIP(hipDeviceSynchronize());
+  if (!rsm::device_idle("rsm_sq_consume")) return -1;
   rsm_consume_totals_t host = {};
   CONSUME_HIP(hipMemcpy(&host, dev, sizeof(host), hipMemcpyDeviceToHost));
   if (totals) *totals = host;
@@ -115,12 +123,18 @@ int rsm_sq_consumer_start(void) {
     CONSUME_HIP(hipHostMalloc(reinterpret_cast<void **>(&g_live.control), sizeof(detail::LiveControl),
                               hipHostMallocDefault));
   // Everything launched so far has finished before the rings change hands.
-  CONSUME_HIP(hipDeviceSynchronize());
+  if (!rsm::device_idle("rsm_sq_consumer_start")) return -1;
   g_live.mode_before = rt->device_state().sq_queue_mode;
   g_live.pace_copy_before = rt->device_state().pace_copy_bytes_per_tick;
   g_live.pace_reduce_before = rt->device_state().pace_reduce_bytes_per_tick;
-  if (!rt->set_sq_mode(detail::kSqLive) || !rt->set_pacing(0, 0))
+  if (!rt->set_sq_mode(detail::kSqLive))
     return rsm::fail("rsm_sq_consumer_start: could not update the device state");
+  if (!rt->set_pacing(0, 0)) {
+    // live rings without a consumer would block their producers: back to the mode before
+    (void)rt->set_sq_mode(g_live.mode_before);
+    (void)rt->set_pacing(g_live.pace_copy_before, g_live.pace_reduce_before);
+    return rsm::fail("rsm_sq_consumer_start: could not update the device state");
+  }
   *g_live.control = detail::LiveControl{};
   detail::ConsumeTotals *totals = static_cast<detail::ConsumeTotals *>(rt->result_scratch());
   static_assert(sizeof(detail::ConsumeTotals) + sizeof(detail::LiveRelay) <= 256, "result scratch");
@@ -140,6 +154,7 @@ int rsm_sq_consumer_start(void) {
     return rsm::fail(std::string("rsm_sq_consumer_start: ") + hipGetErrorString(launched));
   }
   g_live.running = true;
+  rt->persistent_kernel_started(&rsm::consumer_stop_for_teardown);
   // Producers are launched only when every consumer wave is resident: a grid
   // that filled the device first would wait for a consumer that cannot start.
   const auto t0 = std::chrono::steady_clock::now();
@@ -163,6 +178,7 @@ int rsm_sq_consumer_stop(rsm_consume_totals_t *totals) {
   __atomic_store_n(&g_live.control->stop, 1u, __ATOMIC_RELEASE);
   hipError_t waited = hipStreamSynchronize(g_live.stream);
   g_live.running = false;
+  rt->persistent_kernel_stopped();
   const bool expired = __atomic_load_n(&g_live.control->expired, __ATOMIC_ACQUIRE) != 0;
   const bool mode_ok = rt->set_sq_mode(g_live.mode_before) &&
                        rt->set_pacing(g_live.pace_copy_before, g_live.pace_reduce_before);
@@ -189,7 +205,7 @@ int rsm_cq_reader_state(int pe, int block, uint32_t *cq_consumer, uint32_t *quie
   Runtime *rt = Runtime::get();
   if (!rt) return rsm::fail("rsm_init has not been called");
   if (!ring_args_ok(rt, pe, block)) return rsm::fail("rsm_cq_reader_state: arguments out of range");
-  CONSUME_HIP(hipDeviceSynchronize());
+  if (!rsm::device_idle("rsm_cq_reader_state")) return -1;
   detail::SqCounters c;
   const detail::DeviceCtx &ctx = rt->ctx_image(pe, block);
   CONSUME_HIP(hipMemcpy(&c, ctx.counters, sizeof(c), hipMemcpyDeviceToHost));
@@ -216,7 +232,7 @@ int rsm_sq_consumer_state(int pe, int block, uint32_t *consumed, uint32_t *cq_pr
   Runtime *rt = Runtime::get();
   if (!rt) return rsm::fail("rsm_init has not been called");
   if (!ring_args_ok(rt, pe, block)) return rsm::fail("rsm_sq_consumer_state: arguments out of range");
-  CONSUME_HIP(hipDeviceSynchronize());
+  if (!rsm::device_idle("rsm_sq_consumer_state")) return -1;
   detail::SqCounters c;
   CONSUME_HIP(hipMemcpy(&c, rt->ctx_image(pe, block).counters, sizeof(c), hipMemcpyDeviceToHost));
   if (consumed) *consumed = c.consumed;
@@ -230,7 +246,7 @@ int rsm_cq_image(int pe, int block, void *host_out, size_t bytes) {
   if (!rt) return rsm::fail("rsm_init has not been called");
   if (!ring_args_ok(rt, pe, block) || bytes > 64ull * rt->options().sq_size)
     return rsm::fail("rsm_cq_image: arguments out of range");
-  CONSUME_HIP(hipDeviceSynchronize());
+  if (!rsm::device_idle("rsm_cq_image")) return -1;
   CONSUME_HIP(hipMemcpy(host_out, rt->ctx_image(pe, block).ring.cq, bytes, hipMemcpyDeviceToHost));
   return 0;
 }
@@ -241,7 +257,7 @@ int rsm_atomic_ret_image(int pe, int block, void *host_out, size_t bytes) {
   if (!rt) return rsm::fail("rsm_init has not been called");
   if (!ring_args_ok(rt, pe, block) || bytes > 8ull * detail::kAtomicRetSlots)
     return rsm::fail("rsm_atomic_ret_image: arguments out of range");
-  CONSUME_HIP(hipDeviceSynchronize());
+  if (!rsm::device_idle("rsm_atomic_ret_image")) return -1;
   CONSUME_HIP(hipMemcpy(host_out,
                         reinterpret_cast<const void *>(rt->ctx_image(pe, block).ring.atomic_ret_base),
                         bytes, hipMemcpyDeviceToHost));

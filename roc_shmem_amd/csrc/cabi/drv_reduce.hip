@@ -365,9 +365,13 @@ int rsm_tune_reduce_pacing(int dtype, int op, void *dest, const void *source, si
   if (!launch) return rsm::fail("launch description is NULL");
   hipStream_t stream = static_cast<hipStream_t>(launch->stream);
   const unsigned copy_rate = rt->device_state().pace_copy_bytes_per_tick;
+  // what is in force now comes back on every path that does not end with a measured choice
+  const unsigned reduce_rate_before = rt->device_state().pace_reduce_bytes_per_tick;
   hipEvent_t t0 = nullptr, t1 = nullptr;
-  if (hipEventCreate(&t0) != hipSuccess || hipEventCreate(&t1) != hipSuccess)
+  if (hipEventCreate(&t0) != hipSuccess || hipEventCreate(&t1) != hipSuccess) {
+    if (t0) (void)hipEventDestroy(t0);
     return rsm::fail("rsm_tune_reduce_pacing: hipEventCreate failed");
+  }
   int rc = 0;
   // milliseconds per launch at `rate` (0 = free running): eight launches queued back to back
   // after a warm-up, the way a caller's loop issues them (launches timed one by one on an idle
@@ -412,7 +416,7 @@ int rsm_tune_reduce_pacing(int dtype, int op, void *dest, const void *source, si
       if (best_ms < free_ms * 0.99f) { chosen = best_rate; chosen_ms = best_ms; }
     }
   }
-  if (!rt->set_pacing(copy_rate, rc == 0 ? chosen : 0) && rc == 0) rc = -1;
+  if (!rt->set_pacing(copy_rate, rc == 0 ? chosen : reduce_rate_before) && rc == 0) rc = -1;
   (void)hipEventDestroy(t0);
   (void)hipEventDestroy(t1);
   if (rc != 0) {

@@ -172,8 +172,8 @@ int rsm_kat_fetch_incr(uint64_t lane_mask, int n_wgs, int wg_size, uint64_t *per
   hipLaunchKernelGGL(fetch_incr_kernel, dim3(n_wgs), dim3(wg_size), 0, nullptr, lane_mask, counter,
                      out);
   int rc = rsm::after_launch("kat_fetch_incr");
+  if (rc == 0 && !rsm::device_idle("kat_fetch_incr")) rc = -1;
   if (rc == 0) {
-    RSM_HIP(hipDeviceSynchronize());
     RSM_HIP(hipMemcpy(per_thread, out, n * 8, hipMemcpyDeviceToHost));
     RSM_HIP(hipMemcpy(counter_out, counter, 8, hipMemcpyDeviceToHost));
   }
@@ -203,8 +203,8 @@ int rsm_kat_coalesce(uint64_t lane_mask, const int32_t *pe, const uint64_t *src,
   hipLaunchKernelGGL(coalesce_kernel, dim3(1), dim3(64), 0, nullptr, lane_mask, d_pe, d_src, d_dst,
                      d_size, d_send, d_out);
   int rc = rsm::after_launch("kat_coalesce");
+  if (rc == 0 && !rsm::device_idle("kat_coalesce")) rc = -1;
   if (rc == 0) {
-    RSM_HIP(hipDeviceSynchronize());
     RSM_HIP(hipMemcpy(must_send, d_send, 64, hipMemcpyDeviceToHost));
     RSM_HIP(hipMemcpy(out_size, d_out, 64 * 8, hipMemcpyDeviceToHost));
   }

@@ -139,10 +139,13 @@ __host__ void roc_shmem_team_destroy(roc_shmem_team_t team) {
 }
 
 // Every PE is this process: the host-side barrier is "all device work has finished".
-__host__ void roc_shmem_barrier_all() {
-  runtime_or_die("roc_shmem_barrier_all");
-  (void)hipDeviceSynchronize();
+// (While a kernel runs that ends only when told to - the live send-queue consumer, started
+// through the C interface - the wait covers the default stream, on which this interface
+// launches; the whole device would not go idle.)
+static void wait_for_work(host::Runtime *rt) {
+  if (!rt->wait_for_device()) (void)hipStreamSynchronize(nullptr);
 }
+__host__ void roc_shmem_barrier_all() { wait_for_work(runtime_or_die("roc_shmem_barrier_all")); }
 __host__ void roc_shmem_sync_all() { roc_shmem_barrier_all(); }
 __host__ void roc_shmem_quiet() { roc_shmem_barrier_all(); }
 __host__ void roc_shmem_fence() {}
@@ -157,7 +160,7 @@ __host__ void debug_print_sq(int dest_pe, int src_wg, int index_wqe) {
   }
   uint64_t words[8];
   const detail::DeviceCtx &c = rt->ctx_image(dest_pe, src_wg);
-  (void)hipDeviceSynchronize();
+  wait_for_work(rt);
   (void)hipMemcpy(words, c.ring.sq + 8ull * index_wqe, sizeof(words), hipMemcpyDeviceToHost);
   printf("SQ pe %d block %d entry %d:", dest_pe, src_wg, index_wqe);
   for (int i = 0; i < 8; ++i) printf(" %016llx", static_cast<unsigned long long>(words[i]));
@@ -175,7 +178,7 @@ __host__ void debug_print_cq(int dest_pe, int src_wg, int cqe_num) {
   // Completion entries are written by the consumer pass (rsm_sq_consume).
   uint64_t words[8];
   const detail::DeviceCtx &c = rt->ctx_image(dest_pe, src_wg);
-  (void)hipDeviceSynchronize();
+  wait_for_work(rt);
   (void)hipMemcpy(words, c.ring.cq + 8ull * cqe_num, sizeof(words), hipMemcpyDeviceToHost);
   printf("CQ pe %d block %d entry %d:", dest_pe, src_wg, cqe_num);
   for (int i = 0; i < 8; ++i) printf(" %016llx", static_cast<unsigned long long>(words[i]));
@@ -265,7 +268,8 @@ rsm_launch_t collective_launch(host::Runtime *rt, size_t bytes, bool broadcast, 
 // rather than hand them back with a normal return (take_status also puts the barrier pools
 // back in order, which matters to a caller that catches the exit in a test harness only).
 void finish_collective(host::Runtime *rt, const char *what) {
-  check_hip(hipDeviceSynchronize(), what);
+  wait_for_work(rt);
+  check_hip(hipGetLastError(), what);
   const uint32_t status = rt->take_status();
   if (status != 0) {
     fprintf(stderr,
@@ -343,7 +347,7 @@ uint64_t amo(int kind, void *dest, uint64_t value, uint64_t cond, int pe, int wi
   void *remote = remote_of(rt, dest, pe, "roc_shmem_atomic");
   const uint64_t mask = width == 8 ? ~0ull : 0xffffffffull;
   uint64_t old = 0;
-  check_hip(hipDeviceSynchronize(), "roc_shmem_atomic");
+  wait_for_work(rt);
   check_hip(hipMemcpy(&old, remote, width, hipMemcpyDeviceToHost), "roc_shmem_atomic");
   uint64_t next = old;
   switch (kind) {

@@ -118,7 +118,8 @@ Options Options::from_env() {
   if (env_u64("ROC_SHMEM_REBASE_ARGS", &v)) o.rebase_args = v != 0;
   if (env_u64("ROC_SHMEM_REDUCE_LDS", &v)) o.reduce_lds = v != 0;
   if (env_u64("ROC_SHMEM_PACE_COPY", &v)) o.pace_copy = static_cast<uint32_t>(v);
-  if (env_u64("ROC_SHMEM_PACE_REDUCE", &v)) o.pace_reduce = static_cast<uint32_t>(v);
+  if (env_u64("ROC_SHMEM_PACE_REDUCE", &v)) o.pace_reduce = o.pace_reduce_short = static_cast<uint32_t>(v);
+  if (env_u64("ROC_SHMEM_PACE_REDUCE_SHORT", &v)) o.pace_reduce_short = static_cast<uint32_t>(v);
   return o;
 }
 
@@ -258,6 +259,15 @@ std::string Runtime::init(const Options &opt) {
   // 64 bytes) and, 256 bytes in, a scratch area for small kernel results
   RT_HIP(hipMalloc(reinterpret_cast<void **>(&status_dev_), 512));
   RT_HIP(hipMemset(status_dev_, 0, 512));
+  // A timeline build of the device code (-DROCSHMEM_TIMELINE) writes clock readings of every
+  // wave of a large reduction where the pointer at byte 128 of the status block points; the
+  // readings of the last launch are written to ROC_SHMEM_TIMELINE_FILE when the runtime goes.
+  if (getenv("ROC_SHMEM_TIMELINE_FILE")) {
+    RT_HIP(hipMalloc(reinterpret_cast<void **>(&timeline_dev_), detail::kTimelineBytes));
+    RT_HIP(hipMemset(timeline_dev_, 0, detail::kTimelineBytes));
+    RT_HIP(hipMemcpy(status_dev_ + detail::kTimelinePointerWord, &timeline_dev_, sizeof(timeline_dev_),
+                     hipMemcpyHostToDevice));
+  }
 
   RT_HIP(hipMalloc(reinterpret_cast<void **>(&teams_dev_), sizeof(detail::Team) * kMaxTeams));
   RT_HIP(hipMemset(teams_dev_, 0, sizeof(detail::Team) * kMaxTeams));
@@ -283,6 +293,7 @@ std::string Runtime::init(const Options &opt) {
   state_.sq_queue_mode = opt_.sq_queue_mode ? 1u : 0u;
   state_.pace_copy_bytes_per_tick = opt_.pace_copy;
   state_.pace_reduce_bytes_per_tick = opt_.pace_reduce;
+  state_.pace_reduce_short_bytes_per_tick = opt_.pace_reduce_short;
   {
     int dev = 0, cus = 0;
     RT_HIP(hipGetDevice(&dev));
@@ -292,7 +303,6 @@ std::string Runtime::init(const Options &opt) {
   }
   state_.rebase_args = opt_.rebase_args ? 1u : 0u;
   state_.arena_bytes = stride_ * static_cast<uint64_t>(P);
-  state_.stride_mask = (stride_ & (stride_ - 1)) == 0 ? stride_ - 1 : 0;
   reset_queues(nullptr);
   if (!state_layouts_agree())
     return "a translation unit of this program was compiled against other device headers than "
@@ -303,8 +313,34 @@ std::string Runtime::init(const Options &opt) {
   return "";
 }
 
+bool Runtime::wait_for_device() {
+  if (persistent_stop_) return false;
+  return hipDeviceSynchronize() == hipSuccess;
+}
+
+void Runtime::persistent_kernel_started(void (*stop)()) { persistent_stop_ = stop; }
+void Runtime::persistent_kernel_stopped() { persistent_stop_ = nullptr; }
+
 void Runtime::teardown() {
-  (void)hipDeviceSynchronize();
+  if (persistent_stop_) {
+    void (*stop)() = persistent_stop_;
+    stop();                       // unregisters itself (persistent_kernel_stopped)
+    persistent_stop_ = nullptr;
+  }
+  (void)wait_for_device();
+  if (timeline_dev_) {
+    if (const char *path = getenv("ROC_SHMEM_TIMELINE_FILE")) {
+      std::vector<char> host(detail::kTimelineBytes);
+      if (hipMemcpy(host.data(), timeline_dev_, host.size(), hipMemcpyDeviceToHost) == hipSuccess) {
+        if (FILE *f = fopen(path, "wb")) {
+          (void)fwrite(host.data(), 1, host.size(), f);
+          fclose(f);
+        }
+      }
+    }
+    (void)hipFree(timeline_dev_);
+    timeline_dev_ = nullptr;
+  }
   if (teams_dev_) (void)hipFree(teams_dev_);
   if (status_dev_) (void)hipFree(status_dev_);
   if (ctx_table_dev_) (void)hipFree(ctx_table_dev_);
@@ -349,7 +385,9 @@ void *Runtime::sym_malloc(size_t bytes) {
     off = alloc_.alloc(bytes);
   }
   if (off == Pow2Allocator::kNoOffset) return nullptr;
-  return slice_base(current_pe_) + off;
+  // The symmetric address of an object is its address in PE 0's slice, whichever PE the host
+  // thread stands for at the moment: it is what device calls take for "the caller's own copy".
+  return slice_base(0) + off;
 }
 
 bool Runtime::sym_free(void *ptr) {
@@ -446,14 +484,17 @@ bool Runtime::set_sq_queue_mode(bool queue) {
 }
 
 bool Runtime::set_pacing(uint32_t copy_bytes_per_tick, uint32_t reduce_bytes_per_tick) {
-  (void)hipDeviceSynchronize();
+  if (!wait_for_device()) return false;
   state_.pace_copy_bytes_per_tick = copy_bytes_per_tick;
   state_.pace_reduce_bytes_per_tick = reduce_bytes_per_tick;
+  // one rate named by the caller holds for every shape; naming the default brings both defaults back
+  state_.pace_reduce_short_bytes_per_tick =
+      reduce_bytes_per_tick == opt_.pace_reduce ? opt_.pace_reduce_short : reduce_bytes_per_tick;
   return upload_state_everywhere(state_);
 }
 
 bool Runtime::set_sq_mode(uint32_t mode) {
-  (void)hipDeviceSynchronize();
+  if (!wait_for_device()) return false;
   state_.sq_queue_mode = mode;
   return upload_state_everywhere(state_);
 }
@@ -487,9 +528,11 @@ long *Runtime::host_psync() {
 
 uint32_t Runtime::take_status() {
   uint32_t v = 0;
-  (void)hipDeviceSynchronize();
+  const bool idle = wait_for_device();
   (void)hipMemcpy(&v, status_dev_, sizeof(v), hipMemcpyDeviceToHost);
-  if (v) {
+  // (with a persistent kernel running the word is read and left as it is: the pools below may
+  // be in use)
+  if (v && idle) {
     // A wait that gave up leaves synchronisation state behind that later calls would trip
     // over: flags that were set and never consumed, and barrier call counts that differ
     // between the members that got through and those that did not.  Nothing is running
@@ -510,7 +553,7 @@ void Runtime::reset_sync_pools() {
     const size_t off = reinterpret_cast<char *>(host_psync_) - slice_base(0);
     for (int p = 0; p < opt_.num_pes; ++p) (void)hipMemset(slice_base(p) + off, 0, pool_bytes);
   }
-  (void)hipDeviceSynchronize();
+  (void)wait_for_device();
 }
 
 // ---------------------------------------------------------------------------

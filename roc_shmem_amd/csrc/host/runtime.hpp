@@ -64,14 +64,20 @@ struct Options {
   // ROC_SHMEM_REBASE_ARGS (default 1): device calls move symmetric-heap arguments into the
   // calling PE's slice, so a kernel may pass roc_shmem_malloc's pointer straight through.
   bool rebase_args = true;
-  // ROC_SHMEM_PACE_COPY / ROC_SHMEM_PACE_REDUCE: bytes per tick of the 100 MHz clock for the
-  // lockstep pacing of large sharded copies / reductions (device Pacer); 0 = off.  Reductions
-  // are paced by default, at 6.8 TB/s: a little above what MI355X cards sustain, which is where
-  // the schedule gains most (fp32 sum over 8 x 2^26, one card: 6046 GB/s free, 6190 at 62000,
-  // 6316 at 66000, 6374 at 68000, 6255 at 70000, 6196 at 90000).
+  // ROC_SHMEM_PACE_COPY / ROC_SHMEM_PACE_REDUCE / ROC_SHMEM_PACE_REDUCE_SHORT: bytes per tick
+  // of the 100 MHz clock for the lockstep pacing of large sharded copies / reductions (device
+  // Pacer); 0 = off.  Reductions are paced by default at the rate where the schedule gained
+  // most on the cards seen, one rate for passes of 128 KiB per member (workgroups of 1024
+  // lanes) and one for shorter passes (fp32 sum over 8 x 2^26, GB/s at 64000 / 65000 / 66000 /
+  // 67000 / 68000 / 70000 and running free; 32 x 1024 lanes per PE, two cards: 6272 6327 6404
+  // 6445 6375 6318 | 6017 and 6258 6338 6394 6423 6405 6356 | 6015; 32 x 512: 6262 6324 6226
+  // 6116 6023 5965 | 5845 and 6272 6302 6293 6023 5984 5970 | 5864).  A rate the caller sets
+  // (rsm_set_pacing, the tuner) holds for both kinds of pass; setting the default long rate
+  // again brings both defaults back.
   // Copies run free by default: their short passes gain nothing from the schedule.
   uint32_t pace_copy = 0;
-  uint32_t pace_reduce = 68000;
+  uint32_t pace_reduce = 67000;
+  uint32_t pace_reduce_short = 65000;
   // ROC_SHMEM_REDUCE_LDS=1: rsm_to_all runs float / long / bfloat16 sums through the LDS-staged
   // form of the sharded reduction (a measured alternative, slower on MI355X; default 0).
   bool reduce_lds = false;
@@ -101,7 +107,7 @@ class Runtime {
   int current_pe() const { return current_pe_; }
   void set_current_pe(int pe) { current_pe_ = pe; }
 
-  void *sym_malloc(size_t bytes);   // address in the current PE's slice, nullptr on failure
+  void *sym_malloc(size_t bytes);   // the object's symmetric address (in PE 0's slice), nullptr on failure
   bool sym_free(void *ptr);
   void *translate(const void *ptr, int pe) const;
   size_t bytes_in_use() const {
@@ -133,6 +139,16 @@ class Runtime {
   bool set_sq_mode(uint32_t mode);
   // Rates of the lockstep pacing (0 = off); false when the state could not be re-uploaded.
   bool set_pacing(uint32_t copy_bytes_per_tick, uint32_t reduce_bytes_per_tick);
+  // The one place the library waits for the whole device.  A kernel that runs until it is told
+  // to stop (the live send-queue consumer) makes such a wait last until that kernel gives up by
+  // itself and leaves the queues without a consumer, so whoever starts one registers it here
+  // with the routine that stops it: while it is registered, wait_for_device() returns false
+  // without waiting (callers refuse, or wait for their own streams), state changes that need an
+  // idle device (set_pacing, set_sq_mode) fail, and teardown stops the kernel first.
+  bool wait_for_device();
+  void persistent_kernel_started(void (*stop)());
+  void persistent_kernel_stopped();
+  bool persistent_kernel_running() const { return persistent_stop_ != nullptr; }
   bool sq_queue_mode() const { return state_.sq_queue_mode != 0; }
   const detail::DeviceState &device_state() const { return state_; }
   char *arena() const { return arena_; }
@@ -185,6 +201,8 @@ class Runtime {
   uint32_t *rkeys_dev_ = nullptr;
   char *flush_words_dev_ = nullptr;
   uint32_t *status_dev_ = nullptr;
+  void (*persistent_stop_)() = nullptr;   // stops the registered persistent kernel; null = none runs
+  uint64_t *timeline_dev_ = nullptr;   // ROC_SHMEM_TIMELINE_FILE: clock readings of a timeline build
   detail::Team *teams_dev_ = nullptr;   // kMaxTeams objects
   std::vector<int> free_team_slots_;
   std::map<const detail::Team *, TeamRecord> teams_;

@@ -191,6 +191,15 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
   const uint32_t lane_off = tid * 16u;
   const uint32_t access_bytes = nthr * 16u;       // bytes one instruction of the workgroup sweeps
   const uint32_t pass_bytes = access_bytes * U;   // at most 128 KiB
+  // The range and the deal are the same in every lane.  Saying so keeps the loop's bookkeeping
+  // in scalar registers: the callers derive them through 64-bit compares and divisions, which
+  // the compiler carries out on the vector unit, and whatever is computed from a vector value
+  // stays one (twenty vector registers and as many spills in the streaming kernels).
+  v_begin = uniform(v_begin);
+  v_end = uniform(v_end);
+  first_pass = uniform(first_pass);
+  pass_step = uniform(pass_step);
+  start_at = uniform(start_at);
   const size_t byte_end = v_end * 16;
 
   // This workgroup takes passes first_pass, first_pass + pass_step, ... of the range: `mine` of
@@ -204,8 +213,8 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
   // workgroup of 1024 lanes took 10.4 us against 7.1 us by one of 256, now 8.0.
   if (byte_end - byte_begin < pass_bytes && uniform((tid & ~63u) * 16u) >= byte_end - byte_begin)
     return;
-  const uint32_t mine = static_cast<uint32_t>((byte_end - byte_begin + step_bytes - 1) / step_bytes);
-  if (start_at >= mine) start_at %= mine;
+  const uint32_t mine = uniform(static_cast<uint32_t>((byte_end - byte_begin + step_bytes - 1) / step_bytes));
+  if (start_at >= mine) start_at = uniform(start_at % mine);
   // A workgroup that fills the edges of the schedule (Pacer::fill_edges; it has two passes
   // or more, so its first one is whole) takes the first half of its first pass, then its
   // other passes, then the second half of the first: a half pass is the same code over a
@@ -221,6 +230,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
     uint32_t slot = pacer.period;
     if (edge == 1) {
       if (turn >= mine) {
+        timeline_mark(3);   // stores of the last whole pass issued
         if (!halves) break;
         edge = 2;
       } else {
@@ -291,6 +301,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
         __builtin_amdgcn_raw_buffer_store_b128(out[u].raw, rd, lane_off, u * access_bytes, kStore);
     }
     if (edge == 2) break;
+    if (turn <= 1) timeline_mark(2);   // stores of the first burst issued
     if (edge == 0) {
       edge = 1;
       turn = 1;
@@ -298,6 +309,9 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
   }
   // every wave has its own stores in memory before it meets the others
   __builtin_amdgcn_s_waitcnt(0);
+  timeline_mark(4);
+  timeline_mark(6, (__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 15u) | (pacer.fill_edges ? 256u : 0u) |
+                       (static_cast<uint64_t>(pacer.period) << 16));
 }
 
 // The same reduction with the loads staged through LDS: every lane's 16-byte
@@ -479,7 +493,9 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
   if (counted && tid == 0)
     __hip_atomic_fetch_add(streaming_workgroups(), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
+  timeline_mark(0);
   wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, pe_stride, pe_size, psync_pe_step);
+  timeline_mark(1);
 
   // Whether this workgroup stores anything that is not written through (the
   // element path's plain stores): decides how the closing barrier releases.
@@ -534,16 +550,16 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
         start_at = static_cast<uint32_t>(into_arena >> 10) / static_cast<uint32_t>(pass_bytes >> 10) /
                    static_cast<uint32_t>(wgs);
       }
+      const uint32_t rate = pass_bytes >= (128u << 10) ? g_state.pace_reduce_bytes_per_tick
+                                                       : g_state.pace_reduce_short_bytes_per_tick;
       if (nshards > 1) {
-        if (g_state.pace_reduce_bytes_per_tick != 0 && grid_is_resident())
-          pacer = make_edge_filling_pacer(g_state.pace_reduce_bytes_per_tick,
-                                          parts * pass_bytes * static_cast<uint64_t>(pe_size));
+        if (rate != 0 && grid_is_resident())
+          pacer = make_edge_filling_pacer(rate, parts * pass_bytes * static_cast<uint64_t>(pe_size));
       } else if (counted) {
         const uint32_t inside = uniform(__hip_atomic_load(streaming_workgroups(), __ATOMIC_RELAXED,
                                                           __HIP_MEMORY_SCOPE_AGENT));
-        if (static_cast<uint64_t>(inside) * 4u >= wgs * 3u)
-          pacer = make_edge_filling_pacer(g_state.pace_reduce_bytes_per_tick,
-                                          wgs * pass_bytes * static_cast<uint64_t>(pe_size));
+        if (rate != 0 && static_cast<uint64_t>(inside) * 4u >= wgs * 3u)
+          pacer = make_edge_filling_pacer(rate, wgs * pass_bytes * static_cast<uint64_t>(pe_size));
       }
     }
     if (lds_stage != nullptr && stream && nshards > 1) {
@@ -585,6 +601,7 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
 
   wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size, psync_pe_step,
                   !plain_stores);
+  timeline_mark(5);
   if (counted && tid == 0)
     __hip_atomic_fetch_sub(streaming_workgroups(), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }

@@ -9,6 +9,7 @@
 #define ROCSHMEM_MI355X_DEVICE_STATE_HPP
 
 #include <hip/hip_runtime.h>
+#include <stddef.h>
 #include <stdint.h>
 
 namespace rocshmem {
@@ -82,10 +83,17 @@ struct alignas(64) SqCounters {
   uint32_t atomic_counter;  // free-running AMO return-slot index
   uint32_t consumed;        // every WQE below this index has been retired by the consumer pass
   uint32_t cq_producer;     // free-running count of completion entries written
+  uint32_t pad0_;
+  // The reader's pair, one naturally aligned 64-bit word (quiet_counter in the upper half) that
+  // posts and quiets change with single 64-bit atomics, so that concurrent quiets on one queue
+  // always see a consistent (taken, still requested) pair:
   uint32_t cq_consumer;     // completion entries a reader (quiet) has taken (reference: cq_consumer_counter)
   uint32_t quiet_counter;   // completions requested from a live consumer and not yet taken by quiet
-  uint32_t pad_[9];
+  uint32_t pad_[8];
 };
+static_assert(offsetof(SqCounters, cq_consumer) % 8 == 0 &&
+                  offsetof(SqCounters, quiet_counter) == offsetof(SqCounters, cq_consumer) + 4,
+              "cq_consumer and quiet_counter form one aligned 64-bit word");
 
 // One context = one (PE, block) pair (reference: GPUIBContext members,
 // context_ib_device.hpp:278-299, minus all NIC state).
@@ -121,12 +129,15 @@ struct DeviceState {
   // of every PE); 0: arguments are used as given.
   uint32_t rebase_args;
   uint64_t arena_bytes;        // num_pes * slice_stride
-  uint64_t stride_mask;        // slice_stride - 1 when the stride is a power of two, else 0
   // Lockstep pacing of large streaming copies / reductions (see Pacer in copy.hpp): bytes of
   // traffic the memory system takes per tick of the 100 MHz clock when all workgroups issue in
   // step; 0 = workgroups run free.
   uint32_t pace_copy_bytes_per_tick;
   uint32_t pace_reduce_bytes_per_tick;
+  // The rate for reductions whose passes are shorter than 128 KiB per member (workgroups of
+  // fewer than 1024 lanes): they sustain a little less, and a schedule ahead of what the card
+  // sustains costs them more (32 x 512 lanes per PE: 6324 GB/s at 65000, 6023 at 68000).
+  uint32_t pace_reduce_short_bytes_per_tick;
   // Grids that are paced: at most pace_max_grid_lanes lanes (compute units x 1024, what is
   // resident together of the streaming kernels, which need 65-128 vector registers: the slots
   // are sized for all workgroups of the grid running at once) and at least
@@ -135,6 +146,14 @@ struct DeviceState {
   uint32_t pace_max_grid_lanes;
   uint32_t pace_min_grid_workgroups;
 };
+
+// Timeline builds (-DROCSHMEM_TIMELINE): words 32-33 of the status block hold the device
+// address of kTimelineBytes of clock readings, kTimelineMarks 64-bit readings for each of the
+// first kTimelineWaves waves of a grid (wave = workgroup * 16 + wave of the workgroup), or 0.
+constexpr int kTimelinePointerWord = 32;
+constexpr int kTimelineMarks = 8;
+constexpr int kTimelineWaves = 2048 * 16;
+constexpr size_t kTimelineBytes = static_cast<size_t>(kTimelineWaves) * kTimelineMarks * 8;
 
 // Fingerprint of the structures device code and the host library share.  Device
 // code is compiled into every user program (the interface is header-only); a
@@ -146,7 +165,8 @@ struct DeviceState {
 // call counts, not flags that are reset; 4: live queues, cq_consumer;
 // 5: arguments rebased into the caller's slice; 6: pacing; 7: paced bursts follow a
 // schedule of start times; 8: quiet and fence post on live queues; 9: word 16 of the status block
-// counts the workgroups inside large standard reductions).
+// counts the workgroups inside large standard reductions, the completion reader's counters are
+// one 64-bit word).
 constexpr uint32_t kStateRevision = 9;
 constexpr uint32_t kStateLayout =
     (kStateRevision * 0x01000193u) ^

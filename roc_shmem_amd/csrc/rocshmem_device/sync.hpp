@@ -49,6 +49,19 @@ __device__ __forceinline__ uint32_t *streaming_workgroups() {
   return g_state.status + kStreamingWorkgroupsWord;
 }
 
+// Clock reading number `mark` of the calling wave, in builds with -DROCSHMEM_TIMELINE (and when
+// the host has put a buffer in place: ROC_SHMEM_TIMELINE_FILE); nothing otherwise.
+#ifdef ROCSHMEM_TIMELINE
+__device__ __forceinline__ void timeline_mark(int mark, uint64_t value = ~0ull) {
+  uint64_t *buf = *reinterpret_cast<uint64_t *const *>(g_state.status + kTimelinePointerWord);
+  const uint32_t wave = blockIdx.x * 16u + flat_thread_id() / 64u;
+  if (buf && wave < static_cast<uint32_t>(kTimelineWaves) && lane_id() == 0)
+    buf[wave * kTimelineMarks + mark] = value == ~0ull ? wall_clock64() : value;
+}
+#else
+__device__ __forceinline__ void timeline_mark(int, uint64_t = 0) {}
+#endif
+
 // Translate a symmetric address of PE `from_pe` into the slice of PE `to_pe`.
 template <typename T>
 __device__ __forceinline__ T *translate(T *ptr, int from_pe, int to_pe) {
@@ -58,24 +71,26 @@ __device__ __forceinline__ T *translate(T *ptr, int from_pe, int to_pe) {
       reinterpret_cast<uintptr_t>(ptr) + static_cast<uintptr_t>(delta));
 }
 
-// The calling PE's address of the symmetric object that `ptr` names in any
-// PE's slice; pointers outside the symmetric heap (and every pointer when
-// DeviceState::rebase_args is off) come back unchanged.  All PEs live in one
-// process, so a kernel argument holds one value for the workgroups of every
-// PE - the address roc_shmem_malloc returned, which lies in one PE's slice.
-// The roc_shmem_* calls pass their symmetric and local buffer arguments through
-// this, which lets a kernel written for the reference (one process per PE,
-// every process passing its own address: reduction_tester.cpp:74-104,
-// primitive_tester.cpp:32-82) run unchanged.  An address inside the caller's
-// own slice maps to itself.
+// The calling PE's own copy of the symmetric object that `ptr` names by its symmetric address;
+// every other pointer (and every pointer when DeviceState::rebase_args is off) comes back
+// unchanged.  All PEs live in one process, so a kernel argument holds one value for the
+// workgroups of every PE: the address roc_shmem_malloc returned, which is the object's
+// address in PE 0's slice - that address is what stands for "my copy" in a call.  The
+// roc_shmem_* calls pass their symmetric and local buffer arguments through this, which lets a
+// kernel written for the reference (one process per PE, every process passing its own address:
+// reduction_tester.cpp:74-104, primitive_tester.cpp:32-82) run unchanged.  A pointer into
+// another PE's slice - what roc_shmem_ptr returns, say, handed on as the local side of a put or
+// a get or as the word to wait on - is an address like any other and is used as it is, as the
+// reference uses it (context_ib_device.cpp:128-137).  One case cannot be told apart: PE 0's
+// copy, named on purpose by a workgroup of another PE, has the symmetric address itself and is
+// taken for the caller's own copy (roc_shmemx_my_addr and roc_shmem_ptr give explicit control).
 template <typename T>
 __device__ __forceinline__ T *own(T *ptr, int my_pe) {
   const uint64_t rel =
       reinterpret_cast<uint64_t>(ptr) - reinterpret_cast<uint64_t>(g_state.heap_base0);
-  if (!g_state.rebase_args || rel >= g_state.arena_bytes) return ptr;   // below the arena: rel wraps
-  const uint64_t off = g_state.stride_mask ? (rel & g_state.stride_mask) : rel % g_state.slice_stride;
+  if (!g_state.rebase_args || rel >= g_state.slice_stride) return ptr;   // below the arena: rel wraps
   return reinterpret_cast<T *>(const_cast<char *>(g_state.heap_base0) +
-                               static_cast<uint64_t>(my_pe) * g_state.slice_stride + off);
+                               static_cast<uint64_t>(my_pe) * g_state.slice_stride + rel);
 }
 template <typename T>
 __device__ __forceinline__ T *own(T *ptr, const DeviceCtx *c) {

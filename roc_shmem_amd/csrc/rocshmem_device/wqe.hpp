@@ -82,6 +82,11 @@ struct WqeRequest {
   WqeForm form = kWqeData;
 };
 
+// The completion reader's two counters as the one 64-bit word they share (SqCounters).
+__device__ __forceinline__ unsigned long long *reader_word(SqCounters *cnt) {
+  return reinterpret_cast<unsigned long long *>(&cnt->cq_consumer);
+}
+
 // Post one entry per lane that passes `sends == true`.  Called by every lane
 // that is active at the call site (senders and absorbed lanes alike).
 template <int kRingPolicy>
@@ -232,7 +237,8 @@ __device__ __forceinline__ void wave_post_with(DeviceCtx *ctx, bool sends, const
     // quiet_counter (queue_pair.cpp:80-101): completions asked of a live
     // consumer that roc_shmem_ctx_quiet has yet to collect.
     if (g_state.sq_queue_mode == kSqLive)
-      __hip_atomic_fetch_add(&cnt->quiet_counter, n_cqe, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_fetch_add(reader_word(cnt), static_cast<unsigned long long>(n_cqe) << 32, __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
     bounded_wait<uint32_t>(&cnt->published, kWaitEq, base);
     __hip_atomic_store(reinterpret_cast<unsigned long long *>(&ring.mailbox[0]),
                        static_cast<unsigned long long>(be32(base + n)), __ATOMIC_RELAXED,
@@ -246,48 +252,65 @@ __device__ __forceinline__ void wave_post_with(DeviceCtx *ctx, bool sends, const
 }
 
 // quiet on a queue with a live consumer (reference: QueuePair::quiet_internal,
-// queue_pair.cpp:118-191).  Completions arrive in order, so the reader claims
-// every completion requested so far (quiet_counter), polls only the entry of
-// the last one until the consumer has written it - valid when its owner bit
-// equals the lap parity of its running number and its opcode is not "invalid" -
-// then moves the completion queue's consumer index and its doorbell record
-// (mailbox word 2).  The wait is bounded like every other.
+// queue_pair.cpp:118-191).  Completions arrive in order, so the reader looks at what has been
+// requested and not yet taken (quiet_counter), polls only the entry of the last of them until
+// the consumer has written it - valid when its owner bit equals the lap parity of its running
+// number and its opcode is not "invalid" - and only then takes them: it moves the completion
+// queue's consumer index, lowers quiet_counter by what it took and writes the completion
+// queue's doorbell record (mailbox word 2).  As in the reference the counters change after the
+// poll, so several waves may quiet one queue at the same time and each returns only when every
+// completion that was requested before it looked has been written: one that finds nothing
+// requested can rely on whoever took the completions having seen them first.  Both counters
+// sit in one 64-bit word (reader_word) that is changed by compare-and-swap; a wave whose swap
+// fails (another reader took completions, or more were requested meanwhile) looks again.  The
+// wait is bounded like every other.
 __device__ __forceinline__ void quiet_live(DeviceCtx *ctx) {
   SqCounters *cnt = ctx->counters;
   const SqRing &ring = ctx->ring;
-  const uint32_t quiet_val =
-      __hip_atomic_exchange(&cnt->quiet_counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if (quiet_val == 0) return;
-  const uint32_t number = __hip_atomic_fetch_add(&cnt->cq_consumer, quiet_val, __ATOMIC_RELAXED,
-                                                 __HIP_MEMORY_SCOPE_AGENT) +
-                          quiet_val - 1;
-  // last 8 bytes of the completion entry: ... | BE32 qpn | BE16 wqe index | signature | op_own
-  const unsigned long long *tail = reinterpret_cast<const unsigned long long *>(
-      ring.cq + 8ull * (number & (ring.cq_size - 1)) + 7);
-  const uint32_t parity = (number >> ring.cq_log_size) & 1u;
   uint64_t start = wall_clock64();
   uint32_t spins = 0;
   for (;;) {
-    const unsigned long long word =
-        __hip_atomic_load(tail, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const uint32_t op_own = static_cast<uint32_t>(word >> 56);
-    if ((op_own & 1u) == parity && (op_own >> 4) != 0xFu) {
-      // a requester completion of this queue (opcode 0, the queue's number)
-      if ((op_own >> 4) != 0u ||
-          static_cast<uint32_t>(word) != ((ring.ctrl_qp_sq & 0xffffffu) << 8))
-        status_raise(kStatusBadCompletion);
-      break;
+    unsigned long long seen = __hip_atomic_load(reader_word(cnt), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t requested = static_cast<uint32_t>(seen >> 32);
+    const uint32_t taken = static_cast<uint32_t>(seen);
+    if (requested == 0) return;
+    const uint32_t number = taken + requested - 1;
+    // last 8 bytes of the completion entry: ... | BE32 qpn | BE16 wqe index | signature | op_own
+    const unsigned long long *tail = reinterpret_cast<const unsigned long long *>(
+        ring.cq + 8ull * (number & (ring.cq_size - 1)) + 7);
+    const uint32_t parity = (number >> ring.cq_log_size) & 1u;
+    bool gave_up = false;
+    for (;;) {
+      const unsigned long long word =
+          __hip_atomic_load(tail, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const uint32_t op_own = static_cast<uint32_t>(word >> 56);
+      if ((op_own & 1u) == parity && (op_own >> 4) != 0xFu) {
+        // a requester completion of this queue (opcode 0, the queue's number)
+        if ((op_own >> 4) != 0u ||
+            static_cast<uint32_t>(word) != ((ring.ctrl_qp_sq & 0xffffffu) << 8))
+          status_raise(kStatusBadCompletion);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+      if ((++spins & 63u) == 0 &&
+          (status_failed() || wall_clock64() - start > g_state.wait_limit_ticks)) {
+        status_raise(kStatusWaitTimeout);
+        gave_up = true;
+        break;
+      }
     }
-    __builtin_amdgcn_s_sleep(1);
-    if ((++spins & 63u) == 0 &&
-        (status_failed() || wall_clock64() - start > g_state.wait_limit_ticks)) {
-      status_raise(kStatusWaitTimeout);
-      break;
+    // (requested, taken) -> (requested - what this reader saw, taken + the same); a reader
+    // that gave up takes them all the same, so that the counters stay in step with the entries
+    const unsigned long long next = static_cast<unsigned long long>(taken + requested);
+    if (__hip_atomic_compare_exchange_strong(reader_word(cnt), &seen, next, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT)) {
+      __hip_atomic_store(reinterpret_cast<unsigned long long *>(&ring.mailbox[2]),
+                         static_cast<unsigned long long>(be32(number + 1)), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+      return;
     }
+    if (gave_up) return;
   }
-  __hip_atomic_store(reinterpret_cast<unsigned long long *>(&ring.mailbox[2]),
-                     static_cast<unsigned long long>(be32(number + 1)), __ATOMIC_RELAXED,
-                     __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ void wave_post(DeviceCtx *ctx, bool sends, const WqeRequest &rq);

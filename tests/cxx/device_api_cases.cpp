@@ -258,6 +258,85 @@ static void shmem_ptr() {
   roc_shmem_free(r_buf);
 }
 
+// ---- a roc_shmem_ptr result handed on as the local side of a call ------------------------------
+// The reference hands back a plain address (context_ib_device.cpp:128-137) that a program may use
+// like any other local address.  PE `me` copies from PE me+1's copy of `a` into PE me+2's copy of
+// `b` (a put whose source is another PE's memory), fetches PE me+1's `a` into its own `c` through a
+// get whose destination is its own roc_shmem_ptr address, and waits on a word of PE me+1 that PE
+// me+1 sets itself.  Only pointers that name PE 0's copy from elsewhere cannot be told from the
+// symmetric address, so PE 0's copies are named through roc_shmemx_my_addr by PE 0 alone here.
+__global__ void ShmemPtrAsArgumentTest(long *a, long *b, long *c, long *flag, int n, int *errors) {
+  __shared__ roc_shmem_ctx_t ctx;
+  roc_shmem_wg_init();
+  roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
+  const int me = roc_shmem_ctx_my_pe(ctx);
+  const int np = roc_shmem_ctx_n_pes(ctx);
+  const int next = (me + 1) % np, after = (me + 2) % np;
+  // a source in PE next's slice (never PE 0's: see above)
+  if (next != 0) {
+    long *theirs = static_cast<long *>(roc_shmem_ptr(a, next));
+    roc_shmemx_ctx_putmem_wg(ctx, b, theirs, n * sizeof(long), after);
+  } else {
+    roc_shmemx_ctx_putmem_wg(ctx, b, a, n * sizeof(long), after);   // keeps the pattern whole: own a
+  }
+  // a destination given as the caller's own roc_shmem_ptr address
+  long *mine_c = static_cast<long *>(roc_shmem_ptr(c, me));
+  roc_shmemx_ctx_getmem_wg(ctx, mine_c, a, n * sizeof(long), next);
+  if (threadIdx.x == 0) {
+    roc_shmem_ctx_quiet(ctx);
+    // every PE raises its own flag; its left neighbour waits on it through a plain address
+    roc_shmem_ctx_long_p(ctx, flag, 7 + me, me);
+    if (next != 0) {
+      long *their_flag = static_cast<long *>(roc_shmem_ptr(flag, next));
+      roc_shmem_long_wait_until(their_flag, ROC_SHMEM_CMP_EQ, 7 + next);
+      if (roc_shmem_long_test(their_flag, ROC_SHMEM_CMP_NE, 7 + next)) atomicAdd(errors, 1);
+    }
+  }
+  roc_shmem_wg_ctx_destroy(ctx);
+  roc_shmem_wg_finalize();
+}
+
+static void shmem_ptr_as_argument() {
+  current_case = "roc_shmem_ptr results as local arguments";
+  const int n = 512;
+  long *a = static_cast<long *>(roc_shmem_malloc(n * sizeof(long)));
+  long *b = static_cast<long *>(roc_shmem_malloc(n * sizeof(long)));
+  long *c = static_cast<long *>(roc_shmem_malloc(n * sizeof(long)));
+  long *flag = static_cast<long *>(roc_shmem_malloc(sizeof(long)));
+  int *errors = nullptr;
+  (void)hipMalloc(reinterpret_cast<void **>(&errors), sizeof(int));
+  (void)hipMemset(errors, 0, sizeof(int));
+  for (int pe = 0; pe < npes; ++pe) {
+    std::vector<long> v(n);
+    for (int i = 0; i < n; ++i) v[i] = 1000L * pe + i;
+    roc_shmem_putmem(a, v.data(), n * sizeof(long), pe);
+    fill(b, n, -1L, pe);
+    fill(c, n, -2L, pe);
+    fill(flag, 1, 0L, pe);
+  }
+  ShmemPtrAsArgumentTest<<<npes, 256>>>(a, b, c, flag, n, errors);
+  finish_kernel("ShmemPtrAsArgumentTest");
+  int bad = 0;
+  (void)hipMemcpy(&bad, errors, sizeof(int), hipMemcpyDeviceToHost);
+  EXPECT(bad == 0, "test() on another PE's word, named by a plain address, saw a stale value");
+  for (int pe = 0; pe < npes; ++pe) {
+    // b of PE pe was written by PE pe-2 with the a of PE pe-1 (or with its own a when pe-1 is PE 0)
+    const int writer = (pe - 2 + 2 * npes) % npes, from = (writer + 1) % npes;
+    const int expect_a_of = from != 0 ? from : writer;
+    std::vector<long> got_b = load(b, n, pe), got_c = load(c, n, pe);
+    for (int i = 0; i < n; ++i) {
+      EXPECT(got_b[i] == 1000L * expect_a_of + i, "b of PE %d [%d] = %ld, expected a of PE %d", pe, i, got_b[i],
+             expect_a_of);
+      EXPECT(got_c[i] == 1000L * ((pe + 1) % npes) + i, "c of PE %d [%d] = %ld", pe, i, got_c[i]);
+    }
+  }
+  (void)hipFree(errors);
+  roc_shmem_free(flag);
+  roc_shmem_free(c);
+  roc_shmem_free(b);
+  roc_shmem_free(a);
+}
+
 // ---- team_ctx_infra_tester.cpp:41-90 ---------------------------------------------------------------
 #define NUM_TEAMS 39  // ROC_SHMEM_MAX_NUM_TEAMS - 1
 __global__ void TeamCtxInfraTest(roc_shmem_team_t *team, int *errors) {
@@ -1428,7 +1507,8 @@ int main() {
     void (*run)();
   } cases[] = {{"ping_pong", ping_pong},       {"compare_ops", compare_ops},
                {"narrow_ping_pong", narrow_ping_pong},
-               {"shmem_ptr", shmem_ptr},       {"team_ctx_infra", team_ctx_infra},
+               {"shmem_ptr", shmem_ptr},       {"shmem_ptr_as_argument", shmem_ptr_as_argument},
+               {"team_ctx_infra", team_ctx_infra},
                {"team_ctx_primitive", team_ctx_primitive}, {"sync_and_barrier", sync_and_barrier},
                {"strided_team", strided_team},
                {"swarm", swarm},               {"amo_testers", amo_testers},

@@ -117,3 +117,28 @@ def test_active_set_range_check_is_done_in_64_bits():
                 for size in (1, 2, 3, 4, 8, 16, 127, 128):
                     want = int(start < num_pes and start + (size - 1) * (1 << log) < num_pes)
                     assert ok(start, log, size, num_pes) == want, (start, log, size, num_pes)
+
+
+def test_only_the_runtime_waits_for_the_whole_device():
+    # A wait for the whole device while the live send-queue consumer runs lasts until the
+    # consumer gives up by itself and leaves the queues without one.  Every such wait therefore
+    # goes through Runtime::wait_for_device, which refuses while a persistent kernel is
+    # registered: no other host source may call hipDeviceSynchronize itself.
+    import glob
+    import re
+    csrc = os.path.join(ROOT, "roc_shmem_amd", "csrc")
+    offenders = []
+    for path in sorted(glob.glob(os.path.join(csrc, "**", "*.*"), recursive=True)):
+        if os.sep + "build" + os.sep in path or not path.endswith((".cpp", ".hip", ".hpp")):
+            continue
+        text = open(path).read()
+        for m in re.finditer(r"hipDeviceSynchronize\s*\(", text):
+            line = text.count("\n", 0, m.start()) + 1
+            if not path.endswith(os.path.join("host", "runtime.cpp")):
+                offenders.append("%s:%d" % (os.path.relpath(path, ROOT), line))
+    assert not offenders, offenders
+    runtime = open(os.path.join(csrc, "host", "runtime.cpp")).read()
+    # in the runtime: once at the end of init (nothing persistent can run yet) and in wait_for_device
+    assert len(re.findall(r"hipDeviceSynchronize\s*\(", runtime)) == 2
+    body = runtime[runtime.index("bool Runtime::wait_for_device()"):]
+    assert "if (persistent_stop_) return false;" in body[:body.index("}")]

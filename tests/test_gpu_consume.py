@@ -374,6 +374,56 @@ def test_finalize_with_a_running_consumer_stops_it():
         rs.roc_shmem_finalize()
 
 
+def test_calls_that_wait_for_the_whole_device_are_refused_while_a_consumer_runs():
+    # Each of them would otherwise block until the consumer waves give up by themselves
+    # (ROC_SHMEM_CONSUMER_IDLE_S, 5 s) and leave the live queues without a consumer.  They
+    # return an error at once instead, and the consumer goes on serving its queues.
+    import time
+    rs.roc_shmem_init(2, 4 << 20, 2, 64)
+    try:
+        buf = rs.sym_array(1024, np.int64, fill=0)
+        world = rs.roc_shmem_team_world()
+        _, team = rs.roc_shmem_team_split_strided(world, 0, 1, 2)
+        rs.sq_consumer_start()
+        t0 = time.perf_counter()
+        refused = [lambda: rs.synchronize(), lambda: rs.sq_reset(), lambda: rs.take_status(),
+                   lambda: rs.set_pacing(0, 0), lambda: rs.sq_set_mode(1), lambda: rs.sq_consume(),
+                   lambda: rs.sq_state(0, 0), lambda: rs.sq_read(0, 0, 0), lambda: rs.sq_image(0, 0, 4),
+                   lambda: rs.cq_reader_state(0, 0), lambda: rs.sq_consumer_state(0, 0),
+                   lambda: rs.cq_image(0, 0, 4), lambda: rs.atomic_ret_image(0, 0, 8),
+                   lambda: rs.roc_shmem_free(buf.addr), lambda: rs.roc_shmem_team_destroy(team)]
+        for call in refused:
+            try:
+                result = call()
+            except rs.RocShmemError as e:
+                assert "consumer" in str(e), str(e)
+            else:
+                assert result == -1, "call went through: %r" % (result,)   # take_status reports -1
+        assert time.perf_counter() - t0 < 2.0         # nobody sat out the consumer's idle limit
+        assert rs.sq_consumer_running()
+        # the consumer is still there and still serves: a small stream goes through its queues
+        stream = rs.Stream()
+        ops = np.zeros(256, rs.SMALL_OP_DTYPE)
+        ops["kind"] = rs.OP_P64
+        ops["pe"] = np.arange(256) % 2
+        ops["offset"] = buf.offset + (np.arange(256) // 2) * 8
+        ops["value"] = np.arange(256) + 1
+        dev = rs.device_array(ops)
+        rs.roc_shmem_small_ops(dev, 256, None, rs.Launch(2, 64, 0, stream))
+        stream.synchronize()
+        totals = rs.sq_consumer_stop()
+        assert totals["lost"] == 0 and totals["rejected"] == 0 and totals["retired"] >= 256
+        assert rs.take_status() == 0
+        for p in range(2):
+            assert np.array_equal(buf.read(p)[:128], np.arange(256)[p::2] + 1)
+        dev.free()
+        stream.destroy()
+        rs.roc_shmem_team_destroy(team)
+        buf.free()
+    finally:
+        rs.roc_shmem_finalize()
+
+
 def test_a_consumer_left_alone_leaves_by_itself():
     # Every wave of the persistent kernel reaches an exit whatever the host does: with nothing
     # published for ROC_SHMEM_CONSUMER_IDLE_S the waves leave; stop then says so.
