@@ -35,6 +35,10 @@ KERNEL_SOURCES = ["roc_shmem_amd/csrc/rocshmem_device/reduce.hpp", "roc_shmem_am
 
 # Launch shapes chosen by measurement on MI355X (256 CUs).
 TO_ALL_LAUNCH = dict(wgs_per_pe=32, wg_size=1024)
+# The headline: the unchanged roc_shmem_ctx_float_sum_wg_to_all, one call per workgroup over a
+# tile of 2^21 elements (32 tiles per PE dealt to the PE's 32 workgroups of 1024 lanes; each call
+# is 8 passes of 128 KiB per member)
+TO_ALL_STANDARD_LAUNCH = dict(wgs_per_pe=32, wg_size=1024, tile=1 << 21)
 # Shapes the pacing tuner is tried with (256 workgroups either way: 128 KiB or 64 KiB per member per pass).
 TUNE_SHAPES = (dict(wgs_per_pe=32, wg_size=1024), dict(wgs_per_pe=32, wg_size=512))
 PUT_LAUNCH = dict(wgs_per_pe=32, wg_size=512)
@@ -119,7 +123,8 @@ def record_traffic(fetch_csv, write_csv):
     known = 8 * (256 << 20)                          # the copy reads and writes 2 GiB
     reduce_kernel = "void (anonymous namespace)::to_all_kernel<float"
     copy_kernel = "(anonymous namespace)::rma_kernel"
-    out = {"kernel": "to_all_kernel<float, ROC_SHMEM_SUM, sharded>", "copy_bytes_known": known}
+    out = {"kernel": "to_all_kernel<float, ROC_SHMEM_SUM, kTiled> (standard calls, one per workgroup)",
+           "copy_bytes_known": known}
     total = 0.0
     for name, path in (("FETCH_SIZE", fetch_csv), ("WRITE_SIZE", write_csv)):
         k, n_k = mean_kib(path, name, reduce_kernel)
@@ -229,7 +234,7 @@ def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, c
         rs.set_pacing(pacing_before[0], pace)
     if tune:
         tuning, best = {}, None
-        for shape in TUNE_SHAPES:
+        for shape in ([launch_shape] if launch_shape else TUNE_SHAPES):
             res = rs.tune_reduce_pacing(dtype, rs.SUM, dst, src, n, 0, 0, n_pes, psync, rs.Launch(**shape))
             tuning["%dx%d" % (shape["wgs_per_pe"], shape["wg_size"])] = {k: round(v, 4) for k, v in res.items()}
             if best is None or res["paced_ms"] < best[1]["paced_ms"]:
@@ -264,24 +269,32 @@ def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, c
         for p in range(n_pes):
             heap.view(p, 0, n, npd)[:] = host[p]
     if check:
+        # Three windows of the result (the first elements, an odd place in the middle, the last
+        # elements) on every PE: bit for bit against the oracle's statement of the library's
+        # arithmetic (integers exact; float folded in double, bfloat16 in float, ascending member
+        # order, one rounding), and for floating point within the stated tolerance of the fp64 sum.
         m = min(n, 1 << 16)
-        sample = oracle.Heap(n_pes, 2 * m * es)
-        for p in range(n_pes):
-            sample.view(p, 0, m, npd)[:] = host[p][:m]
-        got = [dst.read(p, m) for p in range(n_pes)]
-        if dtype in (rs.LONG, rs.LONGLONG):
-            oracle.to_all(sample, dtype, oracle.SUM, m * es, 0, m)
+        checked = 0
+        for at in sorted({0, max(0, (n // 2 + 12345) // 8 * 8 - m // 2), n - m}):
+            sample = oracle.Heap(n_pes, 2 * m * es)
             for p in range(n_pes):
-                assert np.array_equal(got[p], sample.view(p, m * es, m, npd)), "parity check failed"
-        else:
-            ref = oracle.to_all_f64(sample, dtype, oracle.SUM, 0, m)
-            scale = oracle.abs_sum_f64(sample, dtype, 0, m)
-            tol, eps = (1e-6, 2.0 ** -24) if dtype == rs.FLOAT else (1e-2, 2.0 ** -8)
+                sample.view(p, 0, m, npd)[:] = host[p][at:at + m]
+            got = [dst.read(p, m, at) for p in range(n_pes)]
+            oracle.to_all_rounded_once(sample, dtype, oracle.SUM, m * es, 0, m)
             for p in range(n_pes):
-                g = (oracle.bf16_to_float(got[p]) if dtype == rs.BF16 else got[p]).astype(np.float64)
-                assert (np.abs(g - ref) <= tol * np.maximum(np.abs(ref), eps * scale)).all(), \
-                    "parity check failed"
-        out["parity_checked_elements"] = m
+                assert np.array_equal(got[p].view(np.uint8), sample.view(p, m * es, m, npd).view(np.uint8)), \
+                    "parity check failed (bit-exact, window at %d, PE %d)" % (at, p)
+            if dtype not in (rs.LONG, rs.LONGLONG):
+                ref = oracle.to_all_f64(sample, dtype, oracle.SUM, 0, m)
+                scale = oracle.abs_sum_f64(sample, dtype, 0, m)
+                tol, eps = (1e-6, 2.0 ** -24) if dtype == rs.FLOAT else (1e-2, 2.0 ** -8)
+                for p in range(n_pes):
+                    g = (oracle.bf16_to_float(got[p]) if dtype == rs.BF16 else got[p]).astype(np.float64)
+                    assert (np.abs(g - ref) <= tol * np.maximum(np.abs(ref), eps * scale)).all(), \
+                        "parity check failed (tolerance, window at %d, PE %d)" % (at, p)
+            checked += m
+        out["parity_checked_elements"] = checked
+        out["parity"] = "bit-exact against the oracle in %d windows of %d elements on every PE" % (checked // m, m)
     if cpu:
         cores, host = host_threads()
 
@@ -385,34 +398,37 @@ def cpu_other_legs(oracle):
     return out
 
 
-def bench_putmem(rs, steps, n_pes, msg_bytes_list):
-    """wg putmem from every PE p to PE p+1: GB/s counted as 2*m bytes per message (read+write)."""
+def bench_putmem(rs, steps, n_pes, msg_bytes_list, get_sweep=False):
+    """wg putmem from every PE p to PE p+1: GB/s counted as 2*m bytes per message (read+write).
+    get_sweep: the same sweep with roc_shmemx_ctx_getmem_wg (the reference's tester walks every
+    size for every test type, tester.cpp:503-563), under keys "getmem_<bytes>"."""
     total = 256 << 20
     src = rs.sym_array(total, np.uint8)
     dst = rs.sym_array(total, np.uint8, fill=0)
     random_payload(rs, src, n_pes, seed=2)
     res = {}
-    for m in msg_bytes_list:
-        if m >= PUT_TILE:
-            tile, n_msgs = PUT_TILE, total // PUT_TILE      # large messages tiled across workgroups
-        else:
-            tile, n_msgs = m, min(total // max(m, 256), 1 << 16)
-        stride = max(tile, 256)
-        # A few large workgroups stream best.  A blocking put returns when its loads have, so short
-        # messages are bound by load latency and want as many resident workgroups as the CUs hold
-        # (4 KiB: 2.6 TB/s with 64 x 256 lanes per PE, 4.6 with 256 x 128).
-        launch = rs.Launch(**PUT_LAUNCH) if tile >= (64 << 10) else \
-            rs.Launch(64, 256) if tile > 4096 else rs.Launch(256, 128)
+    for kind, prefix in ((rs.PUT, ""), (rs.GET, "getmem_")) if get_sweep else ((rs.PUT, ""),):
+        for m in msg_bytes_list:
+            if m >= PUT_TILE:
+                tile, n_msgs = PUT_TILE, total // PUT_TILE      # large messages tiled across workgroups
+            else:
+                tile, n_msgs = m, min(total // max(m, 256), 1 << 16)
+            stride = max(tile, 256)
+            # A few large workgroups stream best.  A blocking put returns when its loads have, so short
+            # messages are bound by load latency and want as many resident workgroups as the CUs hold
+            # (4 KiB: 2.6 TB/s with 64 x 256 lanes per PE, 4.6 with 256 x 128).
+            launch = rs.Launch(**PUT_LAUNCH) if tile >= (64 << 10) else \
+                rs.Launch(64, 256) if tile > 4096 else rs.Launch(256, 128)
 
-        def step():
-            rs.roc_shmem_rma(rs.PUT, rs.WG, dst, src, tile, n_msgs, stride, stride, 1, launch)
+            def step():
+                rs.roc_shmem_rma(kind, rs.WG, dst, src, tile, n_msgs, stride, stride, 1, launch)
 
-        step()
-        rs.synchronize()
-        ms = event_time_ms(rs, step, steps) / steps
-        moved = 2.0 * n_pes * tile * n_msgs
-        res[str(m)] = {"GBps": moved / ms / 1e6, "ms": ms, "calls_per_pe": n_msgs, "bytes_per_call": tile,
-                       "Mmsgs_per_s": n_pes * n_msgs / ms / 1e3}
+            step()
+            rs.synchronize()
+            ms = event_time_ms(rs, step, steps) / steps
+            moved = 2.0 * n_pes * tile * n_msgs
+            res[prefix + str(m)] = {"GBps": moved / ms / 1e6, "ms": ms, "calls_per_pe": n_msgs, "bytes_per_call": tile,
+                                    "Mmsgs_per_s": n_pes * n_msgs / ms / 1e3}
     # getmem in the same shape as the largest put
     launch = rs.Launch(**PUT_LAUNCH)
 
@@ -459,6 +475,51 @@ def bench_putmem(rs, steps, n_pes, msg_bytes_list):
         ms = event_time_ms(rs, one_call, steps) / steps
         one[str(m)] = {"GBps": 2.0 * n_pes * m / ms / 1e6, "us": ms * 1e3}
     res["one_workgroup_per_pe_one_call_per_message"] = one
+    src.free()
+    dst.free()
+    return res
+
+
+def bench_nbi_windows(rs, steps, n_pes, msg_bytes_list):
+    """The reference's message-rate pattern (primitive_mr_tester.cpp:32-58: 64 putmem_nbi, one
+    quiet) at workgroup and at wavefront granularity: every workgroup (every wave) issues a window
+    of 64 roc_shmemx_ctx_putmem_nbi_wg (_wave) calls of one size to the next PE, then the
+    workgroup's waves meet and one lane issues the quiet.  GB/s counted as 2*m bytes per message,
+    M messages/s; the launch shape is the best of a few for each size (named in the row).  A
+    kernel is one window per workgroup, so the figures include one launch per 64 calls."""
+    total = 256 << 20
+    src = rs.sym_array(total, np.uint8)
+    dst = rs.sym_array(total, np.uint8, fill=0)
+    random_payload(rs, src, n_pes, seed=2)
+    shapes = {"wg": ((256, 128), (64, 256), (64, 512), (32, 512), (32, 1024)),
+              "wave": ((64, 256), (32, 512), (32, 1024), (64, 512))}
+    res = {}
+    for gran, gname in ((rs.WG, "wg"), (rs.WAVE, "wave")):
+        rows = {}
+        for kind, kname in ((rs.PUT_NBI, "putmem_nbi"), (rs.GET_NBI, "getmem_nbi")):
+            for m in msg_bytes_list:
+                stride, best = max(m, 256), None
+                for wgs, lanes in shapes[gname]:
+                    n_msgs = 64 * (wgs if gname == "wg" else wgs * (lanes // 64))
+                    if n_msgs * stride > total:
+                        continue
+                    launch = rs.Launch(wgs, lanes)
+
+                    def step():
+                        rs.roc_shmem_rma(kind, gran, dst, src, m, n_msgs, stride, stride, 1, launch)
+
+                    step()
+                    rs.synchronize()
+                    ms = event_time_ms(rs, step, steps) / steps
+                    rate = 2.0 * n_pes * m * n_msgs / ms / 1e6
+                    if best is None or rate > best["GBps"]:
+                        best = {"GBps": round(rate, 1), "Mmsgs_per_s": round(n_pes * n_msgs / ms / 1e3, 1),
+                                "us_per_window_kernel": round(ms * 1e3, 2), "launch": "%dx%d" % (wgs, lanes)}
+                if best:
+                    rows["%s_%d" % (kname, m)] = best
+        res[gname] = rows
+    if rs.take_status():
+        raise RuntimeError("device status word raised")
     src.free()
     dst.free()
     return res
@@ -956,6 +1017,8 @@ def main():
     ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="no GPU work: read the two rocprofv3 --pmc counter files of --counter-pair runs and "
                          "write the tracked traffic summary under profiles/")
+    ap.add_argument("--sharded", action="store_true",
+                    help="with --counter-pair: launch the sharded extension instead of the headline's standard calls")
     ap.add_argument("--timeline", metavar="FILE",
                     help="no GPU work: summarise the clock readings a timeline build of the library wrote "
                          "(ROC_SHMEM_TIMELINE_FILE)")
@@ -1041,21 +1104,21 @@ def main():
     rs.roc_shmem_init(n_pes, 1 << 30, 64, 1024)
     if args.counter_pair:
         out = bench_to_all(rs, oracle, 3, 1, rs.FLOAT, n_pes, n, seed=3, check=False,
+                           launch_shape=None if args.sharded else TO_ALL_STANDARD_LAUNCH,
                            pace=0 if args.no_pacing else (args.pace_reduce or None))
         put = bench_putmem(rs, 3, n_pes, [64 << 20])
         rs.roc_shmem_finalize()
         print(json.dumps({"to_all": out, "putmem_copy": put,
                           "copy_bytes_read": n_pes * (256 << 20), "copy_bytes_written": n_pes * (256 << 20)}))
         return
-    # The headline runs as a caller's loop would: the library's default pacing rate, no tuning.
-    # --tune lets the library's tuner pick shape and rate first (outside the timed region),
+    # The headline runs as a caller's loop would: the reference's own symbol
+    # (roc_shmem_ctx_float_sum_wg_to_all), one call per workgroup over its tile of the array, the
+    # library's default pacing rates, no tuning.
+    # --tune lets the library's tuner pick the rate first (outside the timed region),
     # --pace-reduce R / --no-pacing fix the rate (0 = workgroups run free).
-    if args.tune:
-        head = bench_to_all(rs, oracle, args.steps, args.warmup, rs.FLOAT, n_pes, n, seed=3, cpu=True,
-                            spread=True, tune=True)
-    else:
-        head = bench_to_all(rs, oracle, args.steps, args.warmup, rs.FLOAT, n_pes, n, seed=3, cpu=True,
-                            spread=True, pace=0 if args.no_pacing else (args.pace_reduce or None))
+    head = bench_to_all(rs, oracle, args.steps, args.warmup, rs.FLOAT, n_pes, n, seed=3, cpu=True,
+                        spread=True, launch_shape=TO_ALL_STANDARD_LAUNCH, tune=args.tune,
+                        pace=None if args.tune else (0 if args.no_pacing else (args.pace_reduce or None)))
     extra = {}
     # against workgroups that stay, the shape the reduction's own workgroups have, and against the
     # best plain copy the card did in any shape (a 1:1 stream like the reduction's)
@@ -1063,23 +1126,36 @@ def main():
     streams["headline_over_best_plain_copy"] = round(
         head["GBps"] / max(streams["staying"]["copy"]["GBps"], streams["one_per_pass"]["copy"]["GBps"]), 4)
     extra["hbm_streams_on_this_card"] = streams
+    # the sharded extension (the PE's 32 workgroups share one call), same launch shape and rates
+    extra["to_all_float_sum_8x2^26_sharded_extension"] = bench_to_all(
+        rs, oracle, args.steps, 3, rs.FLOAT, n_pes, n, seed=3, spread=True,
+        pace=0 if args.no_pacing else (args.pace_reduce or None))
+    extra["to_all_float_sum_8x2^26_sharded_extension"]["api"] = "roc_shmemx_ctx_float_sum_wg_to_all_shard"
     if not args.quick:
         extra["to_all_float_sum_8x2^26_free_running"] = bench_to_all(
-            rs, oracle, max(args.steps // 2, 3), 2, rs.FLOAT, n_pes, n, seed=3, check=False, pace=0)
+            rs, oracle, max(args.steps // 2, 3), 2, rs.FLOAT, n_pes, n, seed=3, check=False, pace=0,
+            launch_shape=TO_ALL_STANDARD_LAUNCH)
         extra["to_all_float_sum_8x2^26_rate_from_the_tuner"] = bench_to_all(
             rs, oracle, max(args.steps // 2, 3), 2, rs.FLOAT, n_pes, n, seed=3, check=False, tune=True)
+        # workgroups of 512 lanes (passes of 64 KiB per member) at the library's rate for short passes
+        extra["to_all_float_sum_8x2^26_standard_api_32x512"] = bench_to_all(
+            rs, oracle, max(args.steps // 2, 3), 2, rs.FLOAT, n_pes, n, seed=3, check=False,
+            launch_shape=dict(wgs_per_pe=32, wg_size=512, tile=1 << 21))
+        extra["to_all_float_sum_8x2^26_sharded_32x512"] = bench_to_all(
+            rs, oracle, max(args.steps // 2, 3), 2, rs.FLOAT, n_pes, n, seed=3, check=False,
+            launch_shape=dict(wgs_per_pe=32, wg_size=512))
         extra["to_all_bf16_sum_8x2^26"] = {k: v for k, v in bench_to_all(
             rs, oracle, max(args.steps // 2, 3), 2, rs.BF16, n_pes, n, seed=3,
+            launch_shape=dict(wgs_per_pe=32, wg_size=1024, tile=1 << 21),
             pace=0 if args.no_pacing else None).items() if k != "cpu"}
-        # every power of two from 8 B to 64 MiB (BASELINE configs[1]; the reference's own sweep,
-        # clients/functional_tests/tester.cpp:503-563)
-        extra["putmem_wg_8pe"] = bench_putmem(rs, 5, n_pes, [1 << k for k in range(3, 27)])
-        # the unchanged standard call, one per 2^20-element tile, tiles dealt to 64 workgroups per PE
-        extra["to_all_float_sum_8x2^26_standard_api_tiled"] = {
-            k: v for k, v in bench_to_all(rs, oracle, max(args.steps // 2, 3), 2, rs.FLOAT, n_pes, n, seed=3,
-                                          launch_shape=dict(wgs_per_pe=64, wg_size=512, tile=1 << 20)).items()}
-        extra["to_all_float_sum_8x2^26_standard_api_tiled"]["api"] = \
-            "roc_shmem_ctx_float_sum_wg_to_all, one call per tile of 2^20 elements"
+        extra["to_all_bf16_sum_8x2^26_sharded_extension"] = {k: v for k, v in bench_to_all(
+            rs, oracle, max(args.steps // 2, 3), 2, rs.BF16, n_pes, n, seed=3, check=False,
+            pace=0 if args.no_pacing else None).items() if k != "cpu"}
+        # every power of two from 8 B to 64 MiB, put and get (BASELINE configs[1]; the reference's
+        # own sweep, clients/functional_tests/tester.cpp:503-563)
+        extra["putmem_wg_8pe"] = bench_putmem(rs, 5, n_pes, [1 << k for k in range(3, 27)], get_sweep=True)
+        # windows of 64 non-blocking puts / gets and one quiet (primitive_mr_tester.cpp:32-58)
+        extra["nbi_windows_8pe"] = bench_nbi_windows(rs, 5, n_pes, [1 << k for k in range(3, 19)])
         extra["putmem_getmem_per_wave_and_thread_8pe"] = bench_granularities(rs, 5, n_pes)
         extra["collectives_4KiB_8pe_one_wg_of_256"] = bench_small_latencies(rs, n_pes)
     rs.roc_shmem_finalize()
@@ -1110,6 +1186,15 @@ def main():
     if not args.quick:
         cpu["other_legs"] = cpu_other_legs(oracle)
     traffic, traffic_note = measured_traffic()
+
+    def pick(*path):
+        node = extra
+        for key in path:
+            if not isinstance(node, dict) or key not in node:
+                return None
+            node = node[key]
+        return round(node, 1) if isinstance(node, float) else node
+
     line = {
         "metric": "to_all reduce + putmem GB/s (% of HBM peak); small-put/AMO Mops/s",
         "value": round(head["GBps"], 1),
@@ -1125,22 +1210,44 @@ def main():
         "data": "synthetic",
         "config": {"workload": "float sum_to_all over 8 PE slices x 2^26 elements, N(0,1) inputs, "
                                "all slices in one GPU's HBM (BASELINE configs[2], fp32 sum)",
-                   "api": "roc_shmemx_ctx_float_sum_wg_to_all_shard (the sharded extension: the 32 workgroups of "
-                          "a PE share one reduction); the unchanged roc_shmem_ctx_float_sum_wg_to_all, tiled over "
-                          "workgroups, is extra.to_all_float_sum_8x2^26_standard_api_tiled",
+                   "api": "roc_shmem_ctx_float_sum_wg_to_all (the reference's symbol, library/include/roc_shmem.hpp:"
+                          "837-851), one call per workgroup over a tile of 2^21 elements, 32 workgroups of 1024 "
+                          "lanes per PE; the sharded extension is extra.to_all_float_sum_8x2^26_sharded_extension",
                    "pes": n_pes, "elements_per_pe": n, "algorithmic_bytes_per_step": head["bytes_per_step"],
                    "launch": head["launch"], "pacing_bytes_per_tick": head["pacing_bytes_per_tick"],
                    "pacing_tuner": head.get("pacing_tuner"),
-                   "parity_checked_elements": head.get("parity_checked_elements")},
+                   "parity_checked_elements": head.get("parity_checked_elements"), "parity": head.get("parity")},
         "roofline": {"bound": "hbm", "achieved": round(head["GBps"], 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(head["GBps"] / HBM_PEAK_GBPS, 4),
                      "traffic": traffic, "traffic_source": traffic_note},
         "cpu_baseline": {k: (round(v, 2) if isinstance(v, float) else v) for k, v in cpu.items()},
         "per_launch_ms": {"median": round(head["ms_median"], 4), "min": round(head["ms_min"], 4),
                           "max": round(head["ms_max"], 4)},
+        # the legs of the metric in one place (GB/s unless named otherwise; null = not run with --quick)
+        "standard_api_GBps": round(head["GBps"], 1),
+        "sharded_extension_GBps": pick("to_all_float_sum_8x2^26_sharded_extension", "GBps"),
+        "bf16_GBps": pick("to_all_bf16_sum_8x2^26", "GBps"),
+        "standard_api_32x512_GBps": pick("to_all_float_sum_8x2^26_standard_api_32x512", "GBps"),
+        "putmem_64MiB_GBps": pick("putmem_wg_8pe", "67108864", "GBps"),
+        "getmem_64MiB_GBps": pick("putmem_wg_8pe", "getmem_67108864", "GBps"),
+        "putmem_64MiB_shard_GBps": pick("putmem_wg_8pe", "67108864_shared", "GBps"),
+        "putmem_4KiB_GBps": pick("putmem_wg_8pe", "4096", "GBps"),
+        "putmem_64KiB_GBps": pick("putmem_wg_8pe", "65536", "GBps"),
+        "putmem_nbi_wg_4KiB_GBps": pick("nbi_windows_8pe", "wg", "putmem_nbi_4096", "GBps"),
+        "putmem_nbi_wg_64KiB_GBps": pick("nbi_windows_8pe", "wg", "putmem_nbi_65536", "GBps"),
+        "putmem_nbi_wave_4KiB_GBps": pick("nbi_windows_8pe", "wave", "putmem_nbi_4096", "GBps"),
+        "small_put_Mops": pick("small_ops_16x64MiB_1024wg_x256", "put8", "Mops_per_s"),
+        "fetch_add_Mops": pick("small_ops_16x64MiB_1024wg_x256", "fetch_add", "Mops_per_s"),
+        "mixed_live_queue_Mops": pick("small_ops_16x64MiB_1024wg_x256", "mixed_through_live_queues", "Mops_per_s"),
+        "broadcast_GBps": pick("collectives_16x64MiB", "broadcast", "GBps"),
+        "alltoall_GBps": pick("collectives_16x64MiB", "alltoall", "GBps"),
+        "fcollect_GBps": pick("collectives_16x64MiB", "fcollect", "GBps"),
+        "int64_sum_4x2^20_us": pick("to_all_int64_sum_4x2^20", "ms_per_step"),
         "device": device,
         "extra": extra,
     }
+    if line["int64_sum_4x2^20_us"] is not None:
+        line["int64_sum_4x2^20_us"] = round(extra["to_all_int64_sum_4x2^20"]["ms_per_step"] * 1e3, 2)
     print(json.dumps(line))
 
 

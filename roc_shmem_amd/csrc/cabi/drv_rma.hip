@@ -78,9 +78,37 @@ __global__ void __launch_bounds__(1024)
   // is complete when all of them have returned, which no single workgroup can know: there the
   // end of the kernel is the completion point and a quiet per workgroup would only cost (every
   // quiet writes the XCD's whole L2 back: 6.26 -> 6.43 TB/s for 64 MiB messages without it).
-  if (threadIdx.x == 0 && granularity != RSM_WG_SHARED) roc_shmem_ctx_quiet(ctx);
+  // The waves meet first, each with its own stores complete (__syncthreads), so that the one
+  // lane's quiet covers what the whole workgroup has issued - the non-blocking forms return
+  // without the waves having met.
+  if (granularity != RSM_WG_SHARED) {
+    __syncthreads();
+    if (threadIdx.x == 0) roc_shmem_ctx_quiet(ctx);
+  }
   roc_shmem_wg_ctx_destroy(ctx);
   roc_shmem_wg_finalize();
+}
+
+// RSM_WG_SHARED alone, for grids of many short-lived workgroups (one workgroup per share of a few
+// KiB is the launch shape of the fastest plain copy): nothing in front of the call but the
+// kernel's arguments - no context handle in LDS, no workgroup barrier - so that the first payload
+// load is a dozen scalar instructions away from the workgroup's start.
+__global__ void __launch_bounds__(1024)
+    rma_shared_kernel(int is_put, char *dest, const char *source, size_t msg_bytes, size_t n_msgs,
+                      size_t dst_stride, size_t src_stride, int pe_shift) {
+  const int npes = roc_shmem_n_pes();
+  const int target = (roc_shmem_my_pe() + pe_shift) % npes;
+  const int w = static_cast<int>(blockIdx.x / npes);
+  const int nw = static_cast<int>(gridDim.x / npes);
+  for (size_t m = 0; m < n_msgs; ++m) {
+    char *d = dest + m * dst_stride;
+    const char *s = source + m * src_stride;
+    if (is_put) {
+      roc_shmemx_ctx_putmem_wg_shard(ROC_SHMEM_CTX_DEFAULT, d, s, msg_bytes, target, w, nw);
+    } else {
+      roc_shmemx_ctx_getmem_wg_shard(ROC_SHMEM_CTX_DEFAULT, d, s, msg_bytes, target, w, nw);
+    }
+  }
 }
 
 }  // namespace
@@ -107,6 +135,12 @@ extern "C" int rsm_rma(int kind, int granularity, void *dest, const void *source
   if (!rsm::check_extent(dest, (n_msgs - 1) * dst_stride + msg_bytes, "rma: dest") ||
       !rsm::check_extent(source, (n_msgs - 1) * src_stride + msg_bytes, "rma: source"))
     return -1;
+  if (granularity == RSM_WG_SHARED) {
+    hipLaunchKernelGGL(rma_shared_kernel, dim3(l.grid), dim3(l.wg_size), 0, l.stream,
+                       (kind == RSM_PUT || kind == RSM_PUT_NBI) ? 1 : 0, static_cast<char *>(dest),
+                       static_cast<const char *>(source), msg_bytes, n_msgs, dst_stride, src_stride, pe_shift);
+    return rsm::after_launch("rma");
+  }
   hipLaunchKernelGGL(rma_kernel, dim3(l.grid), dim3(l.wg_size), 0, l.stream, kind, granularity,
                      static_cast<char *>(dest), static_cast<const char *>(source), msg_bytes,
                      n_msgs, dst_stride, src_stride, pe_shift);

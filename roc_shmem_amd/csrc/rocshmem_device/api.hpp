@@ -59,6 +59,13 @@ __device__ __forceinline__ DeviceCtx *ctx_of(roc_shmem_ctx_t ctx) {
   return ctx.ctx_opaque ? static_cast<DeviceCtx *>(ctx.ctx_opaque) : launch_ctx();
 }
 
+// The PE a context handle acts for.  A handle names a context of the launching PE's table row
+// (roc_shmem_wg_ctx_create, ROC_SHMEM_CTX_DEFAULT), so this is the grid position's PE and needs
+// no look at the context: the calls that only move data (put, get, the collectives) never load
+// from the context table, which used to put a chain of dependent memory reads - the handle from
+// LDS, then the context's PE from memory - in front of a call's first payload load.
+__device__ __forceinline__ int pe_of(roc_shmem_ctx_t) { return launch_pe(); }
+
 // reference: translate_pe, roc_shmem_gpu.cpp:240-247
 __device__ __forceinline__ int world_pe(roc_shmem_ctx_t ctx, int pe) {
   if (ctx.team_opaque) {
@@ -72,11 +79,12 @@ __device__ __forceinline__ Team *team_of(roc_shmem_team_t team) {
   return reinterpret_cast<Team *>(team);
 }
 
-// This PE's copy of a team-owned pSync slice for the calling context's block.
-__device__ __forceinline__ long *team_psync(const DeviceCtx *c, uint64_t pool_off) {
-  char *slice = g_state.heap_base0 + static_cast<uint64_t>(c->my_pe) * g_state.slice_stride;
+// This PE's copy of a team-owned pSync slice for the calling context's block.  PE and block
+// follow from the grid position (launch_ctx), so nothing is read from the context.
+__device__ __forceinline__ long *team_psync(roc_shmem_ctx_t, uint64_t pool_off) {
+  char *slice = g_state.heap_base0 + static_cast<uint64_t>(launch_pe()) * g_state.slice_stride;
   return reinterpret_cast<long *>(slice + pool_off) +
-         static_cast<size_t>(c->block_id) * kSyncSlots;
+         static_cast<size_t>(launch_wg_rank() % g_state.num_blocks) * kSyncSlots;
 }
 
 }  // namespace detail
@@ -120,11 +128,12 @@ __device__ inline int roc_shmem_wg_team_create_ctx(roc_shmem_team_t team, long o
 __device__ inline void roc_shmem_wg_ctx_destroy(roc_shmem_ctx_t) {}
 
 __device__ inline int roc_shmem_ctx_n_pes(roc_shmem_ctx_t ctx) {
-  return detail::ctx_of(ctx)->num_pes;
+  (void)ctx;
+  return detail::g_state.num_pes;
 }
 __device__ inline int roc_shmem_n_pes() { return detail::g_state.num_pes; }
 __device__ inline int roc_shmem_ctx_my_pe(roc_shmem_ctx_t ctx) {
-  return detail::ctx_of(ctx)->my_pe;
+  return detail::pe_of(ctx);
 }
 __device__ inline int roc_shmem_my_pe() { return detail::launch_pe(); }
 
@@ -159,7 +168,9 @@ __device__ inline T *roc_shmemx_my_addr(T *ptr) {
   const char *base = detail::g_state.heap_base0;
   const uint64_t span = detail::g_state.slice_stride * static_cast<uint64_t>(detail::g_state.num_pes);
   if (c < base || static_cast<uint64_t>(c - base) >= span) return ptr;
-  uint64_t off = static_cast<uint64_t>(c - base) % detail::g_state.slice_stride;
+  // (the usual argument is the symmetric address, in PE 0's slice: no division then)
+  const uint64_t rel = static_cast<uint64_t>(c - base);
+  const uint64_t off = rel < detail::g_state.slice_stride ? rel : rel % detail::g_state.slice_stride;
   return reinterpret_cast<T *>(const_cast<char *>(base) +
                                static_cast<uint64_t>(detail::launch_pe()) *
                                    detail::g_state.slice_stride +
@@ -258,8 +269,8 @@ __device__ inline void roc_shmem_getmem_nbi(void *dest, const void *source, size
 __device__ inline void roc_shmemx_ctx_putmem_nbi_wg(roc_shmem_ctx_t ctx, void *dest,
                                                     const void *source, size_t nelems, int pe) {
   if (nelems == 0) return;
-  const detail::DeviceCtx *c = detail::ctx_of(ctx);
-  detail::wg_copy(detail::translate(detail::own(dest, c), c->my_pe, pe), detail::own(source, c), nelems);
+  const int me = detail::pe_of(ctx);
+  detail::wg_copy(detail::translate(detail::own(dest, me), me, pe), detail::own(source, me), nelems);
 }
 __device__ inline void roc_shmemx_ctx_putmem_wg(roc_shmem_ctx_t ctx, void *dest,
                                                 const void *source, size_t nelems, int pe) {
@@ -279,8 +290,8 @@ __device__ inline void roc_shmemx_ctx_putmem_wg(roc_shmem_ctx_t ctx, void *dest,
 __device__ inline void roc_shmemx_ctx_getmem_nbi_wg(roc_shmem_ctx_t ctx, void *dest,
                                                     const void *source, size_t nelems, int pe) {
   if (nelems == 0) return;
-  const detail::DeviceCtx *c = detail::ctx_of(ctx);
-  detail::wg_copy(detail::own(dest, c), detail::translate(detail::own(source, c), c->my_pe, pe), nelems);
+  const int me = detail::pe_of(ctx);
+  detail::wg_copy(detail::own(dest, me), detail::translate(detail::own(source, me), me, pe), nelems);
 }
 __device__ inline void roc_shmemx_ctx_getmem_wg(roc_shmem_ctx_t ctx, void *dest,
                                                 const void *source, size_t nelems, int pe) {
@@ -298,24 +309,24 @@ __device__ inline void roc_shmemx_ctx_putmem_wg_shard(roc_shmem_ctx_t ctx, void 
                                                       const void *source, size_t nelems, int pe,
                                                       int shard, int nshards) {
   if (nelems == 0) return;
-  const detail::DeviceCtx *c = detail::ctx_of(ctx);
-  detail::wg_copy_shard(detail::translate(detail::own(dest, c), c->my_pe, pe), detail::own(source, c), nelems,
+  const int me = detail::pe_of(ctx);
+  detail::wg_copy_shard(detail::translate(detail::own(dest, me), me, pe), detail::own(source, me), nelems,
                         shard, nshards, detail::g_state.pace_copy_bytes_per_tick);
 }
 __device__ inline void roc_shmemx_ctx_getmem_wg_shard(roc_shmem_ctx_t ctx, void *dest,
                                                       const void *source, size_t nelems, int pe,
                                                       int shard, int nshards) {
   if (nelems == 0) return;
-  const detail::DeviceCtx *c = detail::ctx_of(ctx);
-  detail::wg_copy_shard(detail::own(dest, c), detail::translate(detail::own(source, c), c->my_pe, pe), nelems,
+  const int me = detail::pe_of(ctx);
+  detail::wg_copy_shard(detail::own(dest, me), detail::translate(detail::own(source, me), me, pe), nelems,
                         shard, nshards, detail::g_state.pace_copy_bytes_per_tick);
 }
 __device__ inline void roc_shmemx_ctx_putmem_nbi_wave(roc_shmem_ctx_t ctx, void *dest,
                                                       const void *source, size_t nelems,
                                                       int pe) {
   if (nelems == 0) return;
-  const detail::DeviceCtx *c = detail::ctx_of(ctx);
-  detail::wave_copy(detail::translate(detail::own(dest, c), c->my_pe, pe), detail::own(source, c), nelems);
+  const int me = detail::pe_of(ctx);
+  detail::wave_copy(detail::translate(detail::own(dest, me), me, pe), detail::own(source, me), nelems);
 }
 __device__ inline void roc_shmemx_ctx_putmem_wave(roc_shmem_ctx_t ctx, void *dest,
                                                   const void *source, size_t nelems, int pe) {
@@ -327,8 +338,8 @@ __device__ inline void roc_shmemx_ctx_getmem_nbi_wave(roc_shmem_ctx_t ctx, void 
                                                       const void *source, size_t nelems,
                                                       int pe) {
   if (nelems == 0) return;
-  const detail::DeviceCtx *c = detail::ctx_of(ctx);
-  detail::wave_copy(detail::own(dest, c), detail::translate(detail::own(source, c), c->my_pe, pe), nelems);
+  const int me = detail::pe_of(ctx);
+  detail::wave_copy(detail::own(dest, me), detail::translate(detail::own(source, me), me, pe), nelems);
 }
 __device__ inline void roc_shmemx_ctx_getmem_wave(roc_shmem_ctx_t ctx, void *dest,
                                                   const void *source, size_t nelems, int pe) {
@@ -457,7 +468,7 @@ __device__ __forceinline__ void to_all_active_set(roc_shmem_ctx_t ctx, T *dest, 
                                                   size_t nreduce, int pe_start, int log_stride,
                                                   int pe_size, long *psync, int shard = 0,
                                                   int nshards = 1) {
-  wg_all_reduce<T, Op>(ctx_of(ctx)->my_pe, dest, source, nreduce, pe_start, 1 << log_stride,
+  wg_all_reduce<T, Op>(pe_of(ctx), dest, source, nreduce, pe_start, 1 << log_stride,
                        pe_size, psync, shard, nshards);
 }
 // reference: GPUIBContext::to_all(team, ...), context_ib_tmpl_device.hpp:238-260
@@ -465,11 +476,10 @@ template <typename T, ROC_SHMEM_OP Op>
 __device__ __forceinline__ void to_all_team(roc_shmem_ctx_t ctx, roc_shmem_team_t team, T *dest,
                                             const T *source, size_t nreduce, int shard = 0,
                                             int nshards = 1) {
-  const DeviceCtx *c = ctx_of(ctx);
   const Team *t = team_of(team);
-  wg_all_reduce<T, Op>(c->my_pe, dest, source, nreduce, t->wrt_world.pe_start,
+  wg_all_reduce<T, Op>(pe_of(ctx), dest, source, nreduce, t->wrt_world.pe_start,
                        t->wrt_world.stride, t->wrt_world.size,
-                       team_psync(c, t->reduce_psync_off), shard, nshards);
+                       team_psync(ctx, t->reduce_psync_off), shard, nshards);
 }
 }  // namespace detail
 
@@ -544,7 +554,7 @@ ROCSHMEM_REDUCTION(__hip_bfloat16, bf16, min, ROC_SHMEM_MIN)
       roc_shmem_ctx_t ctx, T *dest, const T *source, int nelem, int pe_root, int pe_start,     \
       int log_pe_stride, int pe_size, long *p_sync) {                                          \
     if (nelem <= 0) return;                                                                    \
-    detail::wg_broadcast_bytes(detail::ctx_of(ctx)->my_pe, dest, source,                       \
+    detail::wg_broadcast_bytes(detail::pe_of(ctx), dest, source,                       \
                                static_cast<size_t>(nelem) * sizeof(T), pe_root, pe_start,      \
                                1 << log_pe_stride, pe_size, p_sync);                           \
   }                                                                                            \
@@ -552,29 +562,27 @@ ROCSHMEM_REDUCTION(__hip_bfloat16, bf16, min, ROC_SHMEM_MIN)
       roc_shmem_ctx_t ctx, roc_shmem_team_t team, T *dest, const T *source, int nelem,         \
       int pe_root) {                                                                           \
     if (nelem <= 0) return;                                                                    \
-    const detail::DeviceCtx *c = detail::ctx_of(ctx);                                          \
     const detail::Team *t = detail::team_of(team);                                             \
-    detail::wg_broadcast_bytes(c->my_pe, dest, source, static_cast<size_t>(nelem) * sizeof(T), \
+    detail::wg_broadcast_bytes(detail::pe_of(ctx), dest, source, static_cast<size_t>(nelem) * sizeof(T), \
                                pe_root, t->wrt_world.pe_start, t->wrt_world.stride,            \
-                               t->wrt_world.size, detail::team_psync(c, t->bcast_psync_off));  \
+                               t->wrt_world.size, detail::team_psync(ctx, t->bcast_psync_off));  \
   }                                                                                            \
   /* extension: `nshards` workgroups of every member share one broadcast (same */              \
   /* arguments in all of them, nelem a size_t; complete when all have returned) */             \
   __device__ inline void roc_shmemx_ctx_##TNAME##_wg_broadcast_shard(                          \
       roc_shmem_ctx_t ctx, T *dest, const T *source, size_t nelem, int pe_root, int pe_start,  \
       int log_pe_stride, int pe_size, long *p_sync, int shard, int nshards) {                  \
-    detail::wg_broadcast_bytes(detail::ctx_of(ctx)->my_pe, dest, source, nelem * sizeof(T),    \
+    detail::wg_broadcast_bytes(detail::pe_of(ctx), dest, source, nelem * sizeof(T),    \
                                pe_root, pe_start, 1 << log_pe_stride, pe_size, p_sync, shard,  \
                                nshards);                                                       \
   }                                                                                            \
   __device__ inline void roc_shmemx_ctx_##TNAME##_wg_broadcast_shard(                          \
       roc_shmem_ctx_t ctx, roc_shmem_team_t team, T *dest, const T *source, size_t nelem,      \
       int pe_root, int shard, int nshards) {                                                   \
-    const detail::DeviceCtx *c = detail::ctx_of(ctx);                                          \
     const detail::Team *t = detail::team_of(team);                                             \
-    detail::wg_broadcast_bytes(c->my_pe, dest, source, nelem * sizeof(T), pe_root,             \
+    detail::wg_broadcast_bytes(detail::pe_of(ctx), dest, source, nelem * sizeof(T), pe_root,             \
                                t->wrt_world.pe_start, t->wrt_world.stride,                     \
-                               t->wrt_world.size, detail::team_psync(c, t->bcast_psync_off),   \
+                               t->wrt_world.size, detail::team_psync(ctx, t->bcast_psync_off),   \
                                shard, nshards);                                                \
   }                                                                                            \
   /* extension: `nshards` workgroups of every member share the exchange */                        \
@@ -582,11 +590,10 @@ ROCSHMEM_REDUCTION(__hip_bfloat16, bf16, min, ROC_SHMEM_MIN)
       roc_shmem_ctx_t ctx, roc_shmem_team_t team, T *dest, const T *source, int nelem,         \
       int shard, int nshards) {                                                                \
     if (nelem <= 0) return;                                                                    \
-    const detail::DeviceCtx *c = detail::ctx_of(ctx);                                          \
     const detail::Team *t = detail::team_of(team);                                             \
-    detail::wg_alltoall_bytes(c->my_pe, dest, source, static_cast<size_t>(nelem) * sizeof(T),  \
+    detail::wg_alltoall_bytes(detail::pe_of(ctx), dest, source, static_cast<size_t>(nelem) * sizeof(T),  \
                               shard, nshards, t->wrt_world.pe_start, t->wrt_world.stride,      \
-                              t->wrt_world.size, detail::team_psync(c, t->alltoall_psync_off)); \
+                              t->wrt_world.size, detail::team_psync(ctx, t->alltoall_psync_off)); \
   }                                                                                            \
   __device__ inline void roc_shmem_ctx_##TNAME##_wg_alltoall(                                  \
       roc_shmem_ctx_t ctx, roc_shmem_team_t team, T *dest, const T *source, int nelem) {       \
@@ -596,11 +603,10 @@ ROCSHMEM_REDUCTION(__hip_bfloat16, bf16, min, ROC_SHMEM_MIN)
       roc_shmem_ctx_t ctx, roc_shmem_team_t team, T *dest, const T *source, int nelem,         \
       int shard, int nshards) {                                                                \
     if (nelem <= 0) return;                                                                    \
-    const detail::DeviceCtx *c = detail::ctx_of(ctx);                                          \
     const detail::Team *t = detail::team_of(team);                                             \
-    detail::wg_fcollect_bytes(c->my_pe, dest, source, static_cast<size_t>(nelem) * sizeof(T),  \
+    detail::wg_fcollect_bytes(detail::pe_of(ctx), dest, source, static_cast<size_t>(nelem) * sizeof(T),  \
                               shard, nshards, t->wrt_world.pe_start, t->wrt_world.stride,      \
-                              t->wrt_world.size, detail::team_psync(c, t->alltoall_psync_off)); \
+                              t->wrt_world.size, detail::team_psync(ctx, t->alltoall_psync_off)); \
   }                                                                                            \
   __device__ inline void roc_shmem_ctx_##TNAME##_wg_fcollect(                                  \
       roc_shmem_ctx_t ctx, roc_shmem_team_t team, T *dest, const T *source, int nelem) {       \
@@ -614,19 +620,17 @@ ROCSHMEM_STANDARD_TYPES(ROCSHMEM_COLLECTIVES)
 // ---------------------------------------------------------------------------
 
 __device__ inline void roc_shmem_ctx_wg_team_sync(roc_shmem_ctx_t ctx, roc_shmem_team_t team) {
-  const detail::DeviceCtx *c = detail::ctx_of(ctx);
   const detail::Team *t = detail::team_of(team);
-  detail::wg_sync_members(c->my_pe, t->wrt_world.pe_start, t->wrt_world.stride,
-                          t->wrt_world.size, detail::team_psync(c, t->barrier_psync_off));
+  detail::wg_sync_members(detail::pe_of(ctx), t->wrt_world.pe_start, t->wrt_world.stride,
+                          t->wrt_world.size, detail::team_psync(ctx, t->barrier_psync_off));
 }
 __device__ inline void roc_shmem_wg_team_sync(roc_shmem_team_t team) {
   roc_shmem_ctx_wg_team_sync(ROC_SHMEM_CTX_DEFAULT, team);
 }
 __device__ inline void roc_shmem_ctx_wg_sync_all(roc_shmem_ctx_t ctx) {
-  const detail::DeviceCtx *c = detail::ctx_of(ctx);
   const detail::Team *t = detail::g_state.team_world;
-  detail::wg_sync_members(c->my_pe, 0, 1, c->num_pes,
-                          detail::team_psync(c, t->barrier_psync_off));
+  detail::wg_sync_members(detail::pe_of(ctx), 0, 1, detail::g_state.num_pes,
+                          detail::team_psync(ctx, t->barrier_psync_off));
 }
 __device__ inline void roc_shmem_wg_sync_all() { roc_shmem_ctx_wg_sync_all(ROC_SHMEM_CTX_DEFAULT); }
 __device__ inline void roc_shmem_ctx_wg_barrier_all(roc_shmem_ctx_t ctx) {

@@ -337,10 +337,21 @@ __device__ __forceinline__ void stream_copy_uniform(char *d, const char *s, size
 // accesses of the group cover does not issue eight (six or seven of them
 // entirely out of range).
 __device__ __forceinline__ void stream_copy_sized(char *d, const char *s, size_t nbytes,
-                                                  uint32_t tid, uint32_t nthr) {
+                                                  uint32_t tid, uint32_t nthr, bool part_of_a_stream = false) {
   const size_t access_bytes = static_cast<size_t>(nthr) * 16u;
   if (nbytes >= kNonTemporalBytes) {
     stream_copy_uniform<2 /* nt */, kStreamUnroll>(d, s, nbytes, tid, nthr);
+  } else if (part_of_a_stream) {
+    // a short share of a transfer that is large as a whole: touched once, like the whole
+    if (nbytes <= access_bytes) {
+      stream_copy_uniform<2, 1>(d, s, nbytes, tid, nthr);
+    } else if (nbytes <= 2 * access_bytes) {
+      stream_copy_uniform<2, 2>(d, s, nbytes, tid, nthr);
+    } else if (nbytes <= 4 * access_bytes) {
+      stream_copy_uniform<2, 4>(d, s, nbytes, tid, nthr);
+    } else {
+      stream_copy_uniform<2, kStreamUnroll>(d, s, nbytes, tid, nthr);
+    }
   } else if (nbytes <= access_bytes) {
     stream_copy_uniform<0, 1>(d, s, nbytes, tid, nthr);
   } else if (nbytes <= 2 * access_bytes) {
@@ -371,7 +382,8 @@ __device__ __forceinline__ size_t stream_head(const char *d, size_t n) {
 // memcpy(dst, src, n) by lanes tid = 0..nthr-1 of a group that passes the
 // same (dst, src, n) in every lane.
 __device__ __forceinline__ void group_copy_uniform(void *dst, const void *src, size_t n,
-                                                   uint32_t tid, uint32_t nthr) {
+                                                   uint32_t tid, uint32_t nthr,
+                                                   bool part_of_a_stream = false) {
   char *d = static_cast<char *>(dst);
   const char *s = static_cast<const char *>(src);
   if (n < 64) {
@@ -385,7 +397,7 @@ __device__ __forceinline__ void group_copy_uniform(void *dst, const void *src, s
   n -= head;
   const size_t body = n & ~static_cast<size_t>(15);
   if ((reinterpret_cast<uintptr_t>(s) & 3u) == 0) {
-    stream_copy_sized(d, s, body, tid, nthr);
+    stream_copy_sized(d, s, body, tid, nthr, part_of_a_stream);
   } else {
     if (body >= kNonTemporalBytes) {
       stream_copy_src_unaligned<true, kStreamUnroll>(d, s, body, tid, nthr);
@@ -433,12 +445,16 @@ __device__ __forceinline__ void group_copy_dealt(void *dst, const void *src, siz
       stream_copy_src_unaligned<true, kStreamUnroll>(d + head, s + head, body, tid, nthr, part, parts);
     }
   } else {
-    size_t share = (n + parts - 1) / parts;
+    // (a division of 32-bit values when they are: a workgroup that lives for one share of a
+    // few KiB should not spend its time in a 64-bit division routine)
+    size_t share = (n >> 32) == 0 && (parts >> 32) == 0
+                       ? (static_cast<uint32_t>(n) + static_cast<uint32_t>(parts) - 1) / static_cast<uint32_t>(parts)
+                       : (n + parts - 1) / parts;
     share = (share + 255) / 256 * 256;
     size_t b = share * part, e = b + share;
     if (b > n) b = n;
     if (e > n) e = n;
-    if (e > b) group_copy_uniform(d + b, s + b, e - b, tid, nthr);
+    if (e > b) group_copy_uniform(d + b, s + b, e - b, tid, nthr, n >= kNonTemporalBytes);
   }
 }
 
