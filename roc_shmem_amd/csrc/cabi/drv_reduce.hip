@@ -267,9 +267,20 @@ size_t dtype_size(int dtype) {
   }
 }
 
-int run(int dtype, int op, const rsm::Launch &l, ReduceArgs a) {
+bool op_defined(int dtype, int op) {
+  switch (dtype) {
+    case RSM_SHORT: case RSM_INT: case RSM_LONG: case RSM_LONGLONG: return op >= RSM_SUM && op <= RSM_XOR;
+    case RSM_FLOAT: case RSM_DOUBLE: return op == RSM_SUM || op == RSM_MAX || op == RSM_MIN || op == RSM_PROD;
+    case RSM_BF16: return op == RSM_SUM || op == RSM_MAX || op == RSM_MIN;
+    default: return false;
+  }
+}
+
+// Everything that can be refused is refused here, before anything is launched.
+int check_args(int dtype, int op, const rsm::Launch &l, const ReduceArgs &a) {
   const size_t es = dtype_size(dtype);
   if (!es) return rsm::fail("to_all: unknown dtype");
+  if (!op_defined(dtype, op)) return rsm::fail("to_all: operator not defined for this dtype");
   if (a.n == 0) return 0;  // zero-element reductions are no-ops (context_tmpl_device.hpp:68-70)
   if (a.n > (~size_t{0} >> 4) || !rsm::check_extent(a.dest, a.n * es, "to_all: dest") ||
       !rsm::check_extent(a.source, a.n * es, "to_all: source") ||
@@ -279,6 +290,12 @@ int run(int dtype, int op, const rsm::Launch &l, ReduceArgs a) {
   // tile == 0: the PE's workgroups share one reduction through the sharded
   // extension; otherwise each standard call covers `tile` elements.
   if (a.tile > 0x7fffffffull) return rsm::fail("to_all: tile does not fit the API's int nreduce");
+  return 0;
+}
+
+int run(int dtype, int op, const rsm::Launch &l, ReduceArgs a, bool checked = false) {
+  if (!checked && check_args(dtype, op, l, a) != 0) return -1;
+  if (a.n == 0) return 0;
   bool ok = false;
   switch (dtype) {
     case RSM_SHORT: ok = launch_int<short>(op, l, a); break;
@@ -342,6 +359,10 @@ int rsm_to_all_noalloc(int dtype, int op, void *dest, const void *source, size_t
                      std::to_string(kNoAllocMaxWgs) + " the library's flag array has room for");
   long *flags = rsm::noalloc_flags();
   if (!flags) return -1;
+  ReduceArgs a{dest, source, nreduce, 0, pe_start, log_pe_stride, pe_size, nullptr, flags,
+               nullptr, 1 << log_pe_stride, true, false};
+  // a call that is going to be refused queues nothing, not even the clearing of the flags
+  if (check_args(dtype, op, l, a) != 0) return -1;
   if (nreduce == 0) return 0;
   // The array is shared by every call on this device and keeps what the last call left: the
   // slices this grid uses start at zero whatever happened before (a call whose waits gave up
@@ -349,9 +370,7 @@ int rsm_to_all_noalloc(int dtype, int op, void *dest, const void *source, size_t
   const size_t n_flags = static_cast<size_t>(l.grid) * ROC_SHMEM_REDUCE_SYNC_SIZE;
   hipLaunchKernelGGL(clear_flags_kernel, dim3(static_cast<unsigned>((n_flags + 255) / 256)), dim3(256),
                      0, l.stream, flags, n_flags);
-  ReduceArgs a{dest, source, nreduce, 0, pe_start, log_pe_stride, pe_size, nullptr, flags,
-               nullptr, 1 << log_pe_stride, true, false};
-  return run(dtype, op, l, a);
+  return run(dtype, op, l, a, true);
 }
 
 int rsm_tune_reduce_pacing(int dtype, int op, void *dest, const void *source, size_t nreduce,

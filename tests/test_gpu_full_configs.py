@@ -58,7 +58,7 @@ def test_config2_putmem_getmem_sweep_8_slices_1GiB_heap():
                     rs.roc_shmem_rma(kind, rs.WG, dst, src, tile, size // tile, tile, tile, 1,
                                      rs.Launch(32, 512))
                 rs.synchronize()
-                for p in (0, 3, 7):
+                for p in range(n_pes):
                     sender = (p - 1) % n_pes if kind == rs.PUT else (p + 1) % n_pes
                     got = dst.read(p, min(size + 64, biggest))
                     assert np.array_equal(got[:size], payload[sender][:size]), (size, kind, p)
@@ -92,9 +92,17 @@ def test_config3_sum_max_min_8_slices_2e26(dtype, kind):
             src.write(p, vals)
             for w, at in enumerate(starts):
                 heap.view(p, w * window * es, window, npd)[:] = vals[at:at + window]
-        launch = rs.Launch(64, 512)
         m = 3 * window
-        for op in (rs.SUM, rs.MAX, rs.MIN):
+        # sum: the benchmark's own configurations, at the library's default pacing rates - the
+        # standard call, one per workgroup over a tile of 2^21 elements, 32 workgroups of 1024
+        # lanes per PE (the headline), and the sharded extension with the same launch; max and min
+        # with 64 x 512 lanes per PE sharing one call (not paced at that grid size)
+        assert rs.get_pacing()[1] != 0
+        cases = [(rs.SUM, rs.Launch(32, 1024, 1 << 21)), (rs.SUM, rs.Launch(32, 1024)),
+                 (rs.MAX, rs.Launch(64, 512)), (rs.MIN, rs.Launch(64, 512))]
+        for op, launch in cases:
+            for p in range(n_pes):
+                dst.fill(0x5A, pe=p)
             rs.roc_shmem_to_all(dtype, op, dst, src, n, 0, 0, n_pes, None, psync, launch)
             rs.synchronize()
             first = dst.read(0)
@@ -305,7 +313,7 @@ def test_config5_broadcast_and_alltoall_16_slices_64MiB():
         rs.roc_shmem_alltoall(4, world, dst, src, block, rs.Launch(16, 512))
         rs.synchronize()
         bb = block * 4
-        for j in (0, 5, 15):
+        for j in range(n_pes):
             got = dst.read(j)
             for i in range(n_pes):
                 assert np.array_equal(got[i * bb:(i + 1) * bb], data[i][j * bb:(j + 1) * bb]), (i, j)

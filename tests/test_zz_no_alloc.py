@@ -101,3 +101,85 @@ def test_sizes_beyond_the_array_are_refused():
             assert (dst.read(p) == 16).all()
         dst.free()
         src.free()
+
+
+def _free_device_memory():
+    """Free bytes of device memory as the HIP runtime reports them (hipMemGetInfo, straight from
+    the runtime's library, which the data-path library has loaded already)."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    free, total = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
+def test_calls_allocate_nothing_and_can_be_recorded_in_a_graph():
+    # What the entry point is for: callers that cannot allocate, a stream under capture among
+    # them.  Two calls (the second smaller, another launch shape) are recorded into one graph and
+    # replayed with new inputs, with eager work and synchronisations between the replays; every
+    # replay is compared with the oracle, and neither the symmetric heap nor the device's free
+    # memory moves across the calls.
+    n_pes, n1, n2 = 8, 70001, 4099
+    with runtime(n_pes, heap_size=32 << 20):
+        stream = rs.Stream()
+        src = rs.sym_array(n1, np.int64)
+        dst1 = rs.sym_array(n1, np.int64, fill=0)
+        dst2 = rs.sym_array(n2, np.int64, fill=0)
+        big, small = rs.Launch(16, 512, 0, stream), rs.Launch(2, 256, 0, stream)
+
+        def calls():
+            rs.roc_shmem_to_all_noalloc(rs.LONG, rs.SUM, dst1, src, n1, 0, 0, n_pes, big)
+            rs.roc_shmem_to_all_noalloc(rs.LONG, rs.XOR, dst2, src, n2, 0, 0, n_pes, small)
+
+        def check(vals):
+            want1 = np.sum(np.stack(vals), axis=0, dtype=np.int64)
+            want2 = np.bitwise_xor.reduce(np.stack(vals)[:, :n2], axis=0)
+            for p in range(n_pes):
+                assert np.array_equal(dst1.read(p), want1), p
+                assert np.array_equal(dst2.read(p), want2), p
+
+        def new_inputs(seed):
+            vals = [random_values(rs.LONG, n1, seed * 100 + p) for p in range(n_pes)]
+            for p in range(n_pes):
+                src.write(p, vals[p])
+                dst1.fill(0, pe=p)
+                dst2.fill(0, pe=p)
+            return vals
+
+        vals = new_inputs(1)
+        calls()                                  # eager, also the first use on this device
+        stream.synchronize()
+        check(vals)
+        heap_before, free_before = rs.heap_bytes_in_use(), _free_device_memory()
+        for _ in range(20):
+            calls()
+        stream.synchronize()
+        assert rs.heap_bytes_in_use() == heap_before
+        assert _free_device_memory() == free_before, "a call changed the device's free memory"
+        with rs.Graph.capture(stream) as graph:
+            calls()
+        # (the HIP runtime keeps device memory for an instantiated graph, the caller's, not the
+        # entry point's: free memory is compared again from after the first replay)
+        vals = new_inputs(9)
+        graph.launch()
+        stream.synchronize()
+        check(vals)
+        free_before = _free_device_memory()
+        for seed in (2, 3, 4, 5):
+            vals = new_inputs(seed)
+            graph.launch()
+            stream.synchronize()
+            check(vals)
+            # eager work of the same kind between the replays
+            rs.roc_shmem_to_all_noalloc(rs.LONG, rs.MAX, dst2, src, n2, 0, 0, n_pes, small)
+            stream.synchronize()
+        assert rs.heap_bytes_in_use() == heap_before
+        assert _free_device_memory() == free_before
+        assert rs.take_status() == 0
+        # a refused call queues nothing: the operator is not defined for the type
+        with pytest.raises(rs.RocShmemError, match="operator not defined"):
+            rs.roc_shmem_to_all_noalloc(rs.FLOAT, rs.XOR, dst2, src, n2, 0, 0, n_pes, small)
+        graph.destroy()
+        stream.destroy()
+        for a in (dst2, dst1, src):
+            a.free()
