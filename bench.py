@@ -176,6 +176,142 @@ def timeline_summary(path):
     return out
 
 
+class ClockSampler:
+    """Clock and power readings while a loop of launches runs: the driver's files
+    (/sys/class/drm/card0/device: the GFX clock level marked current, socket power in microwatts)
+    read by a thread every 20 ms, and `amd-smi metric -c -p --json` (the GFX clock of every XCD)
+    run by a child process meanwhile."""
+
+    SYS = "/sys/class/drm/card0/device"
+
+    def __init__(self):
+        import glob
+        self.power_files = glob.glob(self.SYS + "/hwmon/*/power1_input") + glob.glob(self.SYS + "/hwmon/*/power1_average")
+        self.sclk, self.power, self.xcd_clocks, self.smi_power = [], [], [], []
+        self.stop = False
+
+    def _sys_loop(self):
+        import re
+        while not self.stop:
+            try:
+                with open(self.SYS + "/pp_dpm_sclk") as f:
+                    m = re.search(r"(\d+)Mhz \*", f.read())
+                if m:
+                    self.sclk.append(int(m.group(1)))
+                if self.power_files:
+                    with open(self.power_files[0]) as f:
+                        self.power.append(int(f.read()) / 1e6)
+            except (OSError, ValueError):
+                pass
+            time.sleep(0.02)
+
+    def _smi_loop(self):
+        import subprocess
+        while not self.stop:
+            try:
+                txt = subprocess.run(["amd-smi", "metric", "-c", "-p", "--json"], capture_output=True, text=True,
+                                     timeout=20).stdout
+                rec = json.loads(txt)
+                rec = rec[0] if isinstance(rec, list) else rec
+                rec = rec.get("gpu_data", [rec])[0] if isinstance(rec, dict) and "gpu_data" in rec else rec
+                clocks = [v["clk"]["value"] for k, v in sorted(rec.get("clock", {}).items())
+                          if k.startswith("gfx_") and isinstance(v.get("clk"), dict) and isinstance(v["clk"].get("value"), (int, float))]
+                if clocks:
+                    self.xcd_clocks.append(clocks)
+                pw = rec.get("power", {}).get("socket_power", {})
+                if isinstance(pw, dict) and isinstance(pw.get("value"), (int, float)):
+                    self.smi_power.append(pw["value"])
+            except Exception:   # the tool is optional, its output format differs between releases
+                time.sleep(0.2)
+
+    def __enter__(self):
+        import threading
+        self.threads = [threading.Thread(target=self._sys_loop, daemon=True), threading.Thread(target=self._smi_loop, daemon=True)]
+        for t in self.threads:
+            t.start()
+        return self
+
+    def __exit__(self, *exc):
+        self.stop = True
+        for t in self.threads:
+            t.join(timeout=30)
+        return False
+
+    def summary(self):
+        def stats(v):
+            return None if not v else {"mean": round(float(np.mean(v)), 1), "min": round(float(np.min(v)), 1),
+                                       "max": round(float(np.max(v)), 1), "samples": len(v)}
+        out = {"sysfs_gfx_clock_MHz": stats(self.sclk), "sysfs_socket_power_W": stats(self.power),
+               "amd_smi_socket_power_W": stats(self.smi_power)}
+        if self.xcd_clocks:
+            arr = np.array([c for c in self.xcd_clocks if len(c) == len(self.xcd_clocks[0])], dtype=float)
+            out["amd_smi_gfx_clock_MHz_by_xcd_mean"] = [round(float(x), 0) for x in arr.mean(axis=0)]
+            out["amd_smi_gfx_clock_MHz_mean"] = round(float(arr.mean()), 1)
+            out["amd_smi_samples"] = int(len(arr))
+        return out
+
+
+def bench_clock_ab(rs, oracle, variants, seconds, launches_only=0):
+    """The GFX clock (which the L2 runs at) and the socket power under loops of one kernel each.
+    Every variant moves 4 GiB per launch (the one-way probes 2 GiB).  seconds: length of each sampled loop; launches_only > 0:
+    no sampling, that many launches per variant (for a rocprofv3 --pmc run, whose TCC_CYCLE_sum /
+    128 / duration is the L2 clock the kernel saw)."""
+    out = {}
+    total_elems = 1 << 29                      # 8 x 2^26 four-byte elements
+    for name in variants:
+        kind, _, arg = name.partition(":")
+        n_pes = int(arg) if kind == "members" else 8
+        n = total_elems // n_pes
+        rs.roc_shmem_init(n_pes, 2 * n * 4 + (64 << 20), 64, 1024)
+        dtype, op = (rs.FLOAT, rs.MAX) if kind == "float_max" else (rs.INT, rs.SUM) if kind == "int_sum" else (rs.FLOAT, rs.SUM)
+        npd = rs.NP_DTYPE[dtype]
+        src = rs.sym_array(n, npd)
+        dst = rs.sym_array(n, npd, fill=0)
+        psync = rs.sym_array(max(64, 256 // n_pes) * rs.ROC_SHMEM_REDUCE_SYNC_SIZE, np.int64, fill=0)
+        rng = np.random.default_rng(3)
+        block = rng.standard_normal(min(n, 1 << 24), dtype=np.float32)
+        for p in range(n_pes):
+            vals = np.tile(np.roll(block, 977 * p), -(-n // block.size))[:n]
+            src.write(p, vals.astype(npd) if dtype == rs.FLOAT else (vals * 1000).astype(npd))
+        wgs = 256 // n_pes
+        shard = rs.Launch(wgs, 1024)
+        tiled = rs.Launch(wgs, 1024, n // wgs)
+        if kind == "free":
+            rs.set_pacing(0, 0)
+        if kind == "put":
+            fn = lambda: rs.roc_shmem_rma(rs.PUT, rs.WG_SHARED, dst, src, n * 4, 1, n * 4, n * 4, 1, shard)
+        elif kind in ("read", "write"):
+            fn = lambda: rs.stream_probe(rs.STREAM_READ if kind == "read" else rs.STREAM_WRITE, src, n * 4, None, 7, shard)
+        elif kind == "standard":
+            fn = lambda: rs.roc_shmem_to_all(dtype, op, dst, src, n, 0, 0, n_pes, None, psync, tiled)
+        else:
+            fn = lambda: rs.roc_shmem_to_all(dtype, op, dst, src, n, 0, 0, n_pes, None, psync, shard)
+        for _ in range(3):
+            fn()
+        rs.synchronize()
+        if launches_only:
+            for _ in range(launches_only):
+                fn()
+            rs.synchronize()
+            out[name] = {"launches": launches_only}
+        else:
+            ms1 = event_time_ms(rs, fn, 10) / 10
+            reps = max(10, int(seconds * 1e3 / ms1))
+            with ClockSampler() as sampler:
+                time.sleep(0.1)
+                ms = event_time_ms(rs, fn, reps) / reps
+            # (the one-way probes move half as much per launch: 2 GiB)
+            row = {"GBps": round((1.0 if kind in ("read", "write") else 2.0) * total_elems * 4 / ms / 1e6, 1),
+                   "ms_per_launch": round(ms, 4), "launches": reps}
+            row.update(sampler.summary())
+            out[name] = row
+            print(name, json.dumps(row), file=sys.stderr, flush=True)
+        if rs.take_status():
+            raise RuntimeError("device status word raised")
+        rs.roc_shmem_finalize()
+    return out
+
+
 def host_threads():
     """Threads for the CPU legs: the cores this process may run on, capped by the box's
     per-GPU share of host cores where the environment states one (OMP_NUM_THREADS)."""
@@ -1017,6 +1153,12 @@ def main():
     ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="no GPU work: read the two rocprofv3 --pmc counter files of --counter-pair runs and "
                          "write the tracked traffic summary under profiles/")
+    ap.add_argument("--clock-ab", metavar="VARIANTS", nargs="?", const="default",
+                    help="GFX (L2) clock and socket power under two-second loops of one 4 GiB kernel each, nothing "
+                         "else.  VARIANTS: comma-separated among sharded, standard, free, float_max, int_sum, "
+                         "members:2, members:4, members:16, put, read, write (default: all of them)")
+    ap.add_argument("--clock-ab-launches", type=int, default=0, metavar="N",
+                    help="with --clock-ab under rocprofv3 --pmc: N launches per variant, no sampling")
     ap.add_argument("--sharded", action="store_true",
                     help="with --counter-pair: launch the sharded extension instead of the headline's standard calls")
     ap.add_argument("--timeline", metavar="FILE",
@@ -1037,6 +1179,12 @@ def main():
     import oracle
     import roc_shmem_amd as rs
 
+    if args.clock_ab:
+        names = ["sharded", "standard", "free", "float_max", "int_sum", "members:2", "members:4", "members:16",
+                 "put", "read", "write"] if args.clock_ab == "default" else args.clock_ab.split(",")
+        print(json.dumps({"clock_and_power_by_kernel": bench_clock_ab(rs, oracle, names, 2.0, args.clock_ab_launches),
+                          "library": os.environ.get("ROC_SHMEM_LIBRARY", "librocshmem_mi355x.so")}))
+        return
     if args.reduce_lds:
         out = {}
         for staged in (1, 0):

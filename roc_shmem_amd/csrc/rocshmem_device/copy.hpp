@@ -231,7 +231,12 @@ struct Pacer {
   // Waits for the burst that is due, then books the next one `step` ticks later.
   __device__ __forceinline__ void wait(uint32_t step) {
     if (period == 0) return;
+    // (-DROCSHMEM_AB_NO_SLEEP: an A/B build for measurements that polls the clock without sleeping)
+#ifdef ROCSHMEM_AB_NO_SLEEP
+    while (static_cast<int64_t>(wall_clock64() - next) < 0) {}
+#else
     while (static_cast<int64_t>(wall_clock64() - next) < 0) __builtin_amdgcn_s_sleep(2);
+#endif
     next += step;
   }
   __device__ __forceinline__ void wait_slot() { wait(period); }

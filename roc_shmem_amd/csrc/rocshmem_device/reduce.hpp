@@ -179,7 +179,13 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
   constexpr int kNt = 2;                       // cache policy: non-temporal
   // Results are written through to memory (kWriteThrough), so that the barrier
   // that ends the collective need not write this XCD's L2 back (wg_flag_barrier).
+  // (-DROCSHMEM_AB_PLAIN_STORES: an A/B build for measurements, whose stores stay in the L2
+  // and whose closing barrier writes it back.)
+#ifdef ROCSHMEM_AB_PLAIN_STORES
+  constexpr int kStore = kNt;
+#else
   constexpr int kStore = kNt | kWriteThrough;
+#endif
 
   const int64_t stride = static_cast<int64_t>(g_state.slice_stride);
   char *src0 = const_cast<char *>(reinterpret_cast<const char *>(src)) +
@@ -539,15 +545,23 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
       // the tiles; the memory system serves that badly (8 PEs, 32 x 1024 lanes per PE, one
       // call per workgroup over a tile of 2^21 floats: 4600 GB/s, against 5800 when every
       // member walks a contiguous share of the tile).  A call therefore starts its round-robin
-      // at the turn given by the address bits above one grid's worth of passes, which differ
-      // between the tiles that would otherwise collide: the windows in flight then differ in
-      // every address bit between a pass and a grid's worth of passes, as those of one sharded
-      // call do (6215 GB/s, the sharded form on the same card 6325).
-      // (32-bit arithmetic in KiB: the offset into the arena and a pass are multiples of it.)
+      // at a turn taken from its address: 5 g / W for a tile that begins g passes into the
+      // slice, in a grid of W workgroups.  g / W alone - how many grids' worth of passes lie in
+      // front of the tile - already differs between the tiles that would collide, so that the
+      // windows in flight differ in every address bit between a pass and a grid's worth of
+      // passes, as those of one sharded call do; but with it the rate depended on the slice
+      // stride, the members' arrays lying at distances that bring some windows back onto each
+      // other, and the finer turns of 5 g / W do not show that (1 GiB per PE: 6373-6400 GB/s
+      // either way, the sharded form 6381; 576 MiB: 5970 against 6404; 1100 MiB: 6040 against
+      // 6276; five other strides within 1 % of each other).
+      // The address is taken relative to the caller's slice, so that all members of a call
+      // agree on the turn whatever the slice stride is.  (32-bit arithmetic in KiB: the offset
+      // and a pass are multiples of it.)
       if (nshards == 1 && nvec / full_pass_vecs < wgs) {
-        const uint64_t into_arena = reinterpret_cast<uintptr_t>(vec_dest) -
-                                    reinterpret_cast<uintptr_t>(g_state.heap_base0);
-        start_at = static_cast<uint32_t>(into_arena >> 10) / static_cast<uint32_t>(pass_bytes >> 10) /
+        const uint64_t into_slice = reinterpret_cast<uintptr_t>(vec_dest) -
+                                    reinterpret_cast<uintptr_t>(g_state.heap_base0) -
+                                    static_cast<uint64_t>(my_pe) * g_state.slice_stride;
+        start_at = 5u * (static_cast<uint32_t>(into_slice >> 10) / static_cast<uint32_t>(pass_bytes >> 10)) /
                    static_cast<uint32_t>(wgs);
       }
       const uint32_t rate = pass_bytes >= (128u << 10) ? g_state.pace_reduce_bytes_per_tick
@@ -599,6 +613,9 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
     reduce_elements<T, Op>(dest, source, e0, e1, as, my_pe, tid, nthr);
   }
 
+#ifdef ROCSHMEM_AB_PLAIN_STORES
+  plain_stores = true;
+#endif
   wg_flag_barrier(psync, 1, my_pe, my_idx, pe_start, pe_stride, pe_size, psync_pe_step,
                   !plain_stores);
   timeline_mark(5);
