@@ -228,12 +228,15 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
   const bool halves = pacer.period != 0 && pacer.fill_edges && mine > 1 &&
                       byte_begin + start_at * step_bytes + pass_bytes <= byte_end;
   const uint32_t half_bytes = pass_bytes / 2;
+  // (whole waves in either half: workgroups of a multiple of 128 lanes)
+  const bool closing_by_lower_half = halves && nthr % 128u == 0;
   int edge = halves ? 0 : 1;   // 0: first half of the first pass, 1: whole passes, 2: its second half
   uint32_t turn = 0;           // passes taken so far
   for (;;) {
     size_t b;
     int valid;
     uint32_t slot = pacer.period;
+    uint32_t stride_of_accesses = access_bytes;
     if (edge == 1) {
       if (turn >= mine) {
         timeline_mark(3);   // stores of the last whole pass issued
@@ -248,10 +251,21 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
         valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
       }
     }
-    if (edge != 1) {
+    if (edge == 0 || edge == 2) {
       b = byte_begin + start_at * step_bytes + (edge == 0 ? 0u : half_bytes);
       valid = static_cast<int>(half_bytes);
       slot = pacer.period / 2;
+#ifndef ROCSHMEM_AB_CLOSING_HALF_BY_ALL
+      if (edge == 2 && closing_by_lower_half) {
+        // The closing half pass goes to the lower half of the workgroup's waves alone, each
+        // lane with all U of its accesses inside the window: they are the waves that are
+        // ahead (the hardware serves the older waves of a SIMD first, pass after pass, so the
+        // upper half trails by a slot and more at the end), and with U loads in flight per
+        // member instead of U / 2 the eight members' rounds of the half pass take half as long.
+        if (tid >= nthr / 2) break;
+        stride_of_accesses = access_bytes / 2;
+      }
+#endif
     }
     Acc acc[U][E];
     pacer.wait(slot);
@@ -260,7 +274,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         typename V::Pack p;
-        p.raw = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * access_bytes, kNt);
+        p.raw = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * stride_of_accesses, kNt);
 #pragma unroll
         for (int e = 0; e < E; ++e) acc[u][e] = to_acc<T, Acc>(p.e[e]);
       }
@@ -273,7 +287,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
         __amdgpu_buffer_rsrc_t rs = uniform_rsrc(src0 + (k + c) * member_step + b, valid);
 #pragma unroll
         for (int u = 0; u < U; ++u)
-          p[c][u].raw = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * access_bytes, kNt);
+          p[c][u].raw = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * stride_of_accesses, kNt);
       }
 #pragma unroll
       for (int c = 0; c < C; ++c)
@@ -288,7 +302,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
       typename V::Pack p[U];
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        p[u].raw = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * access_bytes, kNt);
+        p[u].raw = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * stride_of_accesses, kNt);
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -304,7 +318,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
       __amdgpu_buffer_rsrc_t rd = uniform_rsrc(dst0 + m * member_step + b, valid);
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        __builtin_amdgcn_raw_buffer_store_b128(out[u].raw, rd, lane_off, u * access_bytes, kStore);
+        __builtin_amdgcn_raw_buffer_store_b128(out[u].raw, rd, lane_off, u * stride_of_accesses, kStore);
     }
     if (edge == 2) break;
     if (turn <= 1) timeline_mark(2);   // stores of the first burst issued
@@ -502,6 +516,16 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
   timeline_mark(0);
   wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, pe_stride, pe_size, psync_pe_step);
   timeline_mark(1);
+  // How many workgroups stream right now, read once for the whole workgroup: its waves must
+  // agree on whether they follow the schedule (a paced workgroup hands the closing half of its
+  // first pass to the lower half of its waves, reduce_vectors), and the count may cross the
+  // line between two waves' looks.
+  __shared__ uint32_t streaming_now;
+  if (counted) {
+    if (tid == 0)
+      streaming_now = __hip_atomic_load(streaming_workgroups(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+  }
 
   // Whether this workgroup stores anything that is not written through (the
   // element path's plain stores): decides how the closing barrier releases.
@@ -570,8 +594,7 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
         if (rate != 0 && grid_is_resident())
           pacer = make_edge_filling_pacer(rate, parts * pass_bytes * static_cast<uint64_t>(pe_size));
       } else if (counted) {
-        const uint32_t inside = uniform(__hip_atomic_load(streaming_workgroups(), __ATOMIC_RELAXED,
-                                                          __HIP_MEMORY_SCOPE_AGENT));
+        const uint32_t inside = uniform(streaming_now);
         if (rate != 0 && static_cast<uint64_t>(inside) * 4u >= wgs * 3u)
           pacer = make_edge_filling_pacer(rate, wgs * pass_bytes * static_cast<uint64_t>(pe_size));
       }
