@@ -616,18 +616,21 @@ def bench_putmem(rs, steps, n_pes, msg_bytes_list, get_sweep=False):
     return res
 
 
-def bench_nbi_windows(rs, steps, n_pes, msg_bytes_list):
+def bench_nbi_windows(rs, steps, n_pes, msg_bytes_list, max_windows=1):
     """The reference's message-rate pattern (primitive_mr_tester.cpp:32-58: 64 putmem_nbi, one
     quiet) at workgroup and at wavefront granularity: every workgroup (every wave) issues a window
     of 64 roc_shmemx_ctx_putmem_nbi_wg (_wave) calls of one size to the next PE, then the
-    workgroup's waves meet and one lane issues the quiet.  GB/s counted as 2*m bytes per message,
-    M messages/s; the launch shape is the best of a few for each size (named in the row).  A
-    kernel is one window per workgroup, so the figures include one launch per 64 calls."""
+    workgroup's waves meet and one lane issues the quiet (a wave's first lane for the wave forms);
+    a kernel is one such window per workgroup (wave), or up to max_windows of them, as many as the
+    buffers hold (the reference's kernel runs 64 x loop windows; every quiet between two windows
+    drains the workgroup's memory pipeline and writes this XCD's L2 back).  GB/s counted as 2*m
+    bytes per message, M messages/s; the launch shape is the best of a few for each size (named in
+    the row)."""
     total = 256 << 20
     src = rs.sym_array(total, np.uint8)
     dst = rs.sym_array(total, np.uint8, fill=0)
     random_payload(rs, src, n_pes, seed=2)
-    shapes = {"wg": ((256, 128), (64, 256), (64, 512), (32, 512), (32, 1024)),
+    shapes = {"wg": ((256, 128), (128, 256), (64, 256), (64, 512), (32, 512), (32, 1024)),
               "wave": ((64, 256), (32, 512), (32, 1024), (64, 512))}
     res = {}
     for gran, gname in ((rs.WG, "wg"), (rs.WAVE, "wave")):
@@ -636,9 +639,11 @@ def bench_nbi_windows(rs, steps, n_pes, msg_bytes_list):
             for m in msg_bytes_list:
                 stride, best = max(m, 256), None
                 for wgs, lanes in shapes[gname]:
-                    n_msgs = 64 * (wgs if gname == "wg" else wgs * (lanes // 64))
-                    if n_msgs * stride > total:
+                    per_window = 64 * (wgs if gname == "wg" else wgs * (lanes // 64))
+                    n_windows = min(max_windows, total // (per_window * stride))
+                    if n_windows == 0:
                         continue
+                    n_msgs = per_window * n_windows
                     launch = rs.Launch(wgs, lanes)
 
                     def step():
@@ -650,7 +655,8 @@ def bench_nbi_windows(rs, steps, n_pes, msg_bytes_list):
                     rate = 2.0 * n_pes * m * n_msgs / ms / 1e6
                     if best is None or rate > best["GBps"]:
                         best = {"GBps": round(rate, 1), "Mmsgs_per_s": round(n_pes * n_msgs / ms / 1e3, 1),
-                                "us_per_window_kernel": round(ms * 1e3, 2), "launch": "%dx%d" % (wgs, lanes)}
+                                "us_per_kernel": round(ms * 1e3, 2), "windows_per_kernel": n_windows,
+                                "launch": "%dx%d" % (wgs, lanes)}
                 if best:
                     rows["%s_%d" % (kname, m)] = best
         res[gname] = rows
@@ -1304,6 +1310,7 @@ def main():
         extra["putmem_wg_8pe"] = bench_putmem(rs, 5, n_pes, [1 << k for k in range(3, 27)], get_sweep=True)
         # windows of 64 non-blocking puts / gets and one quiet (primitive_mr_tester.cpp:32-58)
         extra["nbi_windows_8pe"] = bench_nbi_windows(rs, 5, n_pes, [1 << k for k in range(3, 19)])
+        extra["nbi_windows_8pe_up_to_8_per_kernel"] = bench_nbi_windows(rs, 5, n_pes, [8, 512, 4096, 65536], 8)
         extra["putmem_getmem_per_wave_and_thread_8pe"] = bench_granularities(rs, 5, n_pes)
         extra["collectives_4KiB_8pe_one_wg_of_256"] = bench_small_latencies(rs, n_pes)
     rs.roc_shmem_finalize()

@@ -9,6 +9,8 @@ using namespace rocshmem;
 
 namespace {
 
+constexpr unsigned kWindowCalls = 64;   // non-blocking calls between two quiets
+
 __global__ void __launch_bounds__(1024)
     rma_kernel(int kind, int granularity, char *dest0, const char *source0, size_t msg_bytes,
                size_t n_msgs, size_t dst_stride, size_t src_stride, int pe_shift) {
@@ -23,7 +25,11 @@ __global__ void __launch_bounds__(1024)
   char *dest = roc_shmemx_my_addr(dest0);
   const char *source = roc_shmemx_my_addr(source0);
 
+  // The non-blocking kinds follow the reference's message-rate kernel (primitive_mr_tester.cpp:
+  // 44-49): windows of 64 calls, a quiet after each window.
+  const bool windows = kind == RSM_PUT_NBI || kind == RSM_GET_NBI;
   if (granularity == RSM_WG) {
+    unsigned in_window = 0;
     for (size_t m = w; m < n_msgs; m += nw) {
       char *d = dest + m * dst_stride;
       const char *s = source + m * src_stride;
@@ -32,6 +38,12 @@ __global__ void __launch_bounds__(1024)
         case RSM_GET: roc_shmemx_ctx_getmem_wg(ctx, d, s, msg_bytes, target); break;
         case RSM_PUT_NBI: roc_shmemx_ctx_putmem_nbi_wg(ctx, d, s, msg_bytes, target); break;
         default: roc_shmemx_ctx_getmem_nbi_wg(ctx, d, s, msg_bytes, target); break;
+      }
+      // (every lane of the workgroup counts alike; the last window's quiet is the kernel's)
+      if (windows && ++in_window == kWindowCalls && m + nw < n_msgs) {
+        in_window = 0;
+        __syncthreads();
+        if (threadIdx.x == 0) roc_shmem_ctx_quiet(ctx);
       }
     }
   } else if (granularity == RSM_WG_SHARED) {
@@ -50,6 +62,7 @@ __global__ void __launch_bounds__(1024)
     const size_t waves_per_wg = blockDim.x / 64;
     const size_t wave = w * waves_per_wg + threadIdx.x / 64;
     const size_t n_waves = nw * waves_per_wg;
+    unsigned in_window = 0;
     for (size_t m = wave; m < n_msgs; m += n_waves) {
       char *d = dest + m * dst_stride;
       const char *s = source + m * src_stride;
@@ -59,10 +72,16 @@ __global__ void __launch_bounds__(1024)
         case RSM_PUT_NBI: roc_shmemx_ctx_putmem_nbi_wave(ctx, d, s, msg_bytes, target); break;
         default: roc_shmemx_ctx_getmem_nbi_wave(ctx, d, s, msg_bytes, target); break;
       }
+      // (a wave's own window: its first lane's quiet covers what the wave has issued)
+      if (windows && ++in_window == kWindowCalls && m + n_waves < n_msgs) {
+        in_window = 0;
+        if (threadIdx.x % 64 == 0) roc_shmem_ctx_quiet(ctx);
+      }
     }
   } else {
     const size_t thread = w * blockDim.x + threadIdx.x;
     const size_t n_threads = nw * blockDim.x;
+    unsigned in_window = 0;
     for (size_t m = thread; m < n_msgs; m += n_threads) {
       char *d = dest + m * dst_stride;
       const char *s = source + m * src_stride;
@@ -72,15 +91,19 @@ __global__ void __launch_bounds__(1024)
         case RSM_PUT_NBI: roc_shmem_ctx_putmem_nbi(ctx, d, s, msg_bytes, target); break;
         default: roc_shmem_ctx_getmem_nbi(ctx, d, s, msg_bytes, target); break;
       }
+      if (windows && ++in_window == kWindowCalls && m + n_threads < n_msgs) {
+        in_window = 0;
+        roc_shmem_ctx_quiet(ctx);
+      }
     }
   }
   // The reference's tester kernels end with a quiet.  A message that the PE's workgroups share
   // is complete when all of them have returned, which no single workgroup can know: there the
   // end of the kernel is the completion point and a quiet per workgroup would only cost (every
   // quiet writes the XCD's whole L2 back: 6.26 -> 6.43 TB/s for 64 MiB messages without it).
-  // The waves meet first, each with its own stores complete (__syncthreads), so that the one
-  // lane's quiet covers what the whole workgroup has issued - the non-blocking forms return
-  // without the waves having met.
+  // The waves meet first (__syncthreads: a workgroup-scope release and acquire around the
+  // barrier), so that the one lane's quiet, an agent-scope release after it, covers what every
+  // wave of the workgroup has issued - the non-blocking forms return without the waves having met.
   if (granularity != RSM_WG_SHARED) {
     __syncthreads();
     if (threadIdx.x == 0) roc_shmem_ctx_quiet(ctx);

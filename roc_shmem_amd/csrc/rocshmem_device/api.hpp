@@ -274,9 +274,10 @@ __device__ inline void roc_shmemx_ctx_putmem_nbi_wg(roc_shmem_ctx_t ctx, void *d
 }
 __device__ inline void roc_shmemx_ctx_putmem_wg(roc_shmem_ctx_t ctx, void *dest,
                                                 const void *source, size_t nelems, int pe) {
-  // On return the source is reusable and every wave's stores have been taken by
-  // this XCD's L2 (each wave waits for its own, then the waves meet), so one
-  // lane's roc_shmem_ctx_quiet or fence afterwards covers the whole workgroup's
+  // On return the source is reusable, and every wave's stores are ordered before
+  // whatever any lane of the workgroup issues next (a workgroup-scope release,
+  // then the waves meet), so one lane's roc_shmem_ctx_quiet or fence afterwards -
+  // an agent-scope release, which is cumulative - covers the whole workgroup's
   // put.  What is not done here is the L2 write-back that makes the bytes
   // visible to PEs on other XCDs: that is quiet's (the reference flushes in
   // the put itself, context_ib_device.cpp:148-165,219-236; with one L2 per XCD a

@@ -57,6 +57,25 @@ def test_kinds_and_granularities(kind, gran):
         run_rma(kind, gran, 4, 1000, 9, seed=kind * 3 + gran)
 
 
+@pytest.mark.parametrize("kind", [rs.PUT_NBI, rs.GET_NBI])
+@pytest.mark.parametrize("gran,msg_bytes,wgs,wg_size,n_msgs", [
+    # windows of 64 non-blocking calls and a quiet per workgroup (wave), as the reference's
+    # message-rate kernel issues them (primitive_mr_tester.cpp:44-49): three whole windows per
+    # workgroup (wave) and part of a fourth; 64 guard bytes between neighbouring messages
+    (rs.WG, 4096, 4, 256, 64 * 4 * 3 + 7),
+    (rs.WG, 65536, 4, 256, 64 * 4 * 3 + 7),
+    (rs.WG, 4096, 3, 1024, 64 * 3 * 2 + 1),
+    (rs.WAVE, 4096, 2, 256, 64 * 8 * 3 + 13),
+    (rs.WAVE, 65536, 2, 128, 64 * 4 * 2 + 5),
+    (rs.THREAD, 96, 1, 64, 64 * 64 * 2 + 9),
+])
+def test_windows_of_non_blocking_calls(kind, gran, msg_bytes, wgs, wg_size, n_msgs):
+    # (the heap hands out powers of two: room for two arrays rounded up, and the library's own)
+    with runtime(4, heap_size=4 << (n_msgs * (msg_bytes + 64) + 256).bit_length()):
+        run_rma(kind, gran, 4, msg_bytes, n_msgs, seed=msg_bytes + gran + kind, wgs=wgs, wg_size=wg_size,
+                stride_pad=64)
+
+
 @pytest.mark.parametrize("msg_bytes", [8, 16, 32, 63, 64, 65, 100, 256, 1024, 4096, 65536, 1 << 20])
 def test_message_size_sweep_wg(msg_bytes):
     # the put/get benchmark sweep at reduced heap size: 8 slices, powers of two from 8 B up
