@@ -158,10 +158,9 @@ def timeline_summary(path):
     us = (rows[:, :6].astype(np.int64) - np.int64(t0)) / 100.0      # 100 MHz clock
     xcd = (rows[:, 6] & 15).astype(int)
     wave_of_wg = np.nonzero(raw[:, 0] != 0)[0] % 16
-    names = ["entered", "entry_barrier_done", "first_burst_stored", "last_whole_pass_stored", "own_stores_landed",
+    names = ["entered", "entry_barrier_done", "first_burst_stored", "last_pass_stored", "own_stores_landed",
              "closing_barrier_done"]
-    out = {"waves": int(len(rows)), "period_ticks": int(rows[0, 6] >> 16),
-           "edge_filling_waves": int(((rows[:, 6] >> 8) & 1).sum())}
+    out = {"waves": int(len(rows)), "period_ticks": int(rows[0, 6] >> 16)}
     for label, sel in (("even_xcds", xcd % 2 == 0), ("odd_xcds", xcd % 2 == 1),
                        ("first_wave_of_each_workgroup", wave_of_wg == 0),
                        ("last_wave_of_each_workgroup", wave_of_wg == wave_of_wg.max())):

@@ -135,7 +135,7 @@ int rsm_take_status(void);                      /* sticky device status word, cl
 /* Lockstep pacing of large sharded transfers and reductions (no counterpart in the
  * reference).  Rates are bytes of memory traffic per tick of the GPU's 100 MHz constant
  * clock; 0 switches pacing off.  Defaults: reductions 67000 (6.7 TB/s) when their passes are
- * 128 KiB per member (workgroups of 1024 lanes) and 65000 with shorter passes, copies 0; also
+ * 128 KiB per member (workgroups of 1024 lanes) and 63000 with shorter passes, copies 0; also
  * settable through ROC_SHMEM_PACE_REDUCE (both kinds of pass), ROC_SHMEM_PACE_REDUCE_SHORT and
  * ROC_SHMEM_PACE_COPY.  A reduce rate set through rsm_set_pacing holds for both kinds of pass
  * (setting the default for long passes again brings both defaults back); rsm_get_pacing
@@ -144,9 +144,10 @@ int rsm_take_status(void);                      /* sticky device status word, cl
  * rsm_rma(..., RSM_WG_SHARED) transfers
  * (roc_shmemx_ctx_{put,get}mem_wg_shard) that fill the chip issue their loads and stores
  * by a common schedule of time slots derived from the rate (a wave that is early waits for
- * its slot, one that is late goes at once) instead of drifting apart; results are the
- * same, only the timing changes.  A rate somewhat above what the card sustains is best
- * (fp32 sum over 8 x 2^26: 6.02 TB/s free, 6.44 at 67000, 6.25 at 90000, 5.74 at 58000);
+ * its slot, one that is late goes at once) instead of drifting apart - in a reduction the
+ * whole chip loads in one slot and stores in the next; results are the same, only the
+ * timing changes.  The best rate is the one the card just sustains (fp32 sum over 8 x 2^26:
+ * 6.00 TB/s free, 6.57 at 67000, 6.46 at 70000, 6.25 at 90000, 5.77 at 58000);
  * rsm_tune_reduce_pacing measures it for one reduction on this card. */
 int rsm_set_pacing(unsigned copy_bytes_per_tick, unsigned reduce_bytes_per_tick);
 int rsm_get_pacing(unsigned *copy_bytes_per_tick, unsigned *reduce_bytes_per_tick);

@@ -68,16 +68,16 @@ struct Options {
   // of the 100 MHz clock for the lockstep pacing of large sharded copies / reductions (device
   // Pacer); 0 = off.  Reductions are paced by default at the rate where the schedule gained
   // most on the cards seen, one rate for passes of 128 KiB per member (workgroups of 1024
-  // lanes) and one for shorter passes (fp32 sum over 8 x 2^26, GB/s at 64000 / 65000 / 66000 /
-  // 67000 / 68000 / 70000 and running free; 32 x 1024 lanes per PE, two cards: 6272 6327 6404
-  // 6445 6375 6318 | 6017 and 6258 6338 6394 6423 6405 6356 | 6015; 32 x 512: 6262 6324 6226
-  // 6116 6023 5965 | 5845 and 6272 6302 6293 6023 5984 5970 | 5864).  A rate the caller sets
+  // lanes) and one for shorter passes (fp32 sum over 8 x 2^26, GB/s at 63000 / 64000 / 65000 /
+  // 66000 / 67000 / 68000 / 70000 and running free; 32 x 1024 lanes per PE: 6236 6321 6411 6503
+  // 6571 6546 6456 | 6001; 32 x 512, whose shorter slots leave less room: 6208 5972 6144 5869
+  // 6196 5814 5819 | 5860, steady up to 63000 and uneven beyond).  A rate the caller sets
   // (rsm_set_pacing, the tuner) holds for both kinds of pass; setting the default long rate
   // again brings both defaults back.
   // Copies run free by default: their short passes gain nothing from the schedule.
   uint32_t pace_copy = 0;
   uint32_t pace_reduce = 67000;
-  uint32_t pace_reduce_short = 65000;
+  uint32_t pace_reduce_short = 63000;
   // ROC_SHMEM_REDUCE_LDS=1: rsm_to_all runs float / long / bfloat16 sums through the LDS-staged
   // form of the sharded reduction (a measured alternative, slower on MI355X; default 0).
   bool reduce_lds = false;

@@ -201,12 +201,12 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t uniform_rsrc(const void *base,
 // while others idle: a plain copy of 8 x 256 MiB runs at 5.9-6.0 TB/s on
 // MI355X although reads alone reach 6.8-7.1 and writes alone 6.3-6.6.  Time is
 // therefore cut into slots of `period` ticks of the 100 MHz constant clock,
-// which every workgroup can read: the workgroups on even XCDs issue the loads
-// of a pass in even slots and its stores in odd slots, those on odd XCDs the
-// other way round.  All of them then start each burst at the same instant,
-// half the chip reading while the other half writes (of each pair of
-// neighbouring XCDs one reads while the other writes; pairing them any other
-// way measured worse), and the bursts sweep one compact window of every array.
+// which every workgroup can read: a workgroup issues the loads of a pass in
+// one slot and its stores in the next.  All workgroups then start each burst
+// at the same instant, and the bursts sweep one compact window of every array.
+// Which slot is whose differs by the kind of stream: see make_pacer (copies:
+// neighbouring XCDs a slot apart, half the chip reading while the other half
+// writes) and make_anchored_pacer (reductions: the whole chip in phase).
 //
 // The slots are a schedule, not a gate: a wave keeps the start time of its
 // next burst, waits for it when it is early and goes at once when it is late.
@@ -227,7 +227,6 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t uniform_rsrc(const void *base,
 struct Pacer {
   uint32_t period;   // ticks per slot; 0 = not paced
   uint64_t next;     // clock value at which the next burst of this wave is due
-  bool fill_edges;   // this workgroup starts and ends with half a pass (make_edge_filling_pacer)
   // Waits for the burst that is due, then books the next one `step` ticks later.
   __device__ __forceinline__ void wait(uint32_t step) {
     if (period == 0) return;
@@ -247,7 +246,7 @@ struct Pacer {
 // pacing.  The first burst (loads) is due at the start of the first slot of
 // this XCD's load parity that has not ended yet.
 __device__ __forceinline__ Pacer make_pacer(uint32_t bytes_per_tick, uint64_t slot_bytes) {
-  Pacer p{0u, 0u, false};
+  Pacer p{0u, 0u};
   if (bytes_per_tick == 0) return p;
   const uint64_t period = (slot_bytes + bytes_per_tick - 1) / bytes_per_tick;
   if (period < 64 || period > 50000) return p;
@@ -260,30 +259,31 @@ __device__ __forceinline__ Pacer make_pacer(uint32_t bytes_per_tick, uint64_t sl
   return p;
 }
 
-// The same slots for a stream whose workgroups can split their first pass
-// (reduce_vectors).  With make_pacer, the XCDs whose parity is out of phase at
-// the start idle until their first slot, and the others idle while those store
-// their last pass: a slot at either end in which half the chip works alone.
-// Here the slot grid is anchored at the launch instead (the clock rounded up
-// to kPaceGranuleTicks, which workgroups that start within 2 us of each other
-// agree on), every XCD starts loading in slot 0, and the workgroups on odd
-// XCDs put themselves one slot behind the others by taking half a pass first -
-// its loads in the first half of slot 0, its stores in the second half - and
-// the other half of that pass last.  Both halves of the chip are then busy from
-// the first slot to the last.  Bare 8 -> 8 fp32 reduction, 8 passes per
-// workgroup, one card, best rate: 6570-6587 GB/s with make_pacer's start (645-
-// 680 us from launch to launch, as the clock's phase at the launch falls),
-// 6404-6418 with the anchored grid and odd XCDs simply one slot behind,
-// 6630-6640 with the halves (641-653 us).
-constexpr uint32_t kPaceGranuleTicks = 200;
-__device__ __forceinline__ Pacer make_edge_filling_pacer(uint32_t bytes_per_tick, uint64_t slot_bytes) {
-  Pacer p{0u, 0u, false};
+// The slots of a reduction (reduce_vectors).  The whole chip is in phase here: every
+// workgroup issues the loads of a pass in one slot and its stores in the next, so that memory
+// serves reads alone for a slot and writes alone for the next.  The slot grid is anchored at
+// the launch (the clock rounded up to kPaceGranuleTicks, which workgroups that start within
+// 2 us of each other agree on) and a reduction of P passes per workgroup takes 2 P slots.
+// 8 -> 8 fp32 reduction of 2^26 elements, 32 workgroups of 1024 lanes per PE, one card, best
+// rate of each: 6030-6080 GB/s running free; 6404-6418 with neighbouring XCDs a slot apart
+// (one half of the chip loading while the other stores; -DROCSHMEM_AB_ALTERNATE_PHASE builds
+// that for measurements), 6423-6445 with the odd XCDs' first pass split in two halves that fill
+// the slot at either end; 6569-6576 in phase.  A mixed stream costs every request more at the
+// memory side (a read 2500-3100 L2 cycles against 1660-2250 in a stream of reads alone) than
+// the burst of one kind that the whole chip issues at once.  A reduction's pass is eight
+// rounds of loads, each waiting for the one before (the fold), and one burst of stores; a
+// copy's pass is one round of each, and copies run best free (make_pacer, off by default).
+constexpr uint32_t kPaceGranuleTicks = 200;   // (100, 400 and 800 ticks measured the same within 0.5 %)
+__device__ __forceinline__ Pacer make_anchored_pacer(uint32_t bytes_per_tick, uint64_t slot_bytes) {
+  Pacer p{0u, 0u};
   if (bytes_per_tick == 0) return p;
   const uint64_t period = (slot_bytes + bytes_per_tick - 1) / bytes_per_tick;
   if (period < 64 || period > 50000) return p;
   p.period = static_cast<uint32_t>(period);
-  p.fill_edges = (__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 1u) != 0;   // XCC_ID
   p.next = (wall_clock64() + kPaceGranuleTicks - 1) / kPaceGranuleTicks * kPaceGranuleTicks;
+#ifdef ROCSHMEM_AB_ALTERNATE_PHASE
+  if (__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 1u) p.next += period;   // XCC_ID
+#endif
   return p;
 }
 

@@ -221,60 +221,20 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
     return;
   const uint32_t mine = uniform(static_cast<uint32_t>((byte_end - byte_begin + step_bytes - 1) / step_bytes));
   if (start_at >= mine) start_at = uniform(start_at % mine);
-  // A workgroup that fills the edges of the schedule (Pacer::fill_edges; it has two passes
-  // or more, so its first one is whole) takes the first half of its first pass, then its
-  // other passes, then the second half of the first: a half pass is the same code over a
-  // window of half the size (the descriptor clips the other accesses), at half the slot.
-  const bool halves = pacer.period != 0 && pacer.fill_edges && mine > 1 &&
-                      byte_begin + start_at * step_bytes + pass_bytes <= byte_end;
-  const uint32_t half_bytes = pass_bytes / 2;
-  // (whole waves in either half: workgroups of a multiple of 128 lanes)
-  const bool closing_by_lower_half = halves && nthr % 128u == 0;
-  int edge = halves ? 0 : 1;   // 0: first half of the first pass, 1: whole passes, 2: its second half
-  uint32_t turn = 0;           // passes taken so far
-  for (;;) {
-    size_t b;
-    int valid;
-    uint32_t slot = pacer.period;
-    uint32_t stride_of_accesses = access_bytes;
-    if (edge == 1) {
-      if (turn >= mine) {
-        timeline_mark(3);   // stores of the last whole pass issued
-        if (!halves) break;
-        edge = 2;
-      } else {
-        uint32_t p = turn + start_at;
-        if (p >= mine) p -= mine;
-        ++turn;
-        b = byte_begin + p * step_bytes;
-        const size_t left = byte_end - b;
-        valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
-      }
-    }
-    if (edge == 0 || edge == 2) {
-      b = byte_begin + start_at * step_bytes + (edge == 0 ? 0u : half_bytes);
-      valid = static_cast<int>(half_bytes);
-      slot = pacer.period / 2;
-#ifndef ROCSHMEM_AB_CLOSING_HALF_BY_ALL
-      if (edge == 2 && closing_by_lower_half) {
-        // The closing half pass goes to the lower half of the workgroup's waves alone, each
-        // lane with all U of its accesses inside the window: they are the waves that are
-        // ahead (the hardware serves the older waves of a SIMD first, pass after pass, so the
-        // upper half trails by a slot and more at the end), and with U loads in flight per
-        // member instead of U / 2 the eight members' rounds of the half pass take half as long.
-        if (tid >= nthr / 2) break;
-        stride_of_accesses = access_bytes / 2;
-      }
-#endif
-    }
+  for (uint32_t turn = 0; turn < mine; ++turn) {
+    uint32_t p = turn + start_at;
+    if (p >= mine) p -= mine;
+    const size_t b = byte_begin + p * step_bytes;
+    const size_t left = byte_end - b;
+    const int valid = static_cast<int>(left < pass_bytes ? left : pass_bytes);
     Acc acc[U][E];
-    pacer.wait(slot);
+    pacer.wait_slot();
     {
       __amdgpu_buffer_rsrc_t rs = uniform_rsrc(src0 + b, valid);
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         typename V::Pack p;
-        p.raw = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * stride_of_accesses, kNt);
+        p.raw = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * access_bytes, kNt);
 #pragma unroll
         for (int e = 0; e < E; ++e) acc[u][e] = to_acc<T, Acc>(p.e[e]);
       }
@@ -287,7 +247,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
         __amdgpu_buffer_rsrc_t rs = uniform_rsrc(src0 + (k + c) * member_step + b, valid);
 #pragma unroll
         for (int u = 0; u < U; ++u)
-          p[c][u].raw = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * stride_of_accesses, kNt);
+          p[c][u].raw = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * access_bytes, kNt);
       }
 #pragma unroll
       for (int c = 0; c < C; ++c)
@@ -302,7 +262,7 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
       typename V::Pack p[U];
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        p[u].raw = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * stride_of_accesses, kNt);
+        p[u].raw = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, u * access_bytes, kNt);
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -313,24 +273,20 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
     for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int e = 0; e < E; ++e) out[u].e[e] = from_acc<T, Acc>(acc[u][e]);
-    pacer.wait(slot);
+    pacer.wait_slot();
     for (int m = 0; m < as.size; ++m) {
       __amdgpu_buffer_rsrc_t rd = uniform_rsrc(dst0 + m * member_step + b, valid);
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        __builtin_amdgcn_raw_buffer_store_b128(out[u].raw, rd, lane_off, u * stride_of_accesses, kStore);
+        __builtin_amdgcn_raw_buffer_store_b128(out[u].raw, rd, lane_off, u * access_bytes, kStore);
     }
-    if (edge == 2) break;
-    if (turn <= 1) timeline_mark(2);   // stores of the first burst issued
-    if (edge == 0) {
-      edge = 1;
-      turn = 1;
-    }
+    if (turn == 0) timeline_mark(2);            // stores of the first burst issued
+    if (turn + 1 == mine) timeline_mark(3);     // stores of the last pass issued
   }
   // every wave has its own stores in memory before it meets the others
   __builtin_amdgcn_s_waitcnt(0);
   timeline_mark(4);
-  timeline_mark(6, (__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 15u) | (pacer.fill_edges ? 256u : 0u) |
+  timeline_mark(6, (__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 15u) |
                        (static_cast<uint64_t>(pacer.period) << 16));
 }
 
@@ -476,7 +432,15 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
   // The range is dealt to pe_size * nshards workgroups: member k's workgroup
   // of shard s is part s * pe_size + k.
   const size_t parts = static_cast<size_t>(pe_size) * nshards;
+  // (-DROCSHMEM_AB_SWAP_DEAL: an A/B build for measurements in which neighbouring members swap
+  // their passes.  With 8 PEs every PE's workgroups run on one XCD, and the odd XCDs end a
+  // large reduction 10-13 us after the even ones (6-8 % later when the workgroups run free);
+  // with the passes swapped it is still the odd XCDs, so it is the XCD and not the address.)
+#ifdef ROCSHMEM_AB_SWAP_DEAL
+  const size_t part = static_cast<size_t>(shard) * pe_size + (my_idx ^ 1);
+#else
   const size_t part = static_cast<size_t>(shard) * pe_size + my_idx;
+#endif
 
   constexpr size_t E = VecOf<T>::kElems;
   // The vector path stores 16-byte aligned and loads at any 4-byte alignment,
@@ -516,10 +480,9 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
   timeline_mark(0);
   wg_flag_barrier(psync, 0, my_pe, my_idx, pe_start, pe_stride, pe_size, psync_pe_step);
   timeline_mark(1);
-  // How many workgroups stream right now, read once for the whole workgroup: its waves must
-  // agree on whether they follow the schedule (a paced workgroup hands the closing half of its
-  // first pass to the lower half of its waves, reduce_vectors), and the count may cross the
-  // line between two waves' looks.
+  // How many workgroups stream right now, read once for the whole workgroup: one look at the
+  // word instead of one per wave, and the workgroup's waves then agree on whether they follow
+  // the schedule (the count may cross the line between two waves' looks).
   __shared__ uint32_t streaming_now;
   if (counted) {
     if (tid == 0)
@@ -536,7 +499,7 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
     // Vectors [v0, v1) in passes first_pass, first_pass + pass_step, ... of this workgroup.
     size_t v0 = 0, v1 = nvec, first_pass = part, pass_step = parts;
     bool short_passes = nvec < parts * full_pass_vecs;
-    Pacer pacer{0u, 0u, false};
+    Pacer pacer{0u, 0u};
     uint32_t start_at = 0;
     if (nshards == 1 && !stream) {
       // One workgroup per member and less than two full passes each: member k takes the k-th
@@ -592,11 +555,11 @@ __device__ __forceinline__ void wg_all_reduce(int my_pe, T *dest, const T *sourc
                                                        : g_state.pace_reduce_short_bytes_per_tick;
       if (nshards > 1) {
         if (rate != 0 && grid_is_resident())
-          pacer = make_edge_filling_pacer(rate, parts * pass_bytes * static_cast<uint64_t>(pe_size));
+          pacer = make_anchored_pacer(rate, parts * pass_bytes * static_cast<uint64_t>(pe_size));
       } else if (counted) {
         const uint32_t inside = uniform(streaming_now);
         if (rate != 0 && static_cast<uint64_t>(inside) * 4u >= wgs * 3u)
-          pacer = make_edge_filling_pacer(rate, wgs * pass_bytes * static_cast<uint64_t>(pe_size));
+          pacer = make_anchored_pacer(rate, wgs * pass_bytes * static_cast<uint64_t>(pe_size));
       }
     }
     if (lds_stage != nullptr && stream && nshards > 1) {

@@ -135,8 +135,9 @@ struct DeviceState {
   uint32_t pace_copy_bytes_per_tick;
   uint32_t pace_reduce_bytes_per_tick;
   // The rate for reductions whose passes are shorter than 128 KiB per member (workgroups of
-  // fewer than 1024 lanes): they sustain a little less, and a schedule ahead of what the card
-  // sustains costs them more (32 x 512 lanes per PE: 6324 GB/s at 65000, 6023 at 68000).
+  // fewer than 1024 lanes): their slots are half as long, they sustain a little less, and a
+  // schedule ahead of what the card sustains costs them more (32 x 512 lanes per PE: 6208 GB/s
+  // at 63000, 5814-6196 from launch shape to launch shape and rate to rate beyond it).
   uint32_t pace_reduce_short_bytes_per_tick;
   // Grids that are paced: at most pace_max_grid_lanes lanes (compute units x 1024, what is
   // resident together of the streaming kernels, which need 65-128 vector registers: the slots
