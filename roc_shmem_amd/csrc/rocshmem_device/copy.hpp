@@ -265,10 +265,11 @@ __device__ __forceinline__ Pacer make_pacer(uint32_t bytes_per_tick, uint64_t sl
 // the launch (the clock rounded up to kPaceGranuleTicks, which workgroups that start within
 // 2 us of each other agree on) and a reduction of P passes per workgroup takes 2 P slots.
 // 8 -> 8 fp32 reduction of 2^26 elements, 32 workgroups of 1024 lanes per PE, one card, best
-// rate of each: 6030-6080 GB/s running free; 6404-6418 with neighbouring XCDs a slot apart
-// (one half of the chip loading while the other stores; -DROCSHMEM_AB_ALTERNATE_PHASE builds
-// that for measurements), 6423-6445 with the odd XCDs' first pass split in two halves that fill
-// the slot at either end; 6569-6576 in phase.  A mixed stream costs every request more at the
+// rate of each: 6030-6080 GB/s running free; 6160-6170 with neighbouring XCDs a slot apart
+// (one half of the chip loading while the other stores, which takes a seventeenth slot in
+// which half the chip works alone; -DROCSHMEM_AB_ALTERNATE_PHASE builds that for
+// measurements), 6423-6445 with the odd XCDs' first pass split in two halves that fill that
+// slot at either end; 6550-6576 in phase.  A mixed stream costs every request more at the
 // memory side (a read 2500-3100 L2 cycles against 1660-2250 in a stream of reads alone) than
 // the burst of one kind that the whole chip issues at once.  A reduction's pass is eight
 // rounds of loads, each waiting for the one before (the fold), and one burst of stores; a
