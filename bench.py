@@ -337,7 +337,7 @@ def device_report():
 def bench_to_all(rs, oracle, steps, warmup, dtype, n_pes, n, seed, check=True, cpu=False,
                  spread=False, launch_shape=None, tune=False, pace=None):
     """Returns a dict with ms_per_step, GB/s (algorithmic 2*P*N*s bytes) and optional CPU figures.
-    pace: None = the pacing rates the library holds (its defaults: 6.7 TB/s, 6.5 with short passes),
+    pace: None = the pacing rates the library holds (its defaults: 6.7 TB/s, 6.3 with short passes),
     0 = workgroups run free, another value = that rate in bytes per tick.
     tune: let the library measure, outside the timed region, which rate suits this reduction on
     this card, with the launch shapes of TUNE_SHAPES; the timed steps then run with the better

@@ -91,10 +91,9 @@ def test_paced_reduction_of_arrays_that_start_off_a_vector_boundary():
             a.free()
 
 
-def test_paced_reduction_in_place_with_half_passes_at_the_edges():
-    """dest == source at the default rate and the headline's launch shape: the workgroups on odd
-    XCDs reduce the first half of their first pass first and its second half last, each byte
-    range read and then overwritten by the same lanes."""
+def test_paced_reduction_in_place():
+    """dest == source at the default rate and the headline's launch shape: every byte range is
+    read in a load slot and overwritten in the next store slot by the same lanes."""
     n_pes, wgs, wg_size = 8, 32, 1024       # 256 workgroups, 128 KiB per member per pass
     with runtime(n_pes, heap_size=512 << 20, num_blocks=32):
         n = (160 << 20) // 4 + 13            # five passes per workgroup and a ragged end
