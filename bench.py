@@ -610,6 +610,20 @@ def bench_putmem(rs, steps, n_pes, msg_bytes_list, get_sweep=False):
         ms = event_time_ms(rs, one_call, steps) / steps
         one[str(m)] = {"GBps": 2.0 * n_pes * m / ms / 1e6, "us": ms * 1e3}
     res["one_workgroup_per_pe_one_call_per_message"] = one
+    # the sharded put in the launch shape of the fastest plain copy: one 256 MiB message per PE, one
+    # small workgroup per share of a few KiB ("<share bytes>x<lanes>"; one, two or four accesses per lane)
+    small = {}
+    for share, lanes in ((4096, 256), (4096, 128), (8192, 256), (2048, 64), (8192, 128)):
+        launch = rs.Launch(total // share, lanes)
+
+        def small_shares():
+            rs.roc_shmem_rma(rs.PUT, rs.WG_SHARED, dst, src, total, 1, total, total, 1, launch)
+
+        small_shares()
+        rs.synchronize()
+        ms = event_time_ms(rs, small_shares, steps) / steps
+        small["%dx%d" % (share, lanes)] = round(2.0 * n_pes * total / ms / 1e6, 1)
+    res["268435456_shared_one_small_workgroup_per_share"] = small
     src.free()
     dst.free()
     return res

@@ -301,12 +301,14 @@ __device__ inline void roc_shmemx_ctx_getmem_wg(roc_shmem_ctx_t ctx, void *dest,
   if (nelems != 0) __syncthreads();
 }
 // extension: one transfer shared by `nshards` workgroups of the calling PE.
+// (Always inlined: as a separate function the call takes its callee's register
+// count, whatever the calling kernel was compiled for.)
 // All of them pass the same dest / source / nelems / pe and their own shard
 // number; a large transfer between mutually aligned buffers is dealt to them
 // pass by pass.  Non-blocking in the sense of the _nbi forms: the source may
 // be reused and the destination read when all shards have returned and
 // roc_shmem_ctx_quiet (or the kernel's end) has passed.
-__device__ inline void roc_shmemx_ctx_putmem_wg_shard(roc_shmem_ctx_t ctx, void *dest,
+__device__ __forceinline__ void roc_shmemx_ctx_putmem_wg_shard(roc_shmem_ctx_t ctx, void *dest,
                                                       const void *source, size_t nelems, int pe,
                                                       int shard, int nshards) {
   if (nelems == 0) return;
@@ -314,7 +316,7 @@ __device__ inline void roc_shmemx_ctx_putmem_wg_shard(roc_shmem_ctx_t ctx, void 
   detail::wg_copy_shard(detail::translate(detail::own(dest, me), me, pe), detail::own(source, me), nelems,
                         shard, nshards, detail::g_state.pace_copy_bytes_per_tick);
 }
-__device__ inline void roc_shmemx_ctx_getmem_wg_shard(roc_shmem_ctx_t ctx, void *dest,
+__device__ __forceinline__ void roc_shmemx_ctx_getmem_wg_shard(roc_shmem_ctx_t ctx, void *dest,
                                                       const void *source, size_t nelems, int pe,
                                                       int shard, int nshards) {
   if (nelems == 0) return;

@@ -273,6 +273,8 @@ __device__ __forceinline__ void reduce_vectors(T *dst, const T *src, size_t v_be
     for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int e = 0; e < E; ++e) out[u].e[e] = from_acc<T, Acc>(acc[u][e]);
+    // (load and store slots of equal length: a load slot of 0.8, 0.9, 1.1 or 1.2 of the store
+    // slot's length measured 6397, 6483, 6557 and 6463 GB/s at the best rate of each against 6565)
     pacer.wait_slot();
     for (int m = 0; m < as.size; ++m) {
       __amdgpu_buffer_rsrc_t rd = uniform_rsrc(dst0 + m * member_step + b, valid);
