@@ -97,8 +97,10 @@ __global__ void __launch_bounds__(1024)
   roc_shmem_wg_ctx_create(ROC_SHMEM_CTX_WG_PRIVATE, &ctx);
   const int me = roc_shmem_ctx_my_pe(ctx);
   const int npes = roc_shmem_ctx_n_pes(ctx);
-  const size_t w = blockIdx.x / npes;
-  const size_t nw = gridDim.x / npes;
+  // (the quotients are the same in every lane, but a division is carried out on the vector unit:
+  // saying so keeps the tile loop's bookkeeping in scalar registers)
+  const size_t w = detail::uniform(static_cast<size_t>(blockIdx.x / npes));
+  const size_t nw = detail::uniform(static_cast<size_t>(gridDim.x / npes));
   const int rel = me - pe_start;
   const bool member = rel >= 0 && (rel & ((1 << log_stride) - 1)) == 0 &&
                       (rel >> log_stride) < pe_size;
