@@ -296,8 +296,13 @@ __device__ __forceinline__ uint64_t grid_workgroups() {
 // paced stream needs).
 __device__ __forceinline__ bool grid_is_resident() {
   const uint64_t wgs = grid_workgroups();
-  return wgs >= g_state.pace_min_grid_workgroups &&
-         wgs * flat_block_size() <= g_state.pace_max_grid_lanes;
+  // A compute unit holds 1024 lanes of these kernels (16 waves at 65-128 vector registers) in
+  // whole workgroups: one of 640 lanes, not one and a half (384 workgroups of 640 lanes passed
+  // a test on lanes alone, a third of them waited for a free compute unit, and the paced
+  // reduction ran at 3.1 TB/s against 4.9 running free).
+  const uint32_t per_cu = 1024u / flat_block_size();
+  const uint64_t cus = g_state.pace_max_grid_lanes / 1024u;
+  return wgs >= g_state.pace_min_grid_workgroups && wgs <= cus * per_cu;
 }
 
 // Body of a group copy whose arguments are the same in every lane
