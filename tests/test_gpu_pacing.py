@@ -42,10 +42,13 @@ def test_paced_reduction_matches_the_oracle(rate, mib):
                 a.free()
 
 
-@pytest.mark.parametrize("n_pes,wgs,wg_size,mib", [(16, 16, 1024, 80), (4, 64, 512, 40), (2, 128, 1024, 72)])
+@pytest.mark.parametrize("n_pes,wgs,wg_size,mib", [(16, 16, 1024, 80), (4, 64, 512, 40), (2, 128, 1024, 72),
+                                                   (8, 48, 640, 60), (8, 32, 768, 60)])
 def test_paced_reduction_with_other_numbers_of_pes(n_pes, wgs, wg_size, mib):
     """256 workgroups in all, two to five passes each, a ragged end, the library's default rate:
-    2, 4 and 16 members (with 2 and 4 PEs the workgroups of a PE are spread over several XCDs)."""
+    2, 4 and 16 members (with 2 and 4 PEs the workgroups of a PE are spread over several XCDs).
+    Also workgroups of 640 and 768 lanes, whose passes are no power of two: 384 of 640 lanes are
+    not all resident (one per compute unit) and run free, 256 of 768 lanes follow the schedule."""
     with runtime(n_pes, heap_size=512 << 20, num_blocks=wgs):   # two power-of-two blocks of 128 MiB
         n = (mib << 20) // 4 + 41
         src = rs.sym_array(n, np.float32)
