@@ -741,9 +741,9 @@ def bench_streams(rs, n_pes, steps=10):
 
 
 def bench_pacing_sweep(rs, n_pes):
-    """Rate of the headline reduction and of a sharded 64 MiB put, running free and paced at fixed
+    """Rate of the headline reduction and of a sharded 256 MiB put, running free and paced at fixed
     rates (no tuner), for two launch shapes: GB/s by rate in bytes per tick of the 100 MHz clock."""
-    out = {"float_sum_to_all_8x2^26": {}, "putmem_wg_shard_64MiB": {}}
+    out = {"float_sum_to_all_8x2^26": {}, "putmem_wg_shard_256MiB": {}}
     n = 1 << 26
     src = rs.sym_array(n, np.float32)
     dst = rs.sym_array(n, np.float32, fill=0)
@@ -761,10 +761,10 @@ def bench_pacing_sweep(rs, n_pes):
             rs.roc_shmem_to_all(rs.FLOAT, rs.SUM, dst, src, n, 0, 0, n_pes, None, psync, launch)
 
         def put():
-            rs.roc_shmem_rma(rs.PUT, rs.WG_SHARED, dst, src, 64 << 20, 4, 64 << 20, 64 << 20, 1, launch)
+            rs.roc_shmem_rma(rs.PUT, rs.WG_SHARED, dst, src, 256 << 20, 1, 256 << 20, 256 << 20, 1, launch)
 
         for name, fn, nbytes, which in (("float_sum_to_all_8x2^26", reduce, 2.0 * n_pes * n * 4, 1),
-                                        ("putmem_wg_shard_64MiB", put, 2.0 * n_pes * (256 << 20), 0)):
+                                        ("putmem_wg_shard_256MiB", put, 2.0 * n_pes * (256 << 20), 0)):
             row = {}
             for r in rates:
                 rs.set_pacing(r if which == 0 else 0, r if which == 1 else 0)
@@ -1058,7 +1058,7 @@ def bench_bcast_a2a(rs, n_pes, slice_bytes):
     dst = rs.sym_array(slice_bytes, np.uint8, fill=0)
     random_payload(rs, src, n_pes, seed=5)
     # best of a sweep over 8/16/32 workgroups per PE x 512/1024 threads for each
-    launch = rs.Launch(16, 1024)
+    launch = rs.Launch(16, 512)
     bcast_launch = fcollect_launch = rs.Launch(8, 1024)
     nelem = slice_bytes // 4
 

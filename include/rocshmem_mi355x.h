@@ -135,14 +135,14 @@ int rsm_take_status(void);                      /* sticky device status word, cl
 /* Lockstep pacing of large sharded transfers and reductions (no counterpart in the
  * reference).  Rates are bytes of memory traffic per tick of the GPU's 100 MHz constant
  * clock; 0 switches pacing off.  Defaults: reductions 67000 (6.7 TB/s) when their passes are
- * 128 KiB per member (workgroups of 1024 lanes) and 63000 with shorter passes, copies 0; also
+ * 128 KiB per member (workgroups of 1024 lanes) and 63000 with shorter passes, copies 67000; also
  * settable through ROC_SHMEM_PACE_REDUCE (both kinds of pass), ROC_SHMEM_PACE_REDUCE_SHORT and
  * ROC_SHMEM_PACE_COPY.  A reduce rate set through rsm_set_pacing holds for both kinds of pass
  * (setting the default for long passes again brings both defaults back); rsm_get_pacing
  * reports the rate for long passes.  With a rate set, the workgroups of large reductions -
- * sharded calls, and standard calls when the whole grid is inside calls like them - and of
- * rsm_rma(..., RSM_WG_SHARED) transfers
- * (roc_shmemx_ctx_{put,get}mem_wg_shard) that fill the chip issue their loads and stores
+ * sharded calls, and standard calls when the whole grid is inside calls like them - of
+ * rsm_rma(..., RSM_WG_SHARED) transfers (roc_shmemx_ctx_{put,get}mem_wg_shard) of 64 passes
+ * or more per workgroup and of large alltoalls that fill the chip issue their loads and stores
  * by a common schedule of time slots derived from the rate (a wave that is early waits for
  * its slot, one that is late goes at once) instead of drifting apart - in a reduction the
  * whole chip loads in one slot and stores in the next; results are the same, only the

@@ -74,8 +74,10 @@ struct Options {
   // 6196 5814 5819 | 5860, steady up to 63000 and uneven beyond).  A rate the caller sets
   // (rsm_set_pacing, the tuner) holds for both kinds of pass; setting the default long rate
   // again brings both defaults back.
-  // Copies run free by default: their short passes gain nothing from the schedule.
-  uint32_t pace_copy = 0;
+  // Copies follow the same kind of schedule when one call keeps a workgroup busy for 64 passes
+  // or more (a sharded put of 256 MiB per PE; an alltoall, whose blocks share one schedule):
+  // alltoall of 16 x 64 MiB 6208-6260 GB/s free, 6421-6448 at 67000.
+  uint32_t pace_copy = 67000;
   uint32_t pace_reduce = 67000;
   uint32_t pace_reduce_short = 63000;
   // ROC_SHMEM_REDUCE_LDS=1: rsm_to_all runs float / long / bfloat16 sums through the LDS-staged

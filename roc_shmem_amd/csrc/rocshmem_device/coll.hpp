@@ -258,12 +258,18 @@ __device__ __forceinline__ void wg_alltoall_bytes(int my_pe, void *dest, const v
   if (len >= kNonTemporalBytes && (alike & 15u) == 0 && stream_head(dst_mine + b, len) == 0) {
     // Large ranges between aligned blocks: the streaming loop itself, its stores written
     // through and waited for, so that the closing barrier skips the L2 write-back.
+    // One schedule across the blocks (Pacer), when the library holds a rate for copies, the
+    // grid fills the chip and every workgroup has passes enough for the slots' start to vanish.
+    Pacer pacer{0u, 0u};
+    const size_t pass_bytes = static_cast<size_t>(nthr) * 16u * kStreamUnroll;
+    if (g_state.pace_copy_bytes_per_tick != 0 && len * pe_size >= 16 * pass_bytes && grid_is_resident())
+      pacer = make_pacer(g_state.pace_copy_bytes_per_tick, grid_workgroups() * pass_bytes);
     for (int jj = 0; jj < pe_size; ++jj) {
       int j = my_idx + jj;      // start at the own index: concurrent members hit different slices
       if (j >= pe_size) j -= pe_size;
-      stream_copy_uniform<2 /* nt */ | kWriteThrough, kStreamUnroll>(
+      stream_copy_paced<2 /* nt */ | kWriteThrough, kStreamUnroll>(
           translate(dst_mine, my_pe, as.pe_at(j)) + b, src + static_cast<size_t>(j) * block_bytes + b,
-          len, tid, nthr);
+          len, tid, nthr, 0, 1, pacer);
     }
     __builtin_amdgcn_s_waitcnt(0);
     through = true;

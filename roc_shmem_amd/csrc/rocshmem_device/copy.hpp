@@ -313,11 +313,12 @@ __device__ __forceinline__ bool grid_is_resident() {
 // tid*16", so no lane carries a 64-bit address, and the descriptor's size
 // field turns the last partial pass into the same code (accesses beyond
 // `valid` load zeros and store nothing).
+// (`pacer` by reference: a caller that moves several ranges one after the other keeps one
+// schedule across them.)
 template <int kAux, int U, int kStoreAux = kAux>
-__device__ __forceinline__ void stream_copy_uniform(char *d, const char *s, size_t nbytes,
-                                                    uint32_t tid, uint32_t nthr,
-                                                    size_t first_pass = 0, size_t pass_step = 1,
-                                                    Pacer pacer = Pacer{0u, 0u}) {
+__device__ __forceinline__ void stream_copy_paced(char *d, const char *s, size_t nbytes,
+                                                  uint32_t tid, uint32_t nthr, size_t first_pass,
+                                                  size_t pass_step, Pacer &pacer) {
   const uint32_t lane_off = tid * 16u;
   const uint32_t access_bytes = nthr * 16u;
   const uint32_t pass_bytes = access_bytes * U;
@@ -349,6 +350,14 @@ __device__ __forceinline__ void stream_copy_uniform(char *d, const char *s, size
 // next quiet does not have to write back (8 PEs, workgroup puts of 4 / 64 / 128 KiB: 4505 /
 // 5815 / 5800 GB/s with stores that stay in the L2 until then, 4565 / 5958 / 5974 written through).
 constexpr int kShortStoreAux = kWriteThrough;
+template <int kAux, int U, int kStoreAux = kAux>
+__device__ __forceinline__ void stream_copy_uniform(char *d, const char *s, size_t nbytes,
+                                                    uint32_t tid, uint32_t nthr,
+                                                    size_t first_pass = 0, size_t pass_step = 1,
+                                                    Pacer pacer = Pacer{0u, 0u}) {
+  stream_copy_paced<kAux, U, kStoreAux>(d, s, nbytes, tid, nthr, first_pass, pass_step, pacer);
+}
+
 // Picks the pass depth by message size, so that a message that one or two
 // accesses of the group cover does not issue eight (six or seven of them
 // entirely out of range).
@@ -450,10 +459,14 @@ __device__ __forceinline__ void group_copy_dealt(void *dst, const void *src, siz
       for (size_t i = head + body + tid; i < n; i += nthr) d[i] = s[i];
     }
     if (coaligned) {
-      // Paced when the library has a measured rate and every workgroup has enough
-      // passes for the slots' start-up to disappear.
+      // Paced when the library holds a rate for copies, the grid fills the chip and every
+      // workgroup has passes enough for the start of the slots to disappear: a call's first
+      // burst waits for the next slot of its kind, up to two slots, and the schedule brings 2 %
+      // (8 PEs, 32 x 1024 lanes per PE, at 67000: one message of 256 MiB per PE, 64 passes per
+      // workgroup, 6413-6437 GB/s free and 6519-6569 paced; four of 64 MiB, 16 passes each,
+      // 6396-6431 free and 6104-6212 paced).
       Pacer pacer{0u, 0u};
-      if (pace_bytes_per_tick != 0 && body >= 16 * parts * pass_bytes && grid_is_resident())
+      if (pace_bytes_per_tick != 0 && body >= 64 * parts * pass_bytes && grid_is_resident())
         pacer = make_pacer(pace_bytes_per_tick, grid_workgroups() * pass_bytes);
       stream_copy_uniform<2 /* nt */, kStreamUnroll>(d + head, s + head, body, tid, nthr, part, parts,
                                                      pacer);

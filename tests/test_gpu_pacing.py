@@ -155,8 +155,8 @@ def test_paced_standard_calls_tiled_over_the_grid_match_the_oracle(rate, wgs, wg
 
 @pytest.mark.parametrize("rate", [40000, 66000, 90000])
 def test_paced_shared_put_and_get_are_exact(rate):
-    n_pes, nbytes = 8, (40 << 20) + 4099        # 32 x 512 per PE: 20 passes per workgroup
-    with runtime(n_pes, heap_size=256 << 20, num_blocks=32):
+    n_pes, nbytes = 8, (72 << 20) + 4099        # 32 x 256 per PE: 72 passes per workgroup
+    with runtime(n_pes, heap_size=512 << 20, num_blocks=32):
         src = rs.sym_array(nbytes + 64, np.uint8)
         dst = rs.sym_array(nbytes + 64, np.uint8, fill=0xA5)
         rng = np.random.default_rng(9)
@@ -168,7 +168,7 @@ def test_paced_shared_put_and_get_are_exact(rate):
             for p in range(n_pes):
                 dst.fill(0xA5, pe=p)
             rs.roc_shmem_rma(kind, rs.WG_SHARED, dst.addr + shift, src.addr + shift, nbytes, 1, nbytes, nbytes, 1,
-                             rs.Launch(32, 512))
+                             rs.Launch(32, 256))
             rs.synchronize()
             for p in range(n_pes):
                 sender = (p - 1) % n_pes if kind == rs.PUT else (p + 1) % n_pes
@@ -176,6 +176,38 @@ def test_paced_shared_put_and_get_are_exact(rate):
                 assert np.array_equal(got[shift:shift + nbytes], payload[sender][shift:shift + nbytes]), (kind, p)
                 assert (got[:shift] == 0xA5).all() and (got[shift + nbytes:] == 0xA5).all()
         rs.set_pacing(0, 0)
+        dst.free()
+        src.free()
+
+
+@pytest.mark.parametrize("rate,n_pes,wgs,wg_size,ragged", [(40000, 16, 16, 512, 0), (67000, 8, 32, 1024, 0),
+                                                          (90000, 16, 16, 1024, 0), (67000, 16, 16, 512, 512)])
+def test_paced_alltoall_is_exact(rate, n_pes, wgs, wg_size, ragged):
+    """An alltoall whose blocks are large enough to stream keeps one schedule across its blocks
+    (256 workgroups, 256 KiB of every block per workgroup; with the ragged size some workgroups'
+    ranges start off a 1 KiB boundary and take the unpaced path beside the others): byte for
+    byte the oracle's result whatever the rate, nothing written beside the blocks."""
+    block = (wgs * (256 << 10)) + ragged
+    nbytes = block * n_pes
+    with runtime(n_pes, heap_size=4 << (nbytes + 64).bit_length(), num_blocks=32):
+        world = rs.roc_shmem_team_world()
+        src = rs.sym_array(nbytes, np.uint8)
+        dst = rs.sym_array(nbytes + 64, np.uint8)
+        heap = oracle.Heap(n_pes, 2 * nbytes + 128)
+        rng = np.random.default_rng(rate + n_pes)
+        for p in range(n_pes):
+            payload = rng.integers(0, 256, size=nbytes, dtype=np.uint8)
+            src.write(p, payload)
+            heap.view(p, 0, nbytes, np.uint8)[:] = payload
+            dst.fill(0xA5, pe=p)
+            heap.view(p, nbytes, nbytes + 64, np.uint8)[:] = 0xA5
+        rs.set_pacing(rate, 0)
+        rs.roc_shmem_alltoall(1, world, dst, src, block, rs.Launch(wgs, wg_size))
+        rs.synchronize()
+        rs.set_pacing(0, 0)
+        oracle.alltoall(heap, nbytes, 0, block)
+        for p in range(n_pes):
+            assert np.array_equal(dst.read(p), heap.view(p, nbytes, nbytes + 64, np.uint8)), p
         dst.free()
         src.free()
 
@@ -192,9 +224,10 @@ def test_tuner_leaves_a_usable_setting_and_the_right_result():
         vals = [random_values(rs.INT, n, 70 + p) for p in range(n_pes)]
         for p in range(n_pes):
             src.write(p, vals[p])
+        copy_rate = rs.get_pacing()[0]
         res = rs.tune_reduce_pacing(rs.INT, rs.SUM, dst, src, n, 0, 0, n_pes, psync, rs.Launch(32, 512))
         assert res["free_ms"] > 0 and res["paced_ms"] > 0 and res["paced_ms"] <= res["free_ms"]
-        assert rs.get_pacing() == (0, res["rate"])
+        assert rs.get_pacing() == (copy_rate, res["rate"])     # the rate for copies is left alone
         assert res["rate"] == 0 or 50000 <= res["rate"] <= 72000
         want = np.sum(np.stack(vals).astype(np.int64), axis=0).astype(np.int32)
         for p in range(n_pes):
