@@ -552,7 +552,10 @@ def bench_putmem(rs, steps, n_pes, msg_bytes_list, get_sweep=False):
             # A few large workgroups stream best.  A blocking put returns when its loads have, so short
             # messages are bound by load latency and want as many resident workgroups as the CUs hold
             # (4 KiB: 2.6 TB/s with 64 x 256 lanes per PE, 4.6 with 256 x 128).
-            launch = rs.Launch(**PUT_LAUNCH) if tile >= (64 << 10) else \
+            # (32 KiB - 128 KiB per call: one or two accesses per lane of 1024 in flight, 3-4 % above the
+            # smaller workgroups' rate on one card)
+            launch = rs.Launch(**PUT_LAUNCH) if tile >= (256 << 10) else \
+                rs.Launch(32, 1024) if tile >= (32 << 10) else \
                 rs.Launch(64, 256) if tile > 4096 else rs.Launch(256, 128)
 
             def step():
