@@ -1333,9 +1333,10 @@ def main():
 
     if not args.quick:
         rs.roc_shmem_init(4, 64 << 20, 64, 1024)
-        # 64 MiB of traffic: launch, two flag barriers and 12 us of streaming; fewer workgroups win
+        # 64 MiB of traffic: launch, two flag barriers and 10 us of streaming (64 x 256 lanes per PE:
+        # 17.3-17.5 us on one card, 64 x 1024 17.7, 64 x 512 18.5, 32 x 512 20.0-21.8)
         extra["to_all_int64_sum_4x2^20"] = bench_to_all(rs, oracle, 50, 10, rs.LONG, 4, 1 << 20, seed=1,
-                                                        launch_shape=dict(wgs_per_pe=32, wg_size=512))
+                                                        launch_shape=dict(wgs_per_pe=64, wg_size=256))
         barrier_launch, rounds = rs.Launch(1, 256), 500
 
         def barriers():
