@@ -26,7 +26,7 @@ def test_config1_int64_sum_4_slices_2e20():
             vals = rng.integers(-(1 << 30), (1 << 30) + 1, size=n, dtype=np.int64)
             src.write(p, vals)
             heap.view(p, 0, n, np.int64)[:] = vals
-        for launch in (rs.Launch(1, 64), rs.Launch(64, 512)):
+        for launch in (rs.Launch(1, 64), rs.Launch(64, 512), rs.Launch(64, 256)):
             for p in range(n_pes):
                 dst.fill(0x5A, pe=p)
             rs.roc_shmem_to_all(rs.LONG, rs.SUM, dst, src, n, 0, 0, n_pes, None, psync, launch)
