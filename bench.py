@@ -1081,6 +1081,14 @@ def bench_bcast_a2a(rs, n_pes, slice_bytes):
     rs.synchronize()
     ms = event_time_ms(rs, a2a, 5) / 5
     res["alltoall"] = {"GBps": 2.0 * n_pes * slice_bytes / ms / 1e6, "ms": ms}
+    # the same with the copies' schedule switched on (off by default: it pays here and costs in other shapes)
+    pacing_before = rs.get_pacing()
+    rs.set_pacing(67000, pacing_before[1])
+    a2a()
+    rs.synchronize()
+    ms = event_time_ms(rs, a2a, 5) / 5
+    rs.set_pacing(*pacing_before)
+    res["alltoall_copies_paced_at_67000"] = {"GBps": 2.0 * n_pes * slice_bytes / ms / 1e6, "ms": ms}
 
     def fcollect():
         rs.roc_shmem_fcollect(4, world, dst, src, block, fcollect_launch)

@@ -135,7 +135,7 @@ int rsm_take_status(void);                      /* sticky device status word, cl
 /* Lockstep pacing of large sharded transfers and reductions (no counterpart in the
  * reference).  Rates are bytes of memory traffic per tick of the GPU's 100 MHz constant
  * clock; 0 switches pacing off.  Defaults: reductions 67000 (6.7 TB/s) when their passes are
- * 128 KiB per member (workgroups of 1024 lanes) and 63000 with shorter passes, copies 67000; also
+ * 128 KiB per member (workgroups of 1024 lanes) and 63000 with shorter passes, copies 0; also
  * settable through ROC_SHMEM_PACE_REDUCE (both kinds of pass), ROC_SHMEM_PACE_REDUCE_SHORT and
  * ROC_SHMEM_PACE_COPY.  A reduce rate set through rsm_set_pacing holds for both kinds of pass
  * (setting the default for long passes again brings both defaults back); rsm_get_pacing

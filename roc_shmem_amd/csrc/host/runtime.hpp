@@ -74,10 +74,11 @@ struct Options {
   // 6196 5814 5819 | 5860, steady up to 63000 and uneven beyond).  A rate the caller sets
   // (rsm_set_pacing, the tuner) holds for both kinds of pass; setting the default long rate
   // again brings both defaults back.
-  // Copies follow the same kind of schedule when one call keeps a workgroup busy for 64 passes
-  // or more (a sharded put of 256 MiB per PE; an alltoall, whose blocks share one schedule):
-  // alltoall of 16 x 64 MiB 6208-6260 GB/s free, 6421-6448 at 67000.
-  uint32_t pace_copy = 67000;
+  // Copies run free by default.  With a rate, sharded puts and gets that keep a workgroup busy
+  // for 64 passes or more and alltoalls whose blocks stream follow a schedule of their own; it
+  // pays in some shapes and costs in others (alltoall at 67000 against free: 16 PEs x 64 MiB
+  // +1.4 to +2.9 %, 8 PEs x 128 MiB by 32 x 1024 lanes per PE -9 %), so it is the caller's choice.
+  uint32_t pace_copy = 0;
   uint32_t pace_reduce = 67000;
   uint32_t pace_reduce_short = 63000;
   // ROC_SHMEM_REDUCE_LDS=1: rsm_to_all runs float / long / bfloat16 sums through the LDS-staged

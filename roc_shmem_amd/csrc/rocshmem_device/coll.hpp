@@ -258,8 +258,10 @@ __device__ __forceinline__ void wg_alltoall_bytes(int my_pe, void *dest, const v
   if (len >= kNonTemporalBytes && (alike & 15u) == 0 && stream_head(dst_mine + b, len) == 0) {
     // Large ranges between aligned blocks: the streaming loop itself, its stores written
     // through and waited for, so that the closing barrier skips the L2 write-back.
-    // One schedule across the blocks (Pacer), when the library holds a rate for copies, the
-    // grid fills the chip and every workgroup has passes enough for the slots' start to vanish.
+    // One schedule across the blocks (Pacer), when the caller has set a rate for copies (off by
+    // default), the grid fills the chip and every workgroup has passes enough for the slots'
+    // start to vanish.  16 PEs x 64 MiB at 67000: 6243-6289 -> 6440-6455 GB/s; other shapes lose
+    // (8 PEs x 128 MiB by 32 x 1024 lanes per PE: 6218 -> 5653), hence the caller's choice.
     Pacer pacer{0u, 0u};
     const size_t pass_bytes = static_cast<size_t>(nthr) * 16u * kStreamUnroll;
     if (g_state.pace_copy_bytes_per_tick != 0 && len * pe_size >= 16 * pass_bytes && grid_is_resident())
