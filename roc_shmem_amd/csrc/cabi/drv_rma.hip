@@ -28,20 +28,23 @@ __global__ void __launch_bounds__(1024)
   // The non-blocking kinds follow the reference's message-rate kernel (primitive_mr_tester.cpp:
   // 44-49): windows of 64 calls, a quiet after each window.
   const bool windows = kind == RSM_PUT_NBI || kind == RSM_GET_NBI;
+  // (a unit - workgroup, wave or lane - issues `span` message numbers' worth between two quiets;
+  // the last window's quiet is the kernel's)
   if (granularity == RSM_WG) {
-    unsigned in_window = 0;
-    for (size_t m = w; m < n_msgs; m += nw) {
-      char *d = dest + m * dst_stride;
-      const char *s = source + m * src_stride;
-      switch (kind) {
-        case RSM_PUT: roc_shmemx_ctx_putmem_wg(ctx, d, s, msg_bytes, target); break;
-        case RSM_GET: roc_shmemx_ctx_getmem_wg(ctx, d, s, msg_bytes, target); break;
-        case RSM_PUT_NBI: roc_shmemx_ctx_putmem_nbi_wg(ctx, d, s, msg_bytes, target); break;
-        default: roc_shmemx_ctx_getmem_nbi_wg(ctx, d, s, msg_bytes, target); break;
+    const size_t span = windows ? kWindowCalls * nw : n_msgs;
+    for (size_t m0 = w; m0 < n_msgs; m0 += span) {
+      const size_t m_end = n_msgs - m0 > span ? m0 + span : n_msgs;
+      for (size_t m = m0; m < m_end; m += nw) {
+        char *d = dest + m * dst_stride;
+        const char *s = source + m * src_stride;
+        switch (kind) {
+          case RSM_PUT: roc_shmemx_ctx_putmem_wg(ctx, d, s, msg_bytes, target); break;
+          case RSM_GET: roc_shmemx_ctx_getmem_wg(ctx, d, s, msg_bytes, target); break;
+          case RSM_PUT_NBI: roc_shmemx_ctx_putmem_nbi_wg(ctx, d, s, msg_bytes, target); break;
+          default: roc_shmemx_ctx_getmem_nbi_wg(ctx, d, s, msg_bytes, target); break;
+        }
       }
-      // (every lane of the workgroup counts alike; the last window's quiet is the kernel's)
-      if (windows && ++in_window == kWindowCalls && m + nw < n_msgs) {
-        in_window = 0;
+      if (windows && n_msgs - m0 > span) {     // every lane of the workgroup counts alike
         __syncthreads();
         if (threadIdx.x == 0) roc_shmem_ctx_quiet(ctx);
       }
@@ -62,39 +65,39 @@ __global__ void __launch_bounds__(1024)
     const size_t waves_per_wg = blockDim.x / 64;
     const size_t wave = w * waves_per_wg + threadIdx.x / 64;
     const size_t n_waves = nw * waves_per_wg;
-    unsigned in_window = 0;
-    for (size_t m = wave; m < n_msgs; m += n_waves) {
-      char *d = dest + m * dst_stride;
-      const char *s = source + m * src_stride;
-      switch (kind) {
-        case RSM_PUT: roc_shmemx_ctx_putmem_wave(ctx, d, s, msg_bytes, target); break;
-        case RSM_GET: roc_shmemx_ctx_getmem_wave(ctx, d, s, msg_bytes, target); break;
-        case RSM_PUT_NBI: roc_shmemx_ctx_putmem_nbi_wave(ctx, d, s, msg_bytes, target); break;
-        default: roc_shmemx_ctx_getmem_nbi_wave(ctx, d, s, msg_bytes, target); break;
+    const size_t span = windows ? kWindowCalls * n_waves : n_msgs;
+    for (size_t m0 = wave; m0 < n_msgs; m0 += span) {
+      const size_t m_end = n_msgs - m0 > span ? m0 + span : n_msgs;
+      for (size_t m = m0; m < m_end; m += n_waves) {
+        char *d = dest + m * dst_stride;
+        const char *s = source + m * src_stride;
+        switch (kind) {
+          case RSM_PUT: roc_shmemx_ctx_putmem_wave(ctx, d, s, msg_bytes, target); break;
+          case RSM_GET: roc_shmemx_ctx_getmem_wave(ctx, d, s, msg_bytes, target); break;
+          case RSM_PUT_NBI: roc_shmemx_ctx_putmem_nbi_wave(ctx, d, s, msg_bytes, target); break;
+          default: roc_shmemx_ctx_getmem_nbi_wave(ctx, d, s, msg_bytes, target); break;
+        }
       }
       // (a wave's own window: its first lane's quiet covers what the wave has issued)
-      if (windows && ++in_window == kWindowCalls && m + n_waves < n_msgs) {
-        in_window = 0;
-        if (threadIdx.x % 64 == 0) roc_shmem_ctx_quiet(ctx);
-      }
+      if (windows && n_msgs - m0 > span && threadIdx.x % 64 == 0) roc_shmem_ctx_quiet(ctx);
     }
   } else {
     const size_t thread = w * blockDim.x + threadIdx.x;
     const size_t n_threads = nw * blockDim.x;
-    unsigned in_window = 0;
-    for (size_t m = thread; m < n_msgs; m += n_threads) {
-      char *d = dest + m * dst_stride;
-      const char *s = source + m * src_stride;
-      switch (kind) {
-        case RSM_PUT: roc_shmem_ctx_putmem(ctx, d, s, msg_bytes, target); break;
-        case RSM_GET: roc_shmem_ctx_getmem(ctx, d, s, msg_bytes, target); break;
-        case RSM_PUT_NBI: roc_shmem_ctx_putmem_nbi(ctx, d, s, msg_bytes, target); break;
-        default: roc_shmem_ctx_getmem_nbi(ctx, d, s, msg_bytes, target); break;
+    const size_t span = windows ? kWindowCalls * n_threads : n_msgs;
+    for (size_t m0 = thread; m0 < n_msgs; m0 += span) {
+      const size_t m_end = n_msgs - m0 > span ? m0 + span : n_msgs;
+      for (size_t m = m0; m < m_end; m += n_threads) {
+        char *d = dest + m * dst_stride;
+        const char *s = source + m * src_stride;
+        switch (kind) {
+          case RSM_PUT: roc_shmem_ctx_putmem(ctx, d, s, msg_bytes, target); break;
+          case RSM_GET: roc_shmem_ctx_getmem(ctx, d, s, msg_bytes, target); break;
+          case RSM_PUT_NBI: roc_shmem_ctx_putmem_nbi(ctx, d, s, msg_bytes, target); break;
+          default: roc_shmem_ctx_getmem_nbi(ctx, d, s, msg_bytes, target); break;
+        }
       }
-      if (windows && ++in_window == kWindowCalls && m + n_threads < n_msgs) {
-        in_window = 0;
-        roc_shmem_ctx_quiet(ctx);
-      }
+      if (windows && n_msgs - m0 > span) roc_shmem_ctx_quiet(ctx);
     }
   }
   // The reference's tester kernels end with a quiet.  A message that the PE's workgroups share

@@ -345,11 +345,14 @@ __device__ __forceinline__ void stream_copy_paced(char *d, const char *s, size_t
   }
 }
 
-// Stores of a message too short for the streaming policy are written through as well: the bytes
-// have to reach memory before another XCD can see them, and what has been written through the
-// next quiet does not have to write back (8 PEs, workgroup puts of 4 / 64 / 128 KiB: 4505 /
-// 5815 / 5800 GB/s with stores that stay in the L2 until then, 4565 / 5958 / 5974 written through).
-constexpr int kShortStoreAux = kWriteThrough;
+// Stores of messages from 64 KiB on are written through even when the message is too short for
+// the streaming policy: the bytes have to reach memory before another XCD can see them, and what
+// has been written through the next quiet does not have to write back (8 PEs, workgroup puts of
+// 64 / 128 KiB: 5815 / 5800 GB/s with stores that stay in the L2 until then, 5958 / 5974 written
+// through).  Shorter messages keep plain stores: written through, a put of 4 KiB gained 1 % in a
+// stream of them, but a call on its own ended later (broadcast, alltoall and fcollect of 4-32 KiB
+// among 8 PEs: 5.8-6.2 -> 6.0-6.6 us).
+constexpr size_t kWriteThroughFromBytes = 64 * 1024;
 template <int kAux, int U, int kStoreAux = kAux>
 __device__ __forceinline__ void stream_copy_uniform(char *d, const char *s, size_t nbytes,
                                                     uint32_t tid, uint32_t nthr,
@@ -378,13 +381,19 @@ __device__ __forceinline__ void stream_copy_sized(char *d, const char *s, size_t
       stream_copy_uniform<2, kStreamUnroll>(d, s, nbytes, tid, nthr);
     }
   } else if (nbytes <= access_bytes) {
-    stream_copy_uniform<0, 1, kShortStoreAux>(d, s, nbytes, tid, nthr);
+    stream_copy_uniform<0, 1>(d, s, nbytes, tid, nthr);
   } else if (nbytes <= 2 * access_bytes) {
-    stream_copy_uniform<0, 2, kShortStoreAux>(d, s, nbytes, tid, nthr);
+    stream_copy_uniform<0, 2>(d, s, nbytes, tid, nthr);
   } else if (nbytes <= 4 * access_bytes) {
-    stream_copy_uniform<0, 4, kShortStoreAux>(d, s, nbytes, tid, nthr);
+    if (nbytes >= kWriteThroughFromBytes) {
+      stream_copy_uniform<0, 4, kWriteThrough>(d, s, nbytes, tid, nthr);
+    } else {
+      stream_copy_uniform<0, 4>(d, s, nbytes, tid, nthr);
+    }
+  } else if (nbytes >= kWriteThroughFromBytes) {
+    stream_copy_uniform<0, kStreamUnroll, kWriteThrough>(d, s, nbytes, tid, nthr);
   } else {
-    stream_copy_uniform<0, kStreamUnroll, kShortStoreAux>(d, s, nbytes, tid, nthr);
+    stream_copy_uniform<0, kStreamUnroll>(d, s, nbytes, tid, nthr);
   }
 }
 
