@@ -267,7 +267,10 @@ int rsm_to_all_team(int dtype, int op, uint64_t team, void *dest, const void *so
  * moves messages m = 0..n_msgs-1 of `msg_bytes` each between its own
  * `source + m*src_stride` / `dest + m*dst_stride` and PE (p+pe_shift)%n_pes,
  * the messages being dealt round-robin to its workgroups, waves or threads
- * according to `granularity`. */
+ * according to `granularity`.  Every workgroup ends with a quiet; with the non-blocking
+ * kinds a workgroup (wave, thread) also issues one after every 64 of its calls, the window
+ * of the reference's message-rate kernel (clients/functional_tests/primitive_mr_tester.cpp:
+ * 44-49). */
 int rsm_rma(int kind, int granularity, void *dest, const void *source, size_t msg_bytes,
             size_t n_msgs, size_t dst_stride, size_t src_stride, int pe_shift,
             const rsm_launch_t *launch);
