@@ -686,8 +686,8 @@ def bench_nbi_windows(rs, steps, n_pes, msg_bytes_list, max_windows=1):
 def bench_streams(rs, n_pes, steps=10):
     """What this card's memory system gives plain streams (rsm_stream_probe): reads alone, writes
     alone and a copy, for two shapes of launch.  `staying`: workgroups that stay and take pass after
-    pass of 128 KiB, the shape a device-side collective has (32 or 64 workgroups of 1024 lanes per
-    PE).  `one_per_pass`: as many small workgroups as passes, handed out by the hardware in address
+    pass, the shape a device-side collective has (32 or 64 workgroups of 1024 or 512 lanes per PE,
+    two to eight accesses per lane and pass; the best of them for each kind).  `one_per_pass`: as many small workgroups as passes, handed out by the hardware in address
     order, which only a kernel launched for the purpose can have.  The harmonic mean of a shape's
     two one-way rates, 2 / (1/read + 1/write), is what a stream that reads and writes as much would
     reach if mixing the directions cost nothing; the copy rows show what it costs.  Also the HIP
@@ -706,7 +706,9 @@ def bench_streams(rs, n_pes, steps=10):
 
     def shapes(staying, span):
         if staying:
-            return [(wgs, 1024, 0) for wgs in (32, 64)]
+            # (workgroups, lanes, bytes per pass): two, four or eight accesses per lane in flight
+            return [(wgs, lanes, lanes * 16 * u) for wgs, lanes in ((32, 1024), (64, 1024), (64, 512))
+                    for u in (2, 4, 8)]
         # one workgroup per pass: (lanes, accesses per lane)
         return [(span // (lanes * 16 * u), lanes, lanes * 16 * u) for lanes, u in ((256, 1), (1024, 1), (256, 4))]
 
